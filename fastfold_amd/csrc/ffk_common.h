@@ -1,0 +1,132 @@
+// Shared device/host helpers for the ffk kernel library (gfx950 / CDNA4 only).
+//
+// Everything here is header-only: dtype traits, 16-byte vector access, wave-level
+// reductions (64-wide wavefronts), MFMA fragment wrappers and the error plumbing
+// behind the C ABI declared in include/ffk.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/ffk.h"
+
+// ---------------------------------------------------------------- errors ----
+extern thread_local char ffk_err_buf[512];
+int ffk_fail(int code, const char* fmt, ...);
+
+#define FFK_REQUIRE(cond, code, ...)                  \
+    do {                                              \
+        if (!(cond)) return ffk_fail((code), __VA_ARGS__); \
+    } while (0)
+
+static inline bool ffk_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Checks the launch that was just issued on this thread.
+static inline int ffk_check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return FFK_OK;
+}
+
+// ---------------------------------------------------------------- dtypes ----
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> struct DT;
+template <> struct DT<float> {
+    static constexpr int VEC = 4;      // elements per 16-byte vector
+    static __device__ __forceinline__ float to_f(float v) { return v; }
+    static __device__ __forceinline__ float from_f(float v) { return v; }
+};
+template <> struct DT<bf16_t> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ float to_f(bf16_t v) { return (float)v; }
+    static __device__ __forceinline__ bf16_t from_f(float v) { return (bf16_t)v; }
+};
+template <> struct DT<f16_t> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ float to_f(f16_t v) { return (float)v; }
+    static __device__ __forceinline__ f16_t from_f(float v) { return (f16_t)v; }
+};
+
+// 16 bytes of T, loaded/stored as one dwordx4 access.
+template <typename T> struct alignas(16) Vec16 {
+    T e[DT<T>::VEC];
+};
+
+template <typename T> __device__ __forceinline__ Vec16<T> ld16(const T* p) {
+    return *reinterpret_cast<const Vec16<T>*>(p);
+}
+template <typename T> __device__ __forceinline__ void st16(T* p, const Vec16<T>& v) {
+    *reinterpret_cast<Vec16<T>*>(p) = v;
+}
+
+// ------------------------------------------------------- wave reductions ----
+// Reduce over groups of `width` adjacent lanes (width a power of two <= 64).
+__device__ __forceinline__ float group_sum(float v, int width) {
+    for (int off = width >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float group_max(float v, int width) {
+    for (int off = width >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ------------------------------------------------------------ fast math ----
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float sigmoid_f(float x) {
+    // 1 / (1 + 2^(-x*log2e))
+    return fast_rcp(1.0f + fast_exp2(-1.4426950408889634f * x));
+}
+template <typename T> __device__ __forceinline__ float exp_for(float x);
+template <> __device__ __forceinline__ float exp_for<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ float exp_for<bf16_t>(float x) { return fast_exp2(1.4426950408889634f * x); }
+template <> __device__ __forceinline__ float exp_for<f16_t>(float x) { return fast_exp2(1.4426950408889634f * x); }
+
+// ----------------------------------------------------------------- MFMA ----
+// A "fragment" is the 16 bytes one lane contributes to a 32x32 MFMA operand:
+// lane l supplies row (l & 31) of the operand and K-group (l >> 5).  For bf16 the
+// 16 bytes are 8 consecutive K elements and one v_mfma_f32_32x32x16_bf16 consumes
+// the pair (K step 16).  For fp32 they are 4 consecutive K elements and four
+// v_mfma_f32_32x32x2_f32 consume them (element t of both operands in step t), which
+// covers K step 8.  Both operands must be fetched with the same K <-> slot mapping;
+// the sum over K is then independent of that mapping.
+//
+// Accumulator layout (both dtypes): lane l holds column (l & 31) of the 32x32 tile;
+// register v (0..15) holds row  8*(v/4) + 4*(l>>5) + (v%4).
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+    static constexpr int KSTEP = 16;   // K elements consumed per fragment pair
+    static constexpr int KLANE = 8;    // K elements per lane per fragment
+    typedef bf16x8 Frag;
+    static __device__ __forceinline__ void mma(f32x16& acc, const Frag& a, const Frag& b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+    }
+    static __device__ __forceinline__ Frag ld(const bf16_t* p) { return *reinterpret_cast<const Frag*>(p); }
+};
+template <> struct Mma<float> {
+    static constexpr int KSTEP = 8;
+    static constexpr int KLANE = 4;
+    typedef f32x4 Frag;
+    static __device__ __forceinline__ void mma(f32x16& acc, const Frag& a, const Frag& b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
+    }
+    static __device__ __forceinline__ Frag ld(const float* p) { return *reinterpret_cast<const Frag*>(p); }
+};
+
+// Row of the 32x32 accumulator tile held in register v by lane `lane`.
+__device__ __forceinline__ int acc_row(int v, int lane) { return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3); }
+
+static inline int ffk_cdiv(long a, long b) { return (int)((a + b - 1) / b); }

@@ -1,0 +1,579 @@
+// Row-wise HBM-bound kernels: fused mask+bias softmax, LayerNorm (forward and backward)
+// and the three elementwise fusions.  Rows are short (128..4096 elements), so a row is
+// owned by a group of `lpr` adjacent lanes of one 64-wide wavefront (several rows per
+// wave), every lane moves 16 bytes per access and consecutive lanes touch consecutive
+// 16-byte vectors: each wave-level access covers whole 128-byte lines.  Reductions are
+// xor-shuffles inside the lane group; all arithmetic is fp32.
+#include "ffk_common.h"
+
+thread_local char ffk_err_buf[512] = "";
+
+int ffk_fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ffk_err_buf, sizeof(ffk_err_buf), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+extern "C" int ffk_version(void) { return 100; }
+extern "C" const char* ffk_last_error_string(void) { return ffk_err_buf; }
+
+namespace {
+
+constexpr int WAVES_PER_BLOCK = 4;
+constexpr int BLOCK = 64 * WAVES_PER_BLOCK;
+constexpr float MASK_FILL = -1e9f;
+
+// Lane-group geometry for a row of `nvec` 16-byte vectors: lanes per row (power of two,
+// 4..64) and vectors per lane (1, 2, 4 or 8).  Returns false if the row does not fit.
+struct RowGeom {
+    int lpr, vpl;
+};
+static bool row_geom(long nvec, RowGeom* g) {
+    int lpr = 8;   // >= 8 lanes x 16 B: every wave-level access covers whole 128-byte lines
+    while (lpr < 64 && (long)lpr * 2 < nvec) lpr <<= 1;
+    long vpl = (nvec + lpr - 1) / lpr;
+    int v = 1;
+    while (v < vpl) v <<= 1;
+    if (v > 8) return false;
+    g->lpr = lpr;
+    g->vpl = v;
+    return true;
+}
+
+static int row_grid(long rows, int lpr) {
+    long rows_per_block = (long)WAVES_PER_BLOCK * (64 / lpr);
+    long blocks = (rows + rows_per_block - 1) / rows_per_block;
+    const long cap = 256L * 16;   // 256 CUs, up to 16 resident blocks each; grid-stride beyond
+    return (int)(blocks < cap ? blocks : cap);
+}
+
+// ------------------------------------------------------------------ softmax ----
+template <typename T, int VPL>
+__global__ __launch_bounds__(BLOCK) void softmax_vec_kernel(T* out, const T* x,   // out may alias x
+                                                           const T* __restrict__ mask,
+                                                           const T* __restrict__ bias, long rows, int cols,
+                                                           int lpr, long hq) {
+    constexpr int VEC = DT<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rpw = 64 / lpr;
+    const int sub = lane / lpr;
+    const int j = lane % lpr;
+    const int nvec = cols / VEC;
+    const long stride = (long)gridDim.x * WAVES_PER_BLOCK * rpw;
+    for (long base = ((long)blockIdx.x * WAVES_PER_BLOCK + wave) * rpw; base < rows; base += stride) {
+        const long row = base + sub;
+        const bool valid = row < rows;
+        const T* xr = x + row * cols;
+        const T* mr = mask ? mask + (row / hq) * cols : nullptr;
+        const T* br = bias ? bias + (row % hq) * cols : nullptr;
+        float v[VPL][VEC];
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = j + i * lpr;
+            if (valid && vi < nvec) {
+                Vec16<T> xv = ld16(xr + vi * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) v[i][e] = DT<T>::to_f(xv.e[e]);
+                if (br) {
+                    Vec16<T> bv = ld16(br + vi * VEC);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) v[i][e] += DT<T>::to_f(bv.e[e]);
+                }
+                if (mr) {
+                    Vec16<T> mv = ld16(mr + vi * VEC);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        if (DT<T>::to_f(mv.e[e]) == 0.0f) v[i][e] = MASK_FILL;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) v[i][e] = -INFINITY;
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) mx = fmaxf(mx, v[i][e]);
+        mx = group_max(mx, lpr);
+        if (!valid) mx = 0.0f;
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                v[i][e] = exp_for<T>(v[i][e] - mx);
+                sum += v[i][e];
+            }
+        sum = group_sum(sum, lpr);
+        const float inv = 1.0f / sum;
+        T* orow = out + row * cols;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = j + i * lpr;
+            if (valid && vi < nvec) {
+                Vec16<T> ov;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) ov.e[e] = DT<T>::from_f(v[i][e] * inv);
+                st16(orow + vi * VEC, ov);
+            }
+        }
+    }
+}
+
+// Any row length / alignment: one wave per row, three passes over the row.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void softmax_generic_kernel(T* out, const T* x, const T* mask,
+                                                               const T* bias, long rows, int cols, long hq) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const long stride = (long)gridDim.x * WAVES_PER_BLOCK;
+    for (long row = (long)blockIdx.x * WAVES_PER_BLOCK + wave; row < rows; row += stride) {
+        const T* xr = x + row * cols;
+        const T* mr = mask ? mask + (row / hq) * cols : nullptr;
+        const T* br = bias ? bias + (row % hq) * cols : nullptr;
+        auto logit = [&](int c) -> float {
+            float v = DT<T>::to_f(xr[c]);
+            if (br) v += DT<T>::to_f(br[c]);
+            if (mr && DT<T>::to_f(mr[c]) == 0.0f) v = MASK_FILL;
+            return v;
+        };
+        float mx = -INFINITY;
+        for (int c = lane; c < cols; c += 64) mx = fmaxf(mx, logit(c));
+        mx = group_max(mx, 64);
+        float sum = 0.0f;
+        for (int c = lane; c < cols; c += 64) sum += exp_for<T>(logit(c) - mx);
+        sum = group_sum(sum, 64);
+        const float inv = 1.0f / sum;
+        T* orow = out + row * cols;
+        // out may alias x: every element is read (above and here) by the lane that writes it
+        for (int c = lane; c < cols; c += 64) orow[c] = DT<T>::from_f(exp_for<T>(logit(c) - mx) * inv);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void softmax_bwd_kernel(T* dx, const T* dy, const T* y, long rows, int cols) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const long stride = (long)gridDim.x * WAVES_PER_BLOCK;
+    for (long row = (long)blockIdx.x * WAVES_PER_BLOCK + wave; row < rows; row += stride) {
+        const T* yr = y + row * cols;
+        const T* gr = dy + row * cols;
+        float dot = 0.0f;
+        for (int c = lane; c < cols; c += 64) dot += DT<T>::to_f(yr[c]) * DT<T>::to_f(gr[c]);
+        dot = group_sum(dot, 64);
+        T* o = dx + row * cols;
+        for (int c = lane; c < cols; c += 64)
+            o[c] = DT<T>::from_f((DT<T>::to_f(gr[c]) - dot) * DT<T>::to_f(yr[c]));
+    }
+}
+
+template <typename T>
+int softmax_launch(T* out, const T* x, const T* mask, const T* bias, long rows, long cols, long hq,
+                   hipStream_t st) {
+    constexpr int VEC = DT<T>::VEC;
+    RowGeom g;
+    const bool vec_ok = cols % VEC == 0 && ffk_aligned16(out) && ffk_aligned16(x) &&
+                        (!mask || ffk_aligned16(mask)) && (!bias || ffk_aligned16(bias)) &&
+                        row_geom(cols / VEC, &g);
+    if (vec_ok) {
+        dim3 grid(row_grid(rows, g.lpr));
+        switch (g.vpl) {
+            case 1: softmax_vec_kernel<T, 1><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
+            case 2: softmax_vec_kernel<T, 2><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
+            case 4: softmax_vec_kernel<T, 4><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
+            default: softmax_vec_kernel<T, 8><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
+        }
+    } else {
+        dim3 grid(row_grid(rows, 64));
+        softmax_generic_kernel<T><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, hq);
+    }
+    return ffk_check_launch("ffk_softmax_fwd");
+}
+
+// ---------------------------------------------------------------- LayerNorm ----
+template <typename T, int VPL>
+__global__ __launch_bounds__(BLOCK) void layernorm_vec_kernel(T* __restrict__ out, float* __restrict__ mean_o,
+                                                             float* __restrict__ rstd_o, const T* __restrict__ x,
+                                                             const T* __restrict__ gamma,
+                                                             const T* __restrict__ beta, long rows, int cols,
+                                                             int lpr, float eps) {
+    constexpr int VEC = DT<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rpw = 64 / lpr;
+    const int sub = lane / lpr;
+    const int j = lane % lpr;
+    const int nvec = cols / VEC;
+    const float inv_n = 1.0f / (float)cols;
+    // gamma / beta stay in registers for the whole grid-stride loop
+    float gm[VPL][VEC], bt[VPL][VEC];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+        const int vi = j + i * lpr;
+        if (vi < nvec) {
+            Vec16<T> gv = ld16(gamma + vi * VEC), bv = ld16(beta + vi * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                gm[i][e] = DT<T>::to_f(gv.e[e]);
+                bt[i][e] = DT<T>::to_f(bv.e[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) gm[i][e] = bt[i][e] = 0.0f;
+        }
+    }
+    const long stride = (long)gridDim.x * WAVES_PER_BLOCK * rpw;
+    for (long base = ((long)blockIdx.x * WAVES_PER_BLOCK + wave) * rpw; base < rows; base += stride) {
+        const long row = base + sub;
+        const bool valid = row < rows;
+        const T* xr = x + row * cols;
+        float v[VPL][VEC];
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = j + i * lpr;
+            if (valid && vi < nvec) {
+                Vec16<T> xv = ld16(xr + vi * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    v[i][e] = DT<T>::to_f(xv.e[e]);
+                    s += v[i][e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) v[i][e] = 0.0f;
+            }
+        }
+        const float mu = group_sum(s, lpr) * inv_n;
+        float q = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = j + i * lpr;
+            if (vi < nvec) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float d = v[i][e] - mu;
+                    q += d * d;
+                }
+            }
+        }
+        const float var = group_sum(q, lpr) * inv_n;
+        const float rs = rsqrtf(var + eps);
+        T* orow = out + row * cols;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int vi = j + i * lpr;
+            if (valid && vi < nvec) {
+                Vec16<T> ov;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) ov.e[e] = DT<T>::from_f((v[i][e] - mu) * rs * gm[i][e] + bt[i][e]);
+                st16(orow + vi * VEC, ov);
+            }
+        }
+        if (valid && j == 0) {
+            if (mean_o) mean_o[row] = mu;
+            if (rstd_o) rstd_o[row] = rs;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void layernorm_generic_kernel(T* out, float* mean_o, float* rstd_o, const T* x,
+                                                                 const T* gamma, const T* beta, long rows,
+                                                                 int cols, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const float inv_n = 1.0f / (float)cols;
+    const long stride = (long)gridDim.x * WAVES_PER_BLOCK;
+    for (long row = (long)blockIdx.x * WAVES_PER_BLOCK + wave; row < rows; row += stride) {
+        const T* xr = x + row * cols;
+        float s = 0.0f;
+        for (int c = lane; c < cols; c += 64) s += DT<T>::to_f(xr[c]);
+        const float mu = group_sum(s, 64) * inv_n;
+        float q = 0.0f;
+        for (int c = lane; c < cols; c += 64) {
+            const float d = DT<T>::to_f(xr[c]) - mu;
+            q += d * d;
+        }
+        const float rs = rsqrtf(group_sum(q, 64) * inv_n + eps);
+        T* orow = out + row * cols;
+        for (int c = lane; c < cols; c += 64)
+            orow[c] = DT<T>::from_f((DT<T>::to_f(xr[c]) - mu) * rs * DT<T>::to_f(gamma[c]) + DT<T>::to_f(beta[c]));
+        if (lane == 0) {
+            if (mean_o) mean_o[row] = mu;
+            if (rstd_o) rstd_o[row] = rs;
+        }
+    }
+}
+
+// dx = rstd * (g - mean(g) - xhat * mean(g * xhat)),  g = dy * gamma ; dgamma += dy * xhat ; dbeta += dy
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void layernorm_bwd_kernel(T* dx, float* dgamma, float* dbeta, const T* dy,
+                                                             const T* x, const float* mean, const float* rstd,
+                                                             const T* gamma, long rows, int cols,
+                                                             long rows_per_wave) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const float inv_n = 1.0f / (float)cols;
+    const long w = (long)blockIdx.x * WAVES_PER_BLOCK + wave;
+    const long r0 = w * rows_per_wave;
+    const long r1 = r0 + rows_per_wave < rows ? r0 + rows_per_wave : rows;
+    // column-partial sums of this wave, kept per lane for columns lane, lane+64, ...
+    for (int c0 = 0; c0 < cols; c0 += 64 * 8) {
+        float pg[8], pb[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) pg[t] = pb[t] = 0.0f;
+        for (long row = r0; row < r1; ++row) {
+            const float mu = mean[row], rs = rstd[row];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int c = c0 + lane + 64 * t;
+                if (c < cols) {
+                    const float g = DT<T>::to_f(dy[row * cols + c]);
+                    pg[t] += g * (DT<T>::to_f(x[row * cols + c]) - mu) * rs;
+                    pb[t] += g;
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int c = c0 + lane + 64 * t;
+            if (c < cols && r0 < r1) {
+                atomicAdd(dgamma + c, pg[t]);
+                atomicAdd(dbeta + c, pb[t]);
+            }
+        }
+    }
+    for (long row = r0; row < r1; ++row) {
+        const float mu = mean[row], rs = rstd[row];
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int c = lane; c < cols; c += 64) {
+            const float g = DT<T>::to_f(dy[row * cols + c]) * DT<T>::to_f(gamma[c]);
+            const float xh = (DT<T>::to_f(x[row * cols + c]) - mu) * rs;
+            s1 += g;
+            s2 += g * xh;
+        }
+        s1 = group_sum(s1, 64) * inv_n;
+        s2 = group_sum(s2, 64) * inv_n;
+        for (int c = lane; c < cols; c += 64) {
+            const float g = DT<T>::to_f(dy[row * cols + c]) * DT<T>::to_f(gamma[c]);
+            const float xh = (DT<T>::to_f(x[row * cols + c]) - mu) * rs;
+            dx[row * cols + c] = DT<T>::from_f(rs * (g - s1 - xh * s2));
+        }
+    }
+}
+
+template <typename T>
+int layernorm_launch(T* out, float* mean, float* rstd, const T* x, const T* gamma, const T* beta, long rows,
+                     long cols, float eps, hipStream_t st) {
+    constexpr int VEC = DT<T>::VEC;
+    RowGeom g;
+    const bool vec_ok = cols % VEC == 0 && ffk_aligned16(out) && ffk_aligned16(x) && ffk_aligned16(gamma) &&
+                        ffk_aligned16(beta) && row_geom(cols / VEC, &g);
+    if (vec_ok) {
+        dim3 grid(row_grid(rows, g.lpr));
+        switch (g.vpl) {
+            case 1: layernorm_vec_kernel<T, 1><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
+            case 2: layernorm_vec_kernel<T, 2><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
+            case 4: layernorm_vec_kernel<T, 4><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
+            default: layernorm_vec_kernel<T, 8><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
+        }
+    } else {
+        dim3 grid(row_grid(rows, 64));
+        layernorm_generic_kernel<T><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, eps);
+    }
+    return ffk_check_launch("ffk_layernorm_fwd");
+}
+
+// -------------------------------------------------------------- elementwise ----
+// kind 0: sigmoid(a + bias) * b          (a = y, b = z)
+// kind 1: c + (a + bias) * dm            (a = x, c = residual)
+// kind 2: c + dm * (b * (a + bias))      (a = ab, b = g, c = z_raw)
+template <typename T, int KIND>
+__global__ __launch_bounds__(BLOCK) void eltwise_kernel(T* __restrict__ out, const T* __restrict__ a,
+                                                       const T* __restrict__ bias, const T* __restrict__ b,
+                                                       const T* __restrict__ c, const T* __restrict__ dm,
+                                                       long n_rows, int C, long I, long J, long dm_sb, long dm_si,
+                                                       long dm_sj, bool vec) {
+    constexpr int VEC = DT<T>::VEC;
+    const int per_row = vec ? C / VEC : C;
+    const long total = n_rows * per_row;
+    for (long idx = (long)blockIdx.x * BLOCK + threadIdx.x; idx < total; idx += (long)gridDim.x * BLOCK) {
+        const long row = idx / per_row;
+        const int col = (int)(idx - row * per_row) * (vec ? VEC : 1);
+        const long off = row * C + col;
+        const T* dmp = nullptr;
+        if (dm) {
+            const long jj = row % J, ii = (row / J) % I, bb = row / (J * I);
+            dmp = dm + bb * dm_sb + ii * dm_si + jj * dm_sj + col;
+        }
+        auto f = [&](float av, float bias_v, float bv, float cv, float dv) -> float {
+            if (KIND == 0) return sigmoid_f(av + bias_v) * bv;
+            if (KIND == 1) return cv + (av + bias_v) * dv;
+            return cv + dv * (bv * (av + bias_v));
+        };
+        if (vec) {
+            Vec16<T> av = ld16(a + off), biasv = ld16(bias + col), bv, cv, dv, ov;
+            if (KIND != 1) bv = ld16(b + off);
+            if (KIND != 0) cv = ld16(c + off);
+            if (dmp) dv = ld16(dmp);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                ov.e[e] = DT<T>::from_f(f(DT<T>::to_f(av.e[e]), DT<T>::to_f(biasv.e[e]),
+                                          KIND != 1 ? DT<T>::to_f(bv.e[e]) : 0.0f,
+                                          KIND != 0 ? DT<T>::to_f(cv.e[e]) : 0.0f,
+                                          dmp ? DT<T>::to_f(dv.e[e]) : 1.0f));
+            st16(out + off, ov);
+        } else {
+            out[off] = DT<T>::from_f(f(DT<T>::to_f(a[off]), DT<T>::to_f(bias[col]),
+                                       KIND != 1 ? DT<T>::to_f(b[off]) : 0.0f,
+                                       KIND != 0 ? DT<T>::to_f(c[off]) : 0.0f,
+                                       dmp ? DT<T>::to_f(dmp[0]) : 1.0f));
+        }
+    }
+}
+
+template <typename T, int KIND>
+int eltwise_launch(void* out, const void* a, const void* bias, const void* b, const void* c, const void* dm,
+                   long B, long I, long J, long C, long dm_sb, long dm_si, long dm_sj, hipStream_t st,
+                   const char* name) {
+    constexpr int VEC = DT<T>::VEC;
+    const long n_rows = B * I * J;
+    bool vec = C % VEC == 0 && ffk_aligned16(out) && ffk_aligned16(a) && ffk_aligned16(bias) &&
+               (!b || ffk_aligned16(b)) && (!c || ffk_aligned16(c));
+    if (dm) vec = vec && ffk_aligned16(dm) && dm_sb % VEC == 0 && dm_si % VEC == 0 && dm_sj % VEC == 0;
+    const long total = n_rows * (vec ? C / VEC : C);
+    long blocks = (total + BLOCK - 1) / BLOCK;
+    if (blocks > 256L * 32) blocks = 256L * 32;
+    eltwise_kernel<T, KIND><<<dim3((int)blocks), BLOCK, 0, st>>>((T*)out, (const T*)a, (const T*)bias, (const T*)b,
+                                                              (const T*)c, (const T*)dm, n_rows, (int)C, I, J,
+                                                              dm_sb, dm_si, dm_sj, vec);
+    return ffk_check_launch(name);
+}
+
+template <int KIND>
+int eltwise_dispatch(int dtype, void* out, const void* a, const void* bias, const void* b, const void* c,
+                     const void* dm, long B, long I, long J, long C, long dm_sb, long dm_si, long dm_sj,
+                     void* stream, const char* name) {
+    FFK_REQUIRE(out && a && bias, FFK_ERR_NULL, "%s: null pointer", name);
+    FFK_REQUIRE(KIND == 1 || b, FFK_ERR_NULL, "%s: null pointer", name);
+    FFK_REQUIRE(KIND == 0 || c, FFK_ERR_NULL, "%s: null pointer", name);
+    FFK_REQUIRE(B > 0 && I > 0 && J > 0 && C > 0 && C < (1L << 30), FFK_ERR_SHAPE, "%s: bad shape [%ld,%ld,%ld,%ld]",
+                name, B, I, J, C);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FFK_F32: return eltwise_launch<float, KIND>(out, a, bias, b, c, dm, B, I, J, C, dm_sb, dm_si, dm_sj, st, name);
+        case FFK_BF16: return eltwise_launch<bf16_t, KIND>(out, a, bias, b, c, dm, B, I, J, C, dm_sb, dm_si, dm_sj, st, name);
+        case FFK_F16: return eltwise_launch<f16_t, KIND>(out, a, bias, b, c, dm, B, I, J, C, dm_sb, dm_si, dm_sj, st, name);
+        default: return ffk_fail(FFK_ERR_DTYPE, "%s: unsupported dtype tag %d", name, dtype);
+    }
+}
+
+}  // namespace
+
+// -------------------------------------------------------------------- C ABI ----
+extern "C" int ffk_softmax_fwd(void* out, const void* x, const void* mask, const void* bias, int64_t B1,
+                               int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int dtype, void* stream) {
+    FFK_REQUIRE(out && x, FFK_ERR_NULL, "ffk_softmax_fwd: null pointer");
+    FFK_REQUIRE(B1 > 0 && B2 > 0 && H > 0 && Nq > 0 && Nk > 0 && Nk < (1L << 30), FFK_ERR_SHAPE,
+                "ffk_softmax_fwd: bad shape [%ld,%ld,%ld,%ld,%ld]", (long)B1, (long)B2, (long)H, (long)Nq, (long)Nk);
+    const long rows = B1 * B2 * H * Nq;
+    // mask row = row / (H*Nq) indexes [B1*B2]; bias row = row % (H*Nq) only when B1 == 1, else
+    // bias is [B1,1,H,Nq,Nk] and the B1 index must be kept: fold it by treating each b1 separately.
+    hipStream_t st = (hipStream_t)stream;
+    const long hq = H * Nq;
+    const size_t esz = dtype == FFK_F32 ? 4 : 2;
+    for (int64_t b1 = 0; b1 < B1; ++b1) {
+        const long r = B2 * hq;
+        const size_t xoff = (size_t)b1 * r * Nk * esz;
+        void* o = (char*)out + xoff;
+        const void* xi = (const char*)x + xoff;
+        const void* mi = mask ? (const char*)mask + (size_t)b1 * B2 * Nk * esz : nullptr;
+        const void* bi = bias ? (const char*)bias + (size_t)b1 * hq * Nk * esz : nullptr;
+        int rc;
+        switch (dtype) {
+            case FFK_F32: rc = softmax_launch<float>((float*)o, (const float*)xi, (const float*)mi, (const float*)bi, r, Nk, hq, st); break;
+            case FFK_BF16: rc = softmax_launch<bf16_t>((bf16_t*)o, (const bf16_t*)xi, (const bf16_t*)mi, (const bf16_t*)bi, r, Nk, hq, st); break;
+            case FFK_F16: rc = softmax_launch<f16_t>((f16_t*)o, (const f16_t*)xi, (const f16_t*)mi, (const f16_t*)bi, r, Nk, hq, st); break;
+            default: return ffk_fail(FFK_ERR_DTYPE, "ffk_softmax_fwd: unsupported dtype tag %d", dtype);
+        }
+        if (rc) return rc;
+    }
+    (void)rows;
+    return FFK_OK;
+}
+
+extern "C" int ffk_softmax_bwd(void* dx, const void* dy, const void* y, int64_t rows, int64_t cols, int dtype,
+                               void* stream) {
+    FFK_REQUIRE(dx && dy && y, FFK_ERR_NULL, "ffk_softmax_bwd: null pointer");
+    FFK_REQUIRE(rows > 0 && cols > 0 && cols < (1L << 30), FFK_ERR_SHAPE, "ffk_softmax_bwd: bad shape [%ld,%ld]",
+                (long)rows, (long)cols);
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(row_grid(rows, 64));
+    switch (dtype) {
+        case FFK_F32: softmax_bwd_kernel<float><<<grid, BLOCK, 0, st>>>((float*)dx, (const float*)dy, (const float*)y, rows, (int)cols); break;
+        case FFK_BF16: softmax_bwd_kernel<bf16_t><<<grid, BLOCK, 0, st>>>((bf16_t*)dx, (const bf16_t*)dy, (const bf16_t*)y, rows, (int)cols); break;
+        case FFK_F16: softmax_bwd_kernel<f16_t><<<grid, BLOCK, 0, st>>>((f16_t*)dx, (const f16_t*)dy, (const f16_t*)y, rows, (int)cols); break;
+        default: return ffk_fail(FFK_ERR_DTYPE, "ffk_softmax_bwd: unsupported dtype tag %d", dtype);
+    }
+    return ffk_check_launch("ffk_softmax_bwd");
+}
+
+extern "C" int ffk_layernorm_fwd(void* out, float* mean, float* rstd, const void* x, const void* gamma,
+                                 const void* beta, int64_t rows, int64_t cols, float eps, int dtype, void* stream) {
+    FFK_REQUIRE(out && x && gamma && beta, FFK_ERR_NULL, "ffk_layernorm_fwd: null pointer");
+    FFK_REQUIRE(rows > 0 && cols > 0 && cols < (1L << 30), FFK_ERR_SHAPE, "ffk_layernorm_fwd: bad shape [%ld,%ld]",
+                (long)rows, (long)cols);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FFK_F32: return layernorm_launch<float>((float*)out, mean, rstd, (const float*)x, (const float*)gamma, (const float*)beta, rows, cols, eps, st);
+        case FFK_BF16: return layernorm_launch<bf16_t>((bf16_t*)out, mean, rstd, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta, rows, cols, eps, st);
+        case FFK_F16: return layernorm_launch<f16_t>((f16_t*)out, mean, rstd, (const f16_t*)x, (const f16_t*)gamma, (const f16_t*)beta, rows, cols, eps, st);
+        default: return ffk_fail(FFK_ERR_DTYPE, "ffk_layernorm_fwd: unsupported dtype tag %d", dtype);
+    }
+}
+
+extern "C" int ffk_layernorm_bwd(void* dx, float* dgamma, float* dbeta, const void* dy, const void* x,
+                                 const float* mean, const float* rstd, const void* gamma, int64_t rows,
+                                 int64_t cols, int dtype, void* stream) {
+    FFK_REQUIRE(dx && dgamma && dbeta && dy && x && mean && rstd && gamma, FFK_ERR_NULL,
+                "ffk_layernorm_bwd: null pointer");
+    FFK_REQUIRE(rows > 0 && cols > 0 && cols < (1L << 30), FFK_ERR_SHAPE, "ffk_layernorm_bwd: bad shape [%ld,%ld]",
+                (long)rows, (long)cols);
+    hipStream_t st = (hipStream_t)stream;
+    const long waves = 256L * 8 * WAVES_PER_BLOCK;
+    const long rpw = (rows + waves - 1) / waves;
+    const long nw = (rows + rpw - 1) / rpw;
+    dim3 grid((int)((nw + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK));
+    switch (dtype) {
+        case FFK_F32: layernorm_bwd_kernel<float><<<grid, BLOCK, 0, st>>>((float*)dx, dgamma, dbeta, (const float*)dy, (const float*)x, mean, rstd, (const float*)gamma, rows, (int)cols, rpw); break;
+        case FFK_BF16: layernorm_bwd_kernel<bf16_t><<<grid, BLOCK, 0, st>>>((bf16_t*)dx, dgamma, dbeta, (const bf16_t*)dy, (const bf16_t*)x, mean, rstd, (const bf16_t*)gamma, rows, (int)cols, rpw); break;
+        case FFK_F16: layernorm_bwd_kernel<f16_t><<<grid, BLOCK, 0, st>>>((f16_t*)dx, dgamma, dbeta, (const f16_t*)dy, (const f16_t*)x, mean, rstd, (const f16_t*)gamma, rows, (int)cols, rpw); break;
+        default: return ffk_fail(FFK_ERR_DTYPE, "ffk_layernorm_bwd: unsupported dtype tag %d", dtype);
+    }
+    return ffk_check_launch("ffk_layernorm_bwd");
+}
+
+extern "C" int ffk_bias_sigmoid_mul(void* out, const void* y, const void* bias, const void* z, int64_t rows,
+                                    int64_t C, int dtype, void* stream) {
+    return eltwise_dispatch<0>(dtype, out, y, bias, z, nullptr, nullptr, 1, 1, rows, C, 0, 0, 0, stream,
+                               "ffk_bias_sigmoid_mul");
+}
+
+extern "C" int ffk_bias_dropout_add(void* out, const void* x, const void* bias, const void* dm,
+                                    const void* residual, int64_t B, int64_t I, int64_t J, int64_t C,
+                                    int64_t dm_sb, int64_t dm_si, int64_t dm_sj, int dtype, void* stream) {
+    return eltwise_dispatch<1>(dtype, out, x, bias, nullptr, residual, dm, B, I, J, C, dm_sb, dm_si, dm_sj, stream,
+                               "ffk_bias_dropout_add");
+}
+
+extern "C" int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const void* g, const void* dm,
+                                        const void* z_raw, int64_t B, int64_t I, int64_t J, int64_t C,
+                                        int64_t dm_sb, int64_t dm_si, int64_t dm_sj, int dtype, void* stream) {
+    return eltwise_dispatch<2>(dtype, out, ab, bias, g, z_raw, dm, B, I, J, C, dm_sb, dm_si, dm_sj, stream,
+                               "ffk_bias_ele_dropout_res");
+}

@@ -1,0 +1,60 @@
+"""Writes tests/golden/evoformer_nn_golden.npz by running the REFERENCE's own
+``fastfold.model.nn.evoformer.EvoformerStack`` (plain PyTorch, CPU, fp32) on seeded synthetic
+weights and inputs.  Run only in the build container, where /root/reference is mounted:
+
+    python tests/golden/make_golden.py
+
+The fixture pins what closed forms cannot: the composition of a block (order of the
+sub-updates, residual placement, OPM reading the updated MSA), the q/k/v and left/right
+concatenation order used when weights are re-packed, and mask handling with padded residues.
+Only inputs' seeds and the reference's outputs are stored; no reference source travels.
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, "/root/reference")
+
+from fastfold_amd.synthetic import synth_nn_state, synth_inputs  # noqa: E402
+
+CASES = [
+    # name, seed, no_blocks, n_seq, n_res, mask_tail_frac, fan_in_scaled
+    ("b1_s8_r12_pad", 11, 1, 8, 12, 0.17, True),
+    ("b2_s6_r10_full", 12, 2, 6, 10, 0.0, True),
+    ("b1_s5_r9_std002", 13, 1, 5, 9, 0.0, False),
+]
+
+
+def main():
+    from fastfold.model.nn.evoformer import EvoformerStack  # the reference
+
+    out = {}
+    for name, seed, nb, s, r, tail, fis in CASES:
+        torch.manual_seed(0)
+        stack = EvoformerStack(c_m=256, c_z=128, c_hidden_msa_att=32, c_hidden_opm=32, c_hidden_mul=128,
+                               c_hidden_pair_att=32, c_s=384, no_heads_msa=8, no_heads_pair=4, no_blocks=nb,
+                               transition_n=4, msa_dropout=0.15, pair_dropout=0.25, blocks_per_ckpt=1,
+                               inf=1e9, eps=1e-8).eval()
+        sd = synth_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=fis)
+        missing, unexpected = stack.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        assert not missing and not unexpected
+        m, z, msa_mask, pair_mask = synth_inputs(seed, s, r, mask_tail_frac=tail)
+        with torch.no_grad():
+            mo, zo, so = stack(torch.from_numpy(m), torch.from_numpy(z), torch.from_numpy(msa_mask),
+                               torch.from_numpy(pair_mask), chunk_size=None, _mask_trans=False)
+        out[name + ".m"] = mo.numpy()
+        out[name + ".z"] = zo.numpy()
+        out[name + ".s"] = so.numpy()
+        out[name + ".cfg"] = np.array([seed, nb, s, r, int(round(tail * 100)), int(fis)], dtype=np.int64)
+        print(name, "m", float(np.abs(mo.numpy() - m).mean()), "z", float(np.abs(zo.numpy() - z).mean()))
+    np.savez_compressed(os.path.join(HERE, "evoformer_nn_golden.npz"), **out)
+    print("wrote", os.path.join(HERE, "evoformer_nn_golden.npz"))
+
+
+if __name__ == "__main__":
+    main()
