@@ -96,3 +96,77 @@ def call(name: str, *args):
     if rc != 0:
         msg = lib.ffk_last_error_string()
         raise RuntimeError("%s failed (status %d): %s" % (name, rc, msg.decode() if msg else "?"))
+
+
+# ------------------------------------------------------------------ fused linear ----
+FFK_TILE_STRIDED, FFK_TILE_QK, FFK_TILE_V, FFK_TILE_BIAS = 0, 1, 2, 3
+FFK_ACT_NONE, FFK_ACT_RELU, FFK_ACT_SIGMOID = 0, 1, 2
+FFK_MAX_TILES = 10
+LOG2E = 1.4426950408889634
+
+
+class Tile(ctypes.Structure):
+    """Mirror of ``ffk_tile`` (include/ffk.h)."""
+    _fields_ = [
+        ("out", c_void_p), ("bias", c_void_p), ("resid", c_void_p), ("gate", c_void_p), ("rowmask", c_void_p),
+        ("s_o", c_int64), ("s_i", c_int64), ("s_h", c_int64), ("s_d", c_int64),
+        ("gate_ld", c_int64), ("m_so", c_int64), ("m_si", c_int64),
+        ("inner", c_int), ("kind", c_int), ("act", c_int), ("ncols", c_int), ("glu", c_int),
+        ("scale", c_float),
+    ]
+
+
+class LinearDesc(ctypes.Structure):
+    """Mirror of ``ffk_linear_desc`` (include/ffk.h)."""
+    _fields_ = [
+        ("a", c_void_p), ("a_so", c_int64), ("a_si", c_int64), ("a_cs", c_int64),
+        ("a_inner", c_int), ("a_chanmajor", c_int),
+        ("ln_gamma", c_void_p), ("ln_beta", c_void_p), ("ln_eps", c_float), ("dtype", c_int),
+        ("w", c_void_p),
+        ("M", c_int), ("K", c_int), ("n_tiles", c_int), ("reserved", c_int),
+        ("tiles", Tile * FFK_MAX_TILES),
+    ]
+
+
+SIGNATURES["ffk_fused_linear"] = [ctypes.POINTER(LinearDesc), _P]
+
+
+def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, gate_ld=0, rowmask=None,
+              m_so=0, m_si=0, s_o=0, s_i=0, s_h=32, s_d=1, inner=1, act=FFK_ACT_NONE, ncols=128, glu=0,
+              scale=1.0):
+    """Builds one epilogue descriptor; tensors may be passed directly (their data_ptr is taken)."""
+    def p(t):
+        return None if t is None else (t if isinstance(t, int) else t.data_ptr())
+    t = Tile()
+    t.out, t.bias, t.resid, t.gate, t.rowmask = p(out), p(bias), p(resid), p(gate), p(rowmask)
+    t.s_o, t.s_i, t.s_h, t.s_d = s_o, s_i, s_h, s_d
+    t.gate_ld, t.m_so, t.m_si = gate_ld, m_so, m_si
+    t.inner, t.kind, t.act, t.ncols, t.glu, t.scale = inner, kind, act, ncols, glu, scale
+    return t
+
+
+def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanmajor=False, a_cs=0,
+                 ln=None, eps=1e-5):
+    """Launches ``ffk_fused_linear``.  ``a`` / ``w`` are tensors (``w`` packed [n_tiles*128, K]);
+    ``ln`` is ``(gamma, beta)`` or None."""
+    d = LinearDesc()
+    d.a = a.data_ptr()
+    d.a_inner = M if a_inner is None else a_inner
+    d.a_so = a_so
+    d.a_si = K if a_si is None else a_si
+    d.a_cs = a_cs
+    d.a_chanmajor = 1 if a_chanmajor else 0
+    if ln is not None:
+        d.ln_gamma, d.ln_beta = ln[0].data_ptr(), ln[1].data_ptr()
+    d.ln_eps = eps
+    d.dtype = dtype_tag(a.dtype)
+    d.w = w.data_ptr()
+    d.M, d.K, d.n_tiles = M, K, len(tiles)
+    if len(tiles) > FFK_MAX_TILES:
+        raise RuntimeError("fused_linear: at most %d N-tiles per launch" % FFK_MAX_TILES)
+    if w.shape[0] != 128 * len(tiles) or w.shape[1] != K or w.dtype != a.dtype:
+        raise RuntimeError("fused_linear: packed weight must be [%d, %d] %s, got %s %s"
+                           % (128 * len(tiles), K, a.dtype, tuple(w.shape), w.dtype))
+    for i, t in enumerate(tiles):
+        d.tiles[i] = t
+    call("ffk_fused_linear", ctypes.byref(d), stream_ptr())

@@ -130,3 +130,19 @@ template <> struct Mma<float> {
 __device__ __forceinline__ int acc_row(int v, int lane) { return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3); }
 
 static inline int ffk_cdiv(long a, long b) { return (int)((a + b - 1) / b); }
+
+// ------------------------------------------------- attention operand tiles ----
+// q / k, v and the additive bias are exchanged between the projection kernel and the
+// attention kernel in 32x32-element tiles (1024 elements each) whose internal order is
+// exactly what one wavefront loads as an MFMA operand / accumulator, so that every
+// lane reads 16 contiguous elements and a wave reads the tile as one contiguous block.
+//
+//  q/k tile (rows n, head dim d):  lane (n%32, kg=d/16) owns d = 16*kg .. 16*kg+15
+__host__ __device__ __forceinline__ int qk_tile_off(int n32, int d) { return (d >> 4) * 512 + n32 * 16 + (d & 15); }
+//  accumulator-order tile: element (row, col) of a 32x32 tile whose column is the lane's
+//  (l & 31) and whose rows are spread over (l >> 5, register) as in the MFMA accumulator:
+//  lane = ((row & 7) >> 2) * 32 + col,  register = 4 * (row >> 3) + (row & 3).
+//  Used for v (row = key, col = head-dim index) and for the bias (row = key, col = query).
+__host__ __device__ __forceinline__ int acc_tile_off(int row, int col) {
+    return ((((row & 7) >> 2) * 32 + col) << 4) + 4 * (row >> 3) + (row & 3);
+}

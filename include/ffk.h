@@ -101,6 +101,72 @@ int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const 
                              int64_t C, int64_t dm_sb, int64_t dm_si, int64_t dm_sj, int dtype,
                              void* stream);
 
+
+/* ------------------------------------------------------------------------------------
+ * Fused linear:  out = epilogue( prologue(A)[M,K] . W[N,K]^T )      (bf16 / fp32 MFMA)
+ *
+ * A tile of rows of A (all K columns, K in {32..256}, K % 32 == 0) is loaded into LDS once,
+ * optionally LayerNorm-ed there (gamma/beta over K), and then multiplied against every
+ * 128-row tile of W; each such N-tile has its own epilogue descriptor, so one pass over
+ * A feeds several consumers (q, k, v, gate, bias projections of one attention, or the
+ * gated left/right projections of a triangle multiplication).
+ *
+ * Row addressing.  Logical row m of A lives at  a + (m / a_inner) * a_so + (m % a_inner) * a_si
+ * (elements; K is contiguous), which expresses plain row-major ([M,K]: a_inner = M) as well as
+ * the transposed traversals of [I,J,C] tensors used by column-wise modules.  With
+ * a_chanmajor != 0 element (m, k) lives at  a + k * a_cs + rowoffset(m)  instead (channel-major
+ * producer, e.g. the triangle contraction output).  Output tiles use the same scheme with
+ * (s_o, s_i) for rows and  (c / 32) * s_h + (c % 32) * s_d  for channel c of the tile.
+ *
+ * Tile kinds:
+ *   FFK_TILE_STRIDED  generic 4-stride store; optional  out = resid + gate * v
+ *   FFK_TILE_QK       q / k of attention in MFMA-operand tiles: [b2][h][n/32][d/16][n%32][d%16]
+ *   FFK_TILE_V        v of attention in PV-operand tiles (see ffk_attention_fwd)
+ *   FFK_TILE_BIAS     pair / triangle bias in score-accumulator tiles (see ffk_attention_fwd)
+ * Per-tile value: v = act(acc + bias[c]) * scale; with glu != 0 the tile's packed channels are
+ * [p 0..31 | g 0..31 | p 32..63 | g 32..63] and v = (p + bias_p) * sigmoid(g + bias_g) (64
+ * outputs); rowmask (0/1 per logical row, own strides) multiplies v.
+ *
+ * Replaces the F.linear + LayerNorm + elementwise chains of fastfold/model/fastnn/ops.py:
+ * 79-82,143-155,305-324,393-399,404-412,659-670 and msa.py:61-72.
+ */
+enum { FFK_TILE_STRIDED = 0, FFK_TILE_QK = 1, FFK_TILE_V = 2, FFK_TILE_BIAS = 3 };
+enum { FFK_ACT_NONE = 0, FFK_ACT_RELU = 1, FFK_ACT_SIGMOID = 2 };
+#define FFK_MAX_TILES 10
+
+typedef struct ffk_tile {
+    void* out;
+    const void* bias;      /* 128 values of the activation dtype (packed tile order) or NULL */
+    const void* resid;     /* same addressing as out (may alias out) or NULL; STRIDED with s_d == 1 only */
+    const void* gate;      /* [M, gate_ld] in logical row order, or NULL; STRIDED with s_d == 1 only */
+    const void* rowmask;   /* 0/1 per logical row at (m / inner) * m_so + (m % inner) * m_si, or NULL */
+    int64_t s_o, s_i, s_h, s_d;
+    int64_t gate_ld;
+    int64_t m_so, m_si;
+    int32_t inner;
+    int32_t kind;
+    int32_t act;
+    int32_t ncols;         /* valid output channels of this tile (<= 128, <= 64 with glu) */
+    int32_t glu;
+    float scale;
+} ffk_tile;
+
+typedef struct ffk_linear_desc {
+    const void* a;
+    int64_t a_so, a_si, a_cs;
+    int32_t a_inner;
+    int32_t a_chanmajor;
+    const void* ln_gamma;  /* NULL = no LayerNorm prologue */
+    const void* ln_beta;
+    float ln_eps;
+    int32_t dtype;
+    const void* w;         /* [n_tiles * 128, K] row-major, zero-padded rows */
+    int32_t M, K, n_tiles, reserved;
+    ffk_tile tiles[FFK_MAX_TILES];
+} ffk_linear_desc;
+
+int ffk_fused_linear(const ffk_linear_desc* desc, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

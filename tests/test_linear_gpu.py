@@ -1,0 +1,224 @@
+"""GPU parity of ffk_fused_linear (through the C ABI) against float64 numpy linear algebra
+(oracle.ops_np): every prologue / epilogue / layout the Evoformer modules use."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops_np
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}   # relative to max |ref|
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def _pack(w, n_tiles):
+    out = torch.zeros(n_tiles * 128, w.shape[1], dtype=w.dtype, device=w.device)
+    out[: w.shape[0]] = w
+    return out
+
+
+def _rel(got, ref):
+    return np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6)
+
+
+def _sig(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,K,N", [(300, 128, 256), (129, 256, 200), (64, 64, 36), (1000, 256, 1024)])
+def test_plain_bias_relu_rowmajor(dev, dtype, M, K, N):
+    from fastfold_amd import _lib
+    g = torch.Generator().manual_seed(M + K)
+    a = torch.randn(M, K, generator=g).to(dev, dtype)
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).to(dev, dtype)
+    b = torch.randn(N, generator=g).to(dev, dtype)
+    nt = (N + 127) // 128
+    wp, bp = _pack(w, nt), torch.zeros(nt * 128, dtype=dtype, device=dev)
+    bp[:N] = b
+    out = torch.full((M, N), 7.0, dtype=dtype, device=dev)
+    tiles = [_lib.make_tile(out.data_ptr() + i * 128 * out.element_size(), bias=bp.data_ptr() + i * 128 * out.element_size(),
+                            inner=M, s_i=N, act=_lib.FFK_ACT_RELU, ncols=min(128, N - i * 128)) for i in range(nt)]
+    if N % (16 // out.element_size()) != 0:
+        pytest.skip("row pitch not 16-byte aligned")
+    _lib.fused_linear(a, wp, tiles, M=M, K=K)
+    ref = np.maximum(ops_np.linear(_np(a), _np(w), _np(b)), 0)
+    assert _rel(_np(out), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("K", [128, 256])
+def test_layernorm_prologue_resid_gate_inplace(dev, dtype, K):
+    from fastfold_amd import _lib
+    M, N = 333, 128
+    g = torch.Generator().manual_seed(K)
+    a = (torch.randn(M, K, generator=g) * 2 + 0.5).to(dev, dtype)
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).to(dev, dtype)
+    b = torch.randn(N, generator=g).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(K, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(K, generator=g)).to(dev, dtype)
+    gate = torch.rand(M, N, generator=g).to(dev, dtype)
+    z = torch.randn(M, N, generator=g).to(dev, dtype)
+    z0 = z.clone()
+    tiles = [_lib.make_tile(z, bias=b, resid=z, gate=gate, gate_ld=N, inner=M, s_i=N)]
+    _lib.fused_linear(a, _pack(w, 1), tiles, M=M, K=K, ln=(gam, bet))
+    x = ops_np.layer_norm(_np(a), _np(gam), _np(bet))
+    if dtype == torch.bfloat16:
+        x = _np(torch.from_numpy(x).to(torch.bfloat16))       # the kernel rounds LN output to the operand dtype
+    ref = _np(z0) + _np(gate) * ops_np.linear(x, _np(w), _np(b))
+    assert _rel(_np(z), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_transposed_rows_in_and_out(dev, dtype):
+    """A is z[I,J,C] traversed as (j, i); the update is written back to z[i, j]."""
+    from fastfold_amd import _lib
+    I, J, C = 21, 13, 128
+    g = torch.Generator().manual_seed(3)
+    z = torch.randn(I, J, C, generator=g).to(dev, dtype)
+    w = (torch.randn(C, C, generator=g) / C ** 0.5).to(dev, dtype)
+    z0 = z.clone()
+    # logical row m = j * I + i  ->  z[i, j]
+    tiles = [_lib.make_tile(z, resid=z, inner=I, s_o=C, s_i=J * C)]
+    _lib.fused_linear(z0, _pack(w, 1), tiles, M=I * J, K=C, a_inner=I, a_so=C, a_si=J * C)
+    ref = _np(z0) + ops_np.linear(_np(z0), _np(w))
+    assert _rel(_np(z), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("r", [24, 37])
+def test_glu_rowmask_channel_major(dev, dtype, r):
+    """Triangle-multiplication projection: (Wp x + bp) * sigmoid(Wg x + bg) * mask, stored [c][i][kpad]."""
+    from fastfold_amd import _lib
+    C, Ch = 128, 128
+    kpad = (r + 7) // 8 * 8
+    g = torch.Generator().manual_seed(r)
+    z = torch.randn(r, r, C, generator=g).to(dev, dtype)
+    wp = (torch.randn(Ch, C, generator=g) / C ** 0.5).to(dev, dtype)
+    wg = (torch.randn(Ch, C, generator=g) / C ** 0.5).to(dev, dtype)
+    bp, bg = torch.randn(Ch, generator=g).to(dev, dtype), torch.randn(Ch, generator=g).to(dev, dtype)
+    mask = (torch.rand(r, r, generator=g) > 0.2).to(dev, dtype)
+    # packed tiles: [p 0..31 | g 0..31 | p 32..63 | g 32..63] per 128 rows
+    idx = []
+    wcat, bcat = [], []
+    for t in range(Ch // 64):
+        for q in range(2):
+            sl = slice(t * 64 + q * 32, t * 64 + q * 32 + 32)
+            wcat += [wp[sl], wg[sl]]
+            bcat += [bp[sl], bg[sl]]
+    wpk, bpk = torch.cat(wcat).contiguous(), torch.cat(bcat).contiguous()
+    for transposed in (False, True):
+        out = torch.zeros(Ch, r, kpad, dtype=dtype, device=dev)
+        es = out.element_size()
+        tiles = []
+        for t in range(Ch // 64):
+            tiles.append(_lib.make_tile(out.data_ptr() + t * 64 * r * kpad * es, bias=bpk.data_ptr() + t * 128 * es,
+                                        glu=1, ncols=64, inner=r, s_o=kpad, s_i=1, s_h=32 * r * kpad, s_d=r * kpad,
+                                        rowmask=mask, m_so=(1 if transposed else r), m_si=(r if transposed else 1)))
+        if transposed:   # logical row (a, b) reads z[b, a]
+            _lib.fused_linear(z, wpk, tiles, M=r * r, K=C, a_inner=r, a_so=C, a_si=r * C)
+        else:
+            _lib.fused_linear(z, wpk, tiles, M=r * r, K=C)
+        zz = _np(z).transpose(1, 0, 2) if transposed else _np(z)
+        mm = _np(mask).T if transposed else _np(mask)
+        ref = ops_np.linear(zz, _np(wp), _np(bp)) * _sig(ops_np.linear(zz, _np(wg), _np(bg))) * mm[..., None]
+        got = _np(out)[:, :, :r].transpose(1, 2, 0)
+        assert _rel(got, ref) < TOL[dtype]
+        assert float(out[:, :, r:].abs().max()) == 0.0 if kpad > r else True
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B2,N,H", [(3, 70, 4), (2, 32, 8)])
+def test_attention_operand_tiles(dev, dtype, B2, N, H):
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    C = H * 32
+    K = 128
+    g = torch.Generator().manual_seed(N)
+    x = torch.randn(B2, N, K, generator=g).to(dev, dtype)
+    wq, wk, wv = ((torch.randn(C, K, generator=g) / K ** 0.5).to(dev, dtype) for _ in range(3))
+    NT = layouts.n_tiles(N)
+    q = torch.zeros(B2, H, NT, 2, 32, 16, dtype=dtype, device=dev)
+    k = torch.zeros_like(q)
+    v = torch.zeros(B2, H, NT, 2, 32, 4, 4, dtype=dtype, device=dev)
+    es = q.element_size()
+    tiles, ws = [], []
+    for buf, w, kind, scale in ((q, wq, _lib.FFK_TILE_QK, 0.25), (k, wk, _lib.FFK_TILE_QK, 1.0), (v, wv, _lib.FFK_TILE_V, 1.0)):
+        for t in range(C // 128):
+            tiles.append(_lib.make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, inner=N, s_o=H * NT * 1024,
+                                        s_h=NT * 1024, scale=scale))
+            ws.append(w[t * 128:(t + 1) * 128])
+    _lib.fused_linear(x, torch.cat(ws).contiguous(), tiles, M=B2 * N, K=K)
+    for buf, w, un, scale in ((q, wq, layouts.untile_qk, 0.25), (k, wk, layouts.untile_qk, 1.0), (v, wv, layouts.untile_v, 1.0)):
+        ref = (ops_np.linear(_np(x), _np(w)) * scale).reshape(B2, N, H, 32).transpose(0, 2, 1, 3)
+        assert _rel(_np(un(buf, N)), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("r,H", [(45, 4), (64, 8)])
+def test_bias_tiles(dev, dtype, r, H):
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    C = 128
+    g = torch.Generator().manual_seed(r)
+    z = torch.randn(r, r, C, generator=g).to(dev, dtype)
+    wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    T = layouts.n_tiles(r)
+    for transposed in (False, True):
+        bt = torch.zeros(H, T, T, 2, 32, 4, 4, dtype=dtype, device=dev)
+        tile = _lib.make_tile(bt, kind=_lib.FFK_TILE_BIAS, inner=r, s_o=T * 1024, s_h=T * T * 1024, ncols=H, scale=_lib.LOG2E)
+        kw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else {}
+        _lib.fused_linear(z, _pack(wb, 1), [tile], M=r * r, K=C, ln=(gam, bet), **kw)
+        zz = _np(z).transpose(1, 0, 2) if transposed else _np(z)
+        x = ops_np.layer_norm(zz, _np(gam), _np(bet))
+        if dtype == torch.bfloat16:
+            x = _np(torch.from_numpy(x).to(torch.bfloat16))
+        ref = (ops_np.linear(x, _np(wb)) * _lib.LOG2E).transpose(2, 0, 1)       # [h, q, k]
+        assert _rel(_np(layouts.untile_bias(bt, r, r)), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("r", [40, 27])
+def test_channel_major_a_with_layernorm(dev, dtype, r):
+    """Triangle-multiplication output stage: A[(i,j), c] = P[c][i][jpad]."""
+    from fastfold_amd import _lib
+    C = 128
+    jpad = (r + 7) // 8 * 8
+    g = torch.Generator().manual_seed(r)
+    P = torch.randn(C, r, jpad, generator=g).to(dev, dtype)
+    w = (torch.randn(C, C, generator=g) / C ** 0.5).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    b = torch.randn(C, generator=g).to(dev, dtype)
+    gate = torch.rand(r * r, C, generator=g).to(dev, dtype)
+    z = torch.randn(r, r, C, generator=g).to(dev, dtype)
+    z0 = z.clone()
+    tiles = [_lib.make_tile(z, bias=b, resid=z, gate=gate, gate_ld=C, inner=r * r, s_i=C)]
+    _lib.fused_linear(P, _pack(w, 1), tiles, M=r * r, K=C, a_inner=r, a_so=jpad, a_si=1, a_chanmajor=True,
+                      a_cs=r * jpad, ln=(gam, bet))
+    x = ops_np.layer_norm(_np(P)[:, :, :r].transpose(1, 2, 0), _np(gam), _np(bet))
+    if dtype == torch.bfloat16:
+        x = _np(torch.from_numpy(x).to(torch.bfloat16))
+    ref = _np(z0) + _np(gate).reshape(r, r, C) * ops_np.linear(x, _np(w), _np(b))
+    assert _rel(_np(z), ref) < TOL[dtype]
+
+
+def test_bad_descriptors_are_rejected(dev):
+    from fastfold_amd import _lib
+    a = torch.zeros(64, 100, device=dev)
+    w = torch.zeros(128, 100, device=dev)
+    out = torch.zeros(64, 128, device=dev)
+    with pytest.raises(RuntimeError):
+        _lib.fused_linear(a, w, [_lib.make_tile(out, inner=64, s_i=128)], M=64, K=100)     # K % 32
+    a = torch.zeros(64, 128, device=dev)
+    w = torch.zeros(128, 128, device=dev)
+    with pytest.raises(RuntimeError):
+        _lib.fused_linear(a, w, [_lib.make_tile(out, inner=0, s_i=128)], M=64, K=128)      # inner
+    with pytest.raises(RuntimeError):
+        _lib.fused_linear(a, w, [_lib.make_tile(out, inner=64, s_i=128, s_d=2, resid=out)], M=64, K=128)
