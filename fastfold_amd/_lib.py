@@ -170,3 +170,49 @@ def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanma
     for i, t in enumerate(tiles):
         d.tiles[i] = t
     call("ffk_fused_linear", ctypes.byref(d), stream_ptr())
+
+
+# ------------------------------------------------------------------ batched GEMM ----
+class BgemmDesc(ctypes.Structure):
+    """Mirror of ``ffk_bgemm_desc`` (include/ffk.h)."""
+    _fields_ = [
+        ("a", c_void_p), ("b", c_void_p), ("out", c_void_p), ("bias", c_void_p), ("resid", c_void_p),
+        ("rowdiv", c_void_p),
+        ("lda", c_int64), ("ldb", c_int64), ("a_bs", c_int64), ("b_bs", c_int64), ("o_bs", c_int64),
+        ("s_o", c_int64), ("s_i", c_int64), ("s_h", c_int64), ("s_d", c_int64),
+        ("inner", c_int), ("M", c_int), ("N", c_int), ("K", c_int), ("batch", c_int),
+        ("dtype", c_int), ("act", c_int), ("out_f32", c_int),
+        ("scale", c_float), ("div_eps", c_float),
+    ]
+
+
+SIGNATURES["ffk_bgemm_nt"] = [ctypes.POINTER(BgemmDesc), _P]
+SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _I, _P]
+SIGNATURES["ffk_key_bias"] = [_P, _P, _L, _L, _L, _L, _I, _P]
+
+
+def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, inner=None, s_o=0, s_i=None,
+             s_h=32, s_d=1, bias=None, resid=None, rowdiv=None, div_eps=0.0, act=FFK_ACT_NONE, scale=1.0,
+             out_f32=False, dtype=None):
+    """Launches ``ffk_bgemm_nt``; default output addressing is row-major [M, N] (``s_i`` = N)."""
+    def p(t):
+        return None if t is None else (t if isinstance(t, int) else t.data_ptr())
+    d = BgemmDesc()
+    d.a, d.b, d.out, d.bias, d.resid, d.rowdiv = p(a), p(b), p(out), p(bias), p(resid), p(rowdiv)
+    d.lda, d.ldb, d.a_bs, d.b_bs, d.o_bs = lda, ldb, a_bs, b_bs, o_bs
+    d.inner = M if inner is None else inner
+    d.s_o, d.s_i, d.s_h, d.s_d = s_o, (N if s_i is None else s_i), s_h, s_d
+    d.M, d.N, d.K, d.batch = M, N, K, batch
+    d.dtype = dtype_tag(a.dtype if dtype is None else dtype)
+    d.act, d.out_f32, d.scale, d.div_eps = act, 1 if out_f32 else 0, scale, div_eps
+    call("ffk_bgemm_nt", ctypes.byref(d), stream_ptr())
+
+
+def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, gate, *, B2, H, Nq, Nk):
+    call("ffk_attention_fwd", ptr(out), ptr(q_t), ptr(k_t), ptr(v_t), ptr(bias_t), ptr(keybias), ptr(gate),
+         B2, H, Nq, Nk, dtype_tag(q_t.dtype), stream_ptr())
+
+
+def key_bias(keybias, mask, *, B, N, mask_sb=0, mask_sn=1):
+    call("ffk_key_bias", ptr(keybias), ptr(mask), B, N, mask_sb, mask_sn,
+         dtype_tag(mask.dtype) if mask is not None else FFK_F32, stream_ptr())

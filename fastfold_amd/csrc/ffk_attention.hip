@@ -1,0 +1,220 @@
+// Flash-style attention for head dimension 32 (see ffk_attention_fwd in include/ffk.h).
+//
+// One wavefront owns 32 queries of one (b2, head) and walks the keys 32 at a time; the
+// four waves of a workgroup take consecutive query tiles of the same (b2, head), so their
+// K / V tile reads hit the same lines.  There is no LDS and no barrier: every operand is
+// stored in HBM in exactly the order a wave consumes it (1024-element tiles, 16 contiguous
+// elements per lane).
+//
+// The score tile is computed transposed, S^T = K . Q^T (rows = keys, columns = queries):
+// a lane then holds 16 keys of ONE query, so the running max / sum are per-lane scalars
+// (one cross-half shuffle per tile), and exp2(S^T - max) is already in the operand layout
+// of the second MFMA  O^T += V^T . P^T  - no transpose of P.  The additive bias tile is
+// stored in accumulator order and simply initialises the accumulator of S^T.
+#include "ffk_common.h"
+
+namespace {
+
+constexpr int THREADS = 256;
+constexpr float NEG_BIG = -3.0e38f;
+
+template <typename T> struct Ops16 {   // the 16 elements one lane owns of a 1024-element tile
+    static constexpr int NV = 16 / DT<T>::VEC;
+    Vec16<T> v[NV];
+    __device__ __forceinline__ void load(const T* p) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) v[i] = ld16(p + i * DT<T>::VEC);
+    }
+    __device__ __forceinline__ float f(int j) const { return DT<T>::to_f(v[j / DT<T>::VEC].e[j % DT<T>::VEC]); }
+    // MFMA fragment number i (KLANE elements each)
+    __device__ __forceinline__ typename Mma<T>::Frag frag(int i) const {
+        return *reinterpret_cast<const typename Mma<T>::Frag*>(&v[i]);
+    }
+};
+
+template <typename T> struct PFrag;
+template <> struct PFrag<bf16_t> {
+    static __device__ __forceinline__ bf16x8 make(const float* p) {
+        bf16x8 r;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r[t] = (bf16_t)p[t];
+        return r;
+    }
+};
+template <> struct PFrag<float> {
+    static __device__ __forceinline__ f32x4 make(const float* p) {
+        f32x4 r;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) r[t] = p[t];
+        return r;
+    }
+};
+
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(THREADS) void attention_kernel(T* __restrict__ out, const T* __restrict__ q_t,
+                                                           const T* __restrict__ k_t, const T* __restrict__ v_t,
+                                                           const T* __restrict__ bias_t,
+                                                           const float* __restrict__ keybias,
+                                                           const T* __restrict__ gate, int H, int Nq, int Nk) {
+    typedef Mma<T> MM;
+    constexpr int NF = 16 / MM::KLANE;            // fragments per 16-element lane slice (bf16 2, fp32 4)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
+    const int qt = blockIdx.x * 4 + wave;
+    if (qt >= QT) return;
+    const int h = blockIdx.y, b2 = blockIdx.z;
+    const long bh = (long)b2 * H + h;
+
+    Ops16<T> qf;
+    qf.load(q_t + ((bh * QT + qt) << 10) + lane * 16);
+    const T* kp = k_t + ((bh * KT) << 10) + lane * 16;
+    const T* vp = v_t + ((bh * KT) << 10) + lane * 16;
+    const T* bp = HAS_BIAS ? bias_t + ((((long)h * QT + qt) * KT) << 10) + lane * 16 : nullptr;
+    const float* mp = keybias + (long)b2 * KT * 32 + 4 * half;
+
+    f32x16 o_acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o_acc[v] = 0.0f;
+    float m_run = NEG_BIG, l_run = 0.0f;
+
+    Ops16<T> kc, vc, bc;
+    f32x4 mc[4];
+    auto load_tile = [&](int kt, Ops16<T>& kk, Ops16<T>& vv, Ops16<T>& bb, f32x4* mm) {
+        kk.load(kp + ((long)kt << 10));
+        vv.load(vp + ((long)kt << 10));
+        if (HAS_BIAS) bb.load(bp + ((long)kt << 10));
+#pragma unroll
+        for (int g = 0; g < 4; ++g) mm[g] = *reinterpret_cast<const f32x4*>(mp + kt * 32 + 8 * g);
+    };
+    load_tile(0, kc, vc, bc, mc);
+
+    for (int kt = 0; kt < KT; ++kt) {
+        Ops16<T> kn, vn, bn;
+        f32x4 mn[4];
+        if (kt + 1 < KT) load_tile(kt + 1, kn, vn, bn, mn);
+
+        // S^T = bias + K . Q^T   (rows: keys, columns: queries)
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = HAS_BIAS ? bc.f(v) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
+
+        float p[16];
+        float mt = NEG_BIG;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            p[v] = s[v] + mc[v >> 2][v & 3];
+            mt = fmaxf(mt, p[v]);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m_run, mt);
+        const float alpha = fast_exp2(m_run - m_new);
+        float ls = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            p[v] = fast_exp2(p[v] - m_new);
+            ls += p[v];
+        }
+        l_run = l_run * alpha + ls;
+        m_run = m_new;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o_acc[v] *= alpha;
+
+        // O^T += V^T . P^T   (rows: head dim, columns: queries)
+#pragma unroll
+        for (int i = 0; i < NF; ++i) MM::mma(o_acc, vc.frag(i), PFrag<T>::make(p + i * MM::KLANE));
+
+        if (kt + 1 < KT) {
+            kc = kn;
+            vc = vn;
+            if (HAS_BIAS) bc = bn;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) mc[g] = mn[g];
+        }
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / l_tot;
+    const int q = qt * 32 + l32;
+    if (q < Nq) {
+        const long rowo = ((long)b2 * Nq + q) * (H * 32) + h * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            T r4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float x = o_acc[4 * g + e] * inv;
+                if (gate) x *= DT<T>::to_f(gate[rowo + 8 * g + e]);
+                r4[e] = DT<T>::from_f(x);
+            }
+            T* dst = out + rowo + 8 * g;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = r4[e];
+        }
+    }
+}
+
+template <typename T>
+__global__ void key_bias_kernel(float* kb, const T* mask, long B, long N, long Npad, long sb, long sn) {
+    const long total = B * Npad;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long b = i / Npad, k = i % Npad;
+        float v = 0.0f;
+        if (k >= N) v = NEG_BIG;
+        else if (mask && DT<T>::to_f(mask[b * sb + k * sn]) == 0.0f) v = -1e9f * 1.4426950408889634f;
+        kb[i] = v;
+    }
+}
+
+template <typename T>
+int launch_attention(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
+                     const void* gate, long B2, long H, long Nq, long Nk, hipStream_t st) {
+    dim3 grid(ffk_cdiv((Nq + 31) / 32, 4), (unsigned)H, (unsigned)B2);
+    if (bias)
+        attention_kernel<T, true><<<grid, THREADS, 0, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
+                                                          (const T*)bias, kb, (const T*)gate, (int)H, (int)Nq, (int)Nk);
+    else
+        attention_kernel<T, false><<<grid, THREADS, 0, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v, nullptr,
+                                                           kb, (const T*)gate, (int)H, (int)Nq, (int)Nk);
+    return ffk_check_launch("ffk_attention_fwd");
+}
+
+}  // namespace
+
+extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t, const void* bias_t,
+                                 const float* keybias, const void* gate, int64_t B2, int64_t H, int64_t Nq,
+                                 int64_t Nk, int dtype, void* stream) {
+    FFK_REQUIRE(out && q_t && k_t && v_t && keybias, FFK_ERR_NULL, "ffk_attention_fwd: null pointer");
+    FFK_REQUIRE(B2 > 0 && B2 < 65536 && H > 0 && H < 65536 && Nq > 0 && Nk > 0 && Nq < (1 << 24) && Nk < (1 << 24),
+                FFK_ERR_SHAPE, "ffk_attention_fwd: bad shape B2=%ld H=%ld Nq=%ld Nk=%ld", (long)B2, (long)H, (long)Nq,
+                (long)Nk);
+    FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(q_t) && ffk_aligned16(k_t) && ffk_aligned16(v_t) &&
+                    ffk_aligned16(keybias) && (!bias_t || ffk_aligned16(bias_t)) && (!gate || ffk_aligned16(gate)),
+                FFK_ERR_ALIGN, "ffk_attention_fwd: buffers must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FFK_BF16: return launch_attention<bf16_t>(out, q_t, k_t, v_t, bias_t, keybias, gate, B2, H, Nq, Nk, st);
+        case FFK_F32: return launch_attention<float>(out, q_t, k_t, v_t, bias_t, keybias, gate, B2, H, Nq, Nk, st);
+        default: return ffk_fail(FFK_ERR_DTYPE, "ffk_attention_fwd: unsupported dtype tag %d", dtype);
+    }
+}
+
+extern "C" int ffk_key_bias(float* keybias, const void* mask, int64_t B, int64_t N, int64_t mask_sb, int64_t mask_sn,
+                            int dtype, void* stream) {
+    FFK_REQUIRE(keybias, FFK_ERR_NULL, "ffk_key_bias: null pointer");
+    FFK_REQUIRE(B > 0 && N > 0, FFK_ERR_SHAPE, "ffk_key_bias: bad shape B=%ld N=%ld", (long)B, (long)N);
+    const long Npad = (N + 31) / 32 * 32;
+    const long total = B * Npad;
+    long blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FFK_BF16: key_bias_kernel<bf16_t><<<dim3((int)blocks), 256, 0, st>>>(keybias, (const bf16_t*)mask, B, N, Npad, mask_sb, mask_sn); break;
+        case FFK_F32: key_bias_kernel<float><<<dim3((int)blocks), 256, 0, st>>>(keybias, (const float*)mask, B, N, Npad, mask_sb, mask_sn); break;
+        case FFK_F16: key_bias_kernel<f16_t><<<dim3((int)blocks), 256, 0, st>>>(keybias, (const f16_t*)mask, B, N, Npad, mask_sb, mask_sn); break;
+        default: return ffk_fail(FFK_ERR_DTYPE, "ffk_key_bias: unsupported dtype tag %d", dtype);
+    }
+    return ffk_check_launch("ffk_key_bias");
+}

@@ -167,6 +167,70 @@ typedef struct ffk_linear_desc {
 
 int ffk_fused_linear(const ffk_linear_desc* desc, void* stream);
 
+
+/* ------------------------------------------------------------------------------------
+ * Batched "NT" GEMM with a K loop:  C[b] = epilogue( A[b][M,K] . B[b][N,K]^T )
+ *
+ * Both operands are K-contiguous (row strides lda / ldb, batch strides a_bs / b_bs, all in
+ * elements; K % 8 == 0 for bf16, % 4 for fp32; rows 16-byte aligned).  The epilogue computes
+ *     v = act(acc + bias[n]) * scale ;  v /= (rowdiv[m] + div_eps) ;  v += resid[m, n]
+ * and stores element (m, n) of batch b at
+ *     out + b * o_bs + (m / inner) * s_o + (m % inner) * s_i + (n / 32) * s_h + (n % 32) * s_d.
+ * out_f32 != 0 stores fp32 regardless of the operand dtype (used for the outer-product-mean
+ * normaliser).  resid uses the output addressing and may alias out.
+ *
+ * Used for: the triangle-multiplication contraction p[c,i,j] = sum_k l[c,i,k] r[c,j,k]
+ * (torch.matmul of permuted operands, fastfold/model/fastnn/ops.py:400-403,529-532), the
+ * outer-product-mean einsum and its output projection (ops.py:152,158-161,173) and the second
+ * linear of the transitions (ops.py:81,96).
+ */
+typedef struct ffk_bgemm_desc {
+    const void* a;
+    const void* b;
+    void* out;
+    const void* bias;      /* [N] operand dtype, or NULL */
+    const void* resid;     /* or NULL */
+    const float* rowdiv;   /* fp32 [M] (per batch: + b * M), or NULL */
+    int64_t lda, ldb, a_bs, b_bs, o_bs;
+    int64_t s_o, s_i, s_h, s_d;
+    int32_t inner;
+    int32_t M, N, K, batch;
+    int32_t dtype, act, out_f32;
+    float scale, div_eps;
+} ffk_bgemm_desc;
+
+int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
+
+
+/* ------------------------------------------------------------------------------------
+ * Flash-style attention core for head dimension 32 (logits never reach HBM):
+ *     o[b2, q, h, :] = softmax_k( q.k^T + bias[h, q, k] + keybias[b2, k] ) . v   (* gate)
+ * in the exp2 domain: q must already carry the factor  d^-1/2 * log2(e)  and bias the
+ * factor log2(e); keybias is fp32 (0 for a valid key, -1e9*log2e for a masked key and a
+ * hugely negative finite value for the padding up to a multiple of 32; build it with
+ * ffk_key_bias).  Operands arrive in 32x32 operand tiles (1024 elements, see
+ * ffk_fused_linear tile kinds):
+ *   q_t, k_t : [B2][H][ceil(N/32)][1024]   FFK_TILE_QK order
+ *   v_t      : [B2][H][ceil(Nk/32)][1024]  FFK_TILE_V  order
+ *   bias_t   : [H][ceil(Nq/32)][ceil(Nk/32)][1024]  FFK_TILE_BIAS order, or NULL
+ *   keybias  : [B2][ceil(Nk/32)*32] fp32
+ *   gate     : [B2*Nq, H*32] row-major multiplicative gate (already sigmoid-ed), or NULL
+ *   out      : [B2*Nq, H*32] row-major
+ * Replaces: the matmul / fused_softmax / matmul (+ bias_sigmod_ele) chain of
+ * SelfAttention.forward (fastfold/model/fastnn/ops.py:310-322) and
+ * fused_attention_core (kernel/attention_core.py:17-52, kernel/triton/attention_core.py:12-190).
+ */
+int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t,
+                      const void* bias_t, const float* keybias, const void* gate,
+                      int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int dtype, void* stream);
+
+/* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
+ * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the
+ * given dtype, or NULL (all keys valid).  Replaces the `1e9 * (mask - 1)` key-padding term of
+ * the reference (ops.py:313, kernel/triton/softmax.py:17-19). */
+int ffk_key_bias(float* keybias, const void* mask, int64_t B, int64_t N, int64_t mask_sb,
+                 int64_t mask_sn, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

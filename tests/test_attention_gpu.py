@@ -1,0 +1,140 @@
+"""GPU parity of the flash attention core and the batched NT GEMM (through the C ABI)
+against the float64 numpy oracle."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops_np
+
+pytestmark = pytest.mark.gpu
+
+LOG2E = 1.4426950408889634
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def _rel(got, ref):
+    return np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("B2,H,N,use_bias,use_gate", [(3, 4, 70, True, True), (2, 8, 32, False, False),
+                                                      (1, 4, 257, True, False), (5, 2, 129, False, True),
+                                                      (2, 4, 300, True, True)])
+def test_attention_core(dev, dtype, tol, B2, H, N, use_bias, use_gate):
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    g = torch.Generator().manual_seed(N + H)
+    q, k, v = (torch.randn(1, B2, H, N, 32, generator=g).to(dev, dtype) for _ in range(3))
+    bias = (2 * torch.randn(1, H, N, N, generator=g)).to(dev, dtype) if use_bias else None
+    mask = (torch.rand(1, B2, N, generator=g) > 0.2).to(dev, dtype)
+    mask[..., 1] = 1
+    gate = torch.rand(B2 * N, H * 32, generator=g).to(dev, dtype) if use_gate else None
+    scale = LOG2E / math.sqrt(32)
+    qs = (q.float() * scale).to(dtype)       # what the projection epilogue would have written
+    qt, kt, vt = layouts.tile_qk(qs[0]), layouts.tile_qk(k[0]), layouts.tile_v(v[0])
+    bt = layouts.tile_bias((bias[0].float() * LOG2E).to(dtype)) if use_bias else None
+    NT = layouts.n_tiles(N)
+    kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
+    _lib.key_bias(kb, mask[0], B=B2, N=N, mask_sb=N, mask_sn=1)
+    assert float(kb[:, :N][mask[0] != 0].abs().max()) == 0.0 and float(kb[:, :N][mask[0] == 0].max()) < -1e9
+    out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
+    _lib.attention_fwd(out, qt, kt, vt, bt, kb, gate, B2=B2, H=H, Nq=N, Nk=N)
+    # oracle on exactly the operands the kernel saw (q rounded after scaling, bias rounded after log2e)
+    q_eff = _np(qs) / scale * math.sqrt(32) / math.sqrt(32)
+    b_eff = _np((bias[0].float() * LOG2E).to(dtype))[None] / LOG2E if use_bias else None
+    ref = ops_np.attention_core(q_eff, _np(k), _np(v), _np(mask), b_eff)[0]          # [B2, N, H*32]
+    if use_gate:
+        ref = ref * _np(gate).reshape(B2, N, H * 32)
+    assert _rel(_np(out).reshape(B2, N, H * 32), ref) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_attention_tiling_invariance_and_masked_keys(dev, dtype, tol):
+    """Changing K/V at masked keys must not change the output; all-valid mask == no mask."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    B2, H, N = 2, 4, 100
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(B2, H, N, 32, generator=g).to(dev, dtype) for _ in range(3))
+    mask = torch.ones(B2, N, device=dev, dtype=dtype)
+    mask[:, 90:] = 0
+    kb = torch.empty(B2, 128, dtype=torch.float32, device=dev)
+    _lib.key_bias(kb, mask, B=B2, N=N, mask_sb=N, mask_sn=1)
+    outs = []
+    for delta in (0.0, 5.0):
+        k2, v2 = k.clone(), v.clone()
+        k2[:, :, 90:] += delta
+        v2[:, :, 90:] -= delta
+        out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
+        _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k2), layouts.tile_v(v2), None, kb, None,
+                           B2=B2, H=H, Nq=N, Nk=N)
+        outs.append(_np(out))
+    assert np.abs(outs[0] - outs[1]).max() == 0.0
+    # same as attending over the first 90 keys only
+    kb90 = torch.empty(B2, 96, dtype=torch.float32, device=dev)
+    _lib.key_bias(kb90, None, B=B2, N=90)
+    out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
+    _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k[:, :, :90].contiguous()),
+                       layouts.tile_v(v[:, :, :90].contiguous()), None, kb90, None, B2=B2, H=H, Nq=N, Nk=90)
+    assert _rel(_np(out), outs[0]) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("r", [52, 128, 200])
+def test_bgemm_trimul_contraction(dev, dtype, tol, r):
+    """p[c,i,j] = sum_k l[c,i,k] r[c,j,k] on channel-major, K-padded operands."""
+    from fastfold_amd import _lib
+    C = 16
+    kpad = (r + 7) // 8 * 8
+    g = torch.Generator().manual_seed(r)
+    left = torch.zeros(C, r, kpad, dtype=dtype, device=dev)
+    right = torch.zeros(C, r, kpad, dtype=dtype, device=dev)
+    left[:, :, :r] = torch.randn(C, r, r, generator=g).to(dev, dtype)
+    right[:, :, :r] = torch.randn(C, r, r, generator=g).to(dev, dtype)
+    out = torch.zeros(C, r, kpad, dtype=dtype, device=dev)
+    _lib.bgemm_nt(left, right, out, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=C, a_bs=r * kpad, b_bs=r * kpad,
+                  o_bs=r * kpad, s_i=kpad)
+    a = _np(left)[:, :, :r].transpose(1, 2, 0)      # [i, k, c]
+    b = _np(right)[:, :, :r].transpose(1, 2, 0)     # [j, k, c]
+    ref = ops_np.trimul_outgoing(a, b)              # [i, j, c]
+    assert _rel(_np(out)[:, :, :r].transpose(1, 2, 0), ref) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("s,r", [(24, 10), (128, 9), (50, 33)])
+def test_bgemm_outer_product_and_projection(dev, dtype, tol, s, r):
+    """OPM: O[(i,j),(d,e)] = sum_s a[s,i,d] b[s,j,e] from K-padded transposed operands, then
+    z + (O Wo^T + bo) / (norm + eps) with an fp32 normaliser."""
+    from fastfold_amd import _lib
+    spad = (s + 7) // 8 * 8
+    g = torch.Generator().manual_seed(s + r)
+    a = torch.randn(s, r, 32, generator=g).to(dev, dtype)
+    b = torch.randn(s, r, 32, generator=g).to(dev, dtype)
+    aT = torch.zeros(r * 32, spad, dtype=dtype, device=dev)
+    bT = torch.zeros(r * 32, spad, dtype=dtype, device=dev)
+    aT[:, :s] = a.permute(1, 2, 0).reshape(r * 32, s)
+    bT[:, :s] = b.permute(1, 2, 0).reshape(r * 32, s)
+    O = torch.zeros(r * r, 1024, dtype=dtype, device=dev)
+    _lib.bgemm_nt(aT, bT, O, M=32 * r, N=32 * r, K=spad, lda=spad, ldb=spad, inner=32, s_o=r * 1024, s_i=32,
+                  s_h=1024, s_d=1)
+    ref_o = ops_np.outer_product(_np(a), _np(b)).reshape(r * r, 1024)
+    assert _rel(_np(O), ref_o) < tol
+    wo = (torch.randn(128, 1024, generator=g) / 32).to(dev, dtype)
+    bo = torch.randn(128, generator=g).to(dev, dtype)
+    norm = (torch.rand(r * r, generator=g) * s).to(dev)
+    z = torch.randn(r * r, 128, generator=g).to(dev, dtype)
+    z0 = z.clone()
+    _lib.bgemm_nt(O, wo, z, M=r * r, N=128, K=1024, lda=1024, ldb=1024, bias=bo, resid=z, rowdiv=norm, div_eps=1e-3)
+    ref = _np(z0) + ops_np.linear(_np(O), _np(wo), _np(bo)) / (_np(norm)[:, None] + 1e-3)
+    assert _rel(_np(z), ref) < tol
+    # fp32 output of a bf16 product (mask normaliser): exact small integers
+    mk = (torch.rand(r, spad, generator=g) > 0.3).to(dev, dtype)
+    mk[:, s:] = 0
+    nrm = torch.empty(r, r, dtype=torch.float32, device=dev)
+    _lib.bgemm_nt(mk, mk, nrm, M=r, N=r, K=spad, lda=spad, ldb=spad, out_f32=True)
+    assert np.array_equal(_np(nrm), _np(mk) @ _np(mk).T)
