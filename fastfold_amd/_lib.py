@@ -146,11 +146,11 @@ def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, g
 
 
 def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanmajor=False, a_cs=0,
-                 ln=None, eps=1e-5):
-    """Launches ``ffk_fused_linear``.  ``a`` / ``w`` are tensors (``w`` packed [n_tiles*128, K]);
-    ``ln`` is ``(gamma, beta)`` or None."""
+                 ln=None, eps=1e-5, a_off=0, w_row_off=0):
+    """Launches ``ffk_fused_linear``.  ``a`` / ``w`` are tensors (``w`` packed [>= n_tiles*128, K]);
+    ``ln`` is ``(gamma, beta)`` or None; ``a_off`` (elements) / ``w_row_off`` (rows) offset the bases."""
     d = LinearDesc()
-    d.a = a.data_ptr()
+    d.a = a.data_ptr() + a_off * a.element_size()
     d.a_inner = M if a_inner is None else a_inner
     d.a_so = a_so
     d.a_si = K if a_si is None else a_si
@@ -160,11 +160,11 @@ def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanma
         d.ln_gamma, d.ln_beta = ln[0].data_ptr(), ln[1].data_ptr()
     d.ln_eps = eps
     d.dtype = dtype_tag(a.dtype)
-    d.w = w.data_ptr()
+    d.w = w.data_ptr() + w_row_off * K * w.element_size()
     d.M, d.K, d.n_tiles = M, K, len(tiles)
     if len(tiles) > FFK_MAX_TILES:
         raise RuntimeError("fused_linear: at most %d N-tiles per launch" % FFK_MAX_TILES)
-    if w.shape[0] != 128 * len(tiles) or w.shape[1] != K or w.dtype != a.dtype:
+    if w.shape[0] < w_row_off + 128 * len(tiles) or w.shape[1] != K or w.dtype != a.dtype:
         raise RuntimeError("fused_linear: packed weight must be [%d, %d] %s, got %s %s"
                            % (128 * len(tiles), K, a.dtype, tuple(w.shape), w.dtype))
     for i, t in enumerate(tiles):

@@ -1,0 +1,262 @@
+"""Launch sequences of the HIP kernels for each Evoformer sub-module (single GPU, DAP size 1).
+
+These functions take plain tensors plus weights already packed for the kernels and issue
+C-ABI calls only; torch is used for buffer allocation and for re-packing weights (once per
+weight version).  Row-addressing conventions are those of ``ffk_fused_linear``: logical row
+``m = hi * inner + lo`` lives at ``hi * s_o + lo * s_i``.
+"""
+import math
+
+import torch
+
+from fastfold_amd import _lib
+from fastfold_amd._lib import (FFK_ACT_NONE, FFK_ACT_RELU, FFK_ACT_SIGMOID, FFK_TILE_BIAS, FFK_TILE_QK,
+                               FFK_TILE_STRIDED, FFK_TILE_V, LOG2E, make_tile)
+
+_WS_BUDGET_DEFAULT = 6 << 30     # bytes of scratch one sub-module may hold at a time
+_WS_BUDGET_CHUNKED = 1 << 30     # when the user asked for chunking (set_chunk_size)
+
+
+def es_of(dtype):
+    return 4 if dtype == torch.float32 else 2
+
+
+def vec_of(dtype):
+    return 16 // es_of(dtype)
+
+
+def round_up(x, m):
+    return (x + m - 1) // m * m
+
+
+def alloc(shape, dtype, device, zero=False):
+    return (torch.zeros if zero else torch.empty)(shape, dtype=dtype, device=device)
+
+
+def pack_rows(mats, dtype, device):
+    """cat([n_i, K]) zero-padded to a multiple of 128 rows, in the kernel dtype."""
+    w = torch.cat([m.detach().to(device=device, dtype=dtype) for m in mats], 0)
+    n, npad = w.shape[0], round_up(w.shape[0], 128)
+    if npad != n:
+        w = torch.cat([w, w.new_zeros(npad - n, w.shape[1])], 0)
+    return w.contiguous()
+
+
+def pack_vec(vecs, dtype, device, total=None):
+    v = torch.cat([x.detach().to(device=device, dtype=dtype).reshape(-1) for x in vecs], 0)
+    total = round_up(v.numel(), 128) if total is None else total
+    if total != v.numel():
+        v = torch.cat([v, v.new_zeros(total - v.numel())], 0)
+    return v.contiguous()
+
+
+def check_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("fastfold_amd: the Evoformer modules run on the GPU only "
+                               "(got a %s tensor); there is no CPU fallback" % t.device)
+
+
+def fits_fused(K, dtype):
+    bk = 32 if dtype == torch.float32 else 64
+    return K <= 256 and K % bk == 0
+
+
+# ------------------------------------------------------------------------- linear ----
+def linear(x2, w_pk, b_pk, N, *, act=FFK_ACT_NONE, out=None, resid=None, ln=None):
+    """out[M, N] = act(LN(x2)[M, K] @ W^T + b) (+ resid).  ``w_pk`` is [>=N (padded to 128), K]."""
+    M, K = x2.shape
+    dt, dev = x2.dtype, x2.device
+    es = es_of(dt)
+    if out is None:
+        out = torch.empty(M, N, dtype=dt, device=dev)
+    if M == 0:
+        return out
+    if fits_fused(K, dt) and N % vec_of(dt) == 0:
+        nt = (N + 127) // 128
+        for t0 in range(0, nt, _lib.FFK_MAX_TILES):
+            tiles = []
+            for t in range(t0, min(nt, t0 + _lib.FFK_MAX_TILES)):
+                tiles.append(make_tile(out.data_ptr() + t * 128 * es,
+                                       bias=None if b_pk is None else b_pk.data_ptr() + t * 128 * es,
+                                       resid=None if resid is None else resid.data_ptr() + t * 128 * es,
+                                       inner=M, s_i=N, act=act, ncols=min(128, N - t * 128)))
+            _lib.fused_linear(x2, w_pk, tiles, M=M, K=K, ln=ln, w_row_off=t0 * 128)
+    else:
+        if ln is not None:
+            raise RuntimeError("linear: LayerNorm prologue needs K <= 256")
+        if K % vec_of(dt) != 0:
+            raise RuntimeError("linear: in_features=%d must be a multiple of %d for %s" % (K, vec_of(dt), dt))
+        _lib.bgemm_nt(x2, w_pk, out, M=M, N=N, K=K, lda=K, ldb=K, bias=b_pk, resid=resid, act=act)
+    return out
+
+
+# --------------------------------------------------------------------- transition ----
+def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
+    """out = x + W2 relu(W1 LN(x) + b1) + b2 over rows of x [M, C]; out may alias x."""
+    M, C = x.shape
+    dt, dev = x.dtype, x.device
+    es = es_of(dt)
+    rows = max(128, min(M, (budget // (hidden * es)) // 128 * 128))
+    hid = torch.empty(min(rows, M), hidden, dtype=dt, device=dev)
+    nt = hidden // 128
+    for r0 in range(0, M, rows):
+        n = min(rows, M - r0)
+        for t0 in range(0, nt, _lib.FFK_MAX_TILES):
+            tiles = [make_tile(hid.data_ptr() + t * 128 * es, bias=b1_pk.data_ptr() + t * 128 * es, inner=n,
+                               s_i=hidden, act=FFK_ACT_RELU)
+                     for t in range(t0, min(nt, t0 + _lib.FFK_MAX_TILES))]
+            _lib.fused_linear(x, w1_pk, tiles, M=n, K=C, ln=ln, a_off=r0 * C, w_row_off=t0 * 128)
+        _lib.bgemm_nt(hid, w2, out.data_ptr() + r0 * C * es, M=n, N=C, K=hidden, lda=hidden, ldb=hidden, bias=b2,
+                      resid=x.data_ptr() + r0 * C * es, dtype=dt)
+    return out
+
+
+# ---------------------------------------------------------------------- attention ----
+def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_pk, out_bias_pk, c_out,
+              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False):
+    """Gated multi-head attention (head dim 32) over N tokens for each of B2 batch rows.
+
+    x holds the C-channel rows addressed by ``a_map = (inner, s_o, s_i)``; w_pk is the packed
+    [q; k; v; gate(; bias)] weight.  The attention update is projected by wo_pk and written as
+    ``out = resid + update + out_bias`` with the same row addressing (``resid=None``: no residual).
+    With ``bias_in_launch`` the last N-tile of w_pk produces the [H, N, N] additive bias into
+    ``bias_t`` from the same normalised rows.
+    """
+    dt, dev = x.dtype, x.device
+    es = es_of(dt)
+    HC = H * 32
+    if HC % 128 != 0:
+        raise RuntimeError("attention: n_head * 32 must be a multiple of 128 (got %d heads)" % H)
+    M = B2 * N
+    NT = (N + 31) // 32
+    zero = (N % 32) != 0
+    q_t = alloc((B2, H, NT, 1024), dt, dev, zero)
+    k_t = alloc((B2, H, NT, 1024), dt, dev, zero)
+    v_t = alloc((B2, H, NT, 1024), dt, dev, zero)
+    gate = torch.empty(M, HC, dtype=dt, device=dev)
+    tpg = HC // 128
+    qscale = LOG2E / math.sqrt(32.0)
+    tiles = []
+    for buf, kind, scale in ((q_t, FFK_TILE_QK, qscale), (k_t, FFK_TILE_QK, 1.0), (v_t, FFK_TILE_V, 1.0)):
+        for t in range(tpg):
+            tiles.append(make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, inner=N,
+                                   s_o=H * NT * 1024, s_h=NT * 1024, scale=scale))
+    for t in range(tpg):
+        tiles.append(make_tile(gate.data_ptr() + t * 128 * es, bias=gate_bias_pk.data_ptr() + t * 128 * es,
+                               inner=M, s_i=HC, act=FFK_ACT_SIGMOID))
+    if bias_in_launch:
+        tiles.append(make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H,
+                               scale=LOG2E))
+    a_inner, a_so, a_si = a_map
+    _lib.fused_linear(x, w_pk, tiles, M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln)
+    kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
+    _lib.key_bias(kb, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
+    o = torch.empty(M, HC, dtype=dt, device=dev)
+    _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, gate, B2=B2, H=H, Nq=N, Nk=N)
+    del q_t, k_t, v_t, gate
+    tiles = []
+    for t in range((c_out + 127) // 128):
+        tiles.append(make_tile(out.data_ptr() + t * 128 * es,
+                               bias=None if out_bias_pk is None else out_bias_pk.data_ptr() + t * 128 * es,
+                               resid=None if resid is None else resid.data_ptr() + t * 128 * es,
+                               inner=a_inner, s_o=a_so, s_i=a_si, ncols=min(128, c_out - t * 128)))
+    _lib.fused_linear(o, wo_pk, tiles, M=M, K=HC)
+    return out
+
+
+def pair_bias(z, *, r, C, H, ln, wb_pk):
+    """bias_t[h][q/32][k/32][tile] = log2e * (LN(z)[q, k, :] . Wb[h, :]) in score-accumulator tiles."""
+    NT = (r + 31) // 32
+    bias_t = alloc((H, NT, NT, 1024), z.dtype, z.device, zero=(r % 32) != 0)
+    tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=r, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H, scale=LOG2E)
+    _lib.fused_linear(z, wb_pk, [tile], M=r * r, K=C, ln=ln)
+    return bias_t
+
+
+# ----------------------------------------------------------- triangle multiplication ----
+def pack_trimul(proj_w, proj_b, gate_w, gate_b, og_w, og_b, c, dtype, device):
+    """[left GLU tiles | right GLU tiles | output-gate tiles]; a GLU tile packs 64 channels as
+    [p c0..c0+31 | g c0..c0+31 | p c0+32..c0+63 | g c0+32..c0+63]."""
+    if c % 64 != 0:
+        raise RuntimeError("triangle multiplication: hidden width must be a multiple of 64, got %d" % c)
+    ws, bs = [], []
+    for side in range(2):
+        for t in range(c // 64):
+            for q in range(2):
+                sl = slice(side * c + t * 64 + q * 32, side * c + t * 64 + q * 32 + 32)
+                ws += [proj_w[sl], gate_w[sl]]
+                bs += [proj_b[sl], gate_b[sl]]
+    n_glu = 2 * (c // 64)
+    w = pack_rows(ws, dtype, device)
+    b = pack_vec(bs, dtype, device)
+    wg = pack_rows([og_w], dtype, device)
+    bg = pack_vec([og_b], dtype, device)
+    return torch.cat([w, wg], 0).contiguous(), torch.cat([b, bg], 0).contiguous(), n_glu
+
+
+def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask):
+    """out = z + sigmoid(Wg LN(z) + bg) * (Wout LN2(p) + b_out),  p[i,j,:] = sum_k a[i,k,:] b[j,k,:]
+    (outgoing) or sum_k a[k,i,:] b[k,j,:] (incoming), a/b the masked gated projections."""
+    dt, dev = z.dtype, z.device
+    es = es_of(dt)
+    M = r * r
+    kpad = round_up(r, vec_of(dt))
+    zero = kpad != r
+    lr = alloc((2, c, r, kpad), dt, dev, zero)
+    g = torch.empty(M, C, dtype=dt, device=dev)
+    tiles = []
+    if incoming:      # logical row (a, b) reads z[b, a]
+        a_map, m_so, m_si = (r, C, r * C), 1, r
+    else:
+        a_map, m_so, m_si = (M, 0, C), r, 1
+    for side in range(2):
+        for t in range(c // 64):
+            ti = side * (c // 64) + t
+            tiles.append(make_tile(lr.data_ptr() + (side * c + t * 64) * r * kpad * es,
+                                   bias=b_pk.data_ptr() + ti * 128 * es, glu=1, ncols=64, inner=r, s_o=kpad, s_i=1,
+                                   s_h=32 * r * kpad, s_d=r * kpad, rowmask=mask, m_so=m_so, m_si=m_si))
+    for t in range((C + 127) // 128):
+        kw = dict(inner=r, s_o=C, s_i=r * C) if incoming else dict(inner=M, s_i=C)
+        tiles.append(make_tile(g.data_ptr() + t * 128 * es, bias=b_pk.data_ptr() + (n_glu + t) * 128 * es,
+                               act=FFK_ACT_SIGMOID, ncols=min(128, C - t * 128), **kw))
+    _lib.fused_linear(z, w_pk, tiles, M=M, K=C, a_inner=a_map[0], a_so=a_map[1], a_si=a_map[2], ln=ln1)
+    p = torch.empty(c, r, kpad, dtype=dt, device=dev)
+    _lib.bgemm_nt(lr[0], lr[1], p, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=c, a_bs=r * kpad, b_bs=r * kpad,
+                  o_bs=r * kpad, s_i=kpad)
+    del lr
+    tiles = []
+    for t in range((C + 127) // 128):
+        tiles.append(make_tile(out.data_ptr() + t * 128 * es, bias=out_bias_pk.data_ptr() + t * 128 * es,
+                               gate=g.data_ptr() + t * 128 * es, gate_ld=C, resid=z.data_ptr() + t * 128 * es,
+                               inner=M, s_i=C, ncols=min(128, C - t * 128)))
+    _lib.fused_linear(p, wout_pk, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
+                      ln=ln2)
+    return out
+
+
+# ------------------------------------------------------------------ outer product mean ----
+def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, bo, budget, eps=1e-3):
+    """out = z + (Wo vec(sum_s a[s,i,:] (x) b[s,j,:]) + bo) / (sum_s mask[s,i] mask[s,j] + eps),
+    a, b the masked 32-channel projections of LN(m).  m is [s, r, C] rows, mask [s, r]."""
+    dt, dev = m.dtype, m.device
+    es = es_of(dt)
+    spad = round_up(s, vec_of(dt))
+    ab = alloc((2, r * 32, spad), dt, dev, zero=spad != s)
+    tile = make_tile(ab, bias=bab_pk, ncols=64, inner=s, s_o=32 * spad, s_i=1, s_h=r * 32 * spad, s_d=spad,
+                     rowmask=mask, m_so=1, m_si=r)
+    # logical row (i, s') reads m[s', i]
+    _lib.fused_linear(m, wab_pk, [tile], M=s * r, K=C, a_inner=s, a_so=C, a_si=r * C, ln=ln)
+    mt = torch.zeros(r, spad, dtype=dt, device=dev)
+    mt[:, :s] = mask.t()
+    nrm = torch.empty(r, r, dtype=torch.float32, device=dev)
+    _lib.bgemm_nt(mt, mt, nrm, M=r, N=r, K=spad, lda=spad, ldb=spad, out_f32=True)
+    ci = max(1, min(r, budget // (r * 1024 * es)))
+    O = torch.empty(ci * r, 1024, dtype=dt, device=dev)
+    for i0 in range(0, r, ci):
+        n = min(ci, r - i0)
+        _lib.bgemm_nt(ab.data_ptr() + i0 * 32 * spad * es, ab[1], O, M=32 * n, N=32 * r, K=spad, lda=spad, ldb=spad,
+                      inner=32, s_o=r * 1024, s_i=32, s_h=1024, s_d=1, dtype=dt)
+        _lib.bgemm_nt(O, wo, out.data_ptr() + i0 * r * Cz * es, M=n * r, N=Cz, K=1024, lda=1024, ldb=1024, bias=bo,
+                      rowdiv=nrm.data_ptr() + i0 * r * 4, div_eps=eps, resid=z.data_ptr() + i0 * r * Cz * es, dtype=dt)
+    return out

@@ -1,0 +1,136 @@
+"""Evoformer block and 48-block stack with the reference's interface
+(fastfold/model/fastnn/evoformer.py:17-332), single GPU (DAP size 1).
+
+Padding contract.  The reference pads the residue axis by ``padding_size = 1`` in the first
+block even at DAP size 1, carries ``[1, s, r+1, c]`` / ``[1, r+1, r+1, c]`` tensors between
+blocks and strips the pad in the last block (evoformer.py:42-62,78-89).  The padded key is
+masked in every attention and every masked projection, and padded rows are discarded, so
+results on the un-padded region do not depend on it.  ``Evoformer.forward`` keeps that
+*interface* (same shapes in and out for first / middle / last blocks) but computes on the
+un-padded region only; ``EvoformerStack`` never materialises the pad at all.
+"""
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .msa import MSACore
+from .ops import Linear, OutProductMean
+from .triangle import PairCore
+
+
+class Evoformer(nn.Module):
+
+    def __init__(self, c_m: int, c_z: int, first_block: bool, last_block: bool, is_multimer: bool = False):
+        super(Evoformer, self).__init__()
+        self.first_block = first_block
+        self.last_block = last_block
+        self.msa = MSACore(c_m, c_z, p_drop=0.15)
+        self.communication = OutProductMean(n_feat=c_m, n_feat_out=c_z, n_feat_proj=32)
+        self.pair = PairCore(d_pair=c_z)
+        self.is_multimer = is_multimer
+
+    # -- un-padded core on [1, s, r, c_m] / [1, r, r, c_z] / [1, s, r] / [1, r, r] ----------
+    def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
+        if self.is_multimer:
+            # multimer order (evoformer.py:70-76): OPM and pair stack first, MSA stack on the old z
+            z_ori = z
+            z_new = self.communication.forward(m, msa_mask, z)
+            self.pair.inplace([z_new], pair_mask)
+            m_new = self.msa.inplace(m, z_ori, msa_mask) if inplace else self.msa.forward(m, z_ori, msa_mask)
+            if inplace:
+                z.copy_(z_new)
+                return m_new, z
+            return m_new, z_new
+        if inplace:
+            m = self.msa.inplace(m, z, msa_mask)
+            self.communication._run(m, msa_mask, z, z)
+            self.pair.inplace([z], pair_mask)
+            return m, z
+        m = self.msa.forward(m, z, msa_mask)
+        z = self.communication.forward(m, msa_mask, z)
+        self.pair.inplace([z], pair_mask)     # z is already a fresh tensor
+        return m, z
+
+    def _enter(self, m, z, r):
+        if self.first_block:
+            return m.unsqueeze(0).contiguous(), z.unsqueeze(0).contiguous()
+        if m.dim() != 4 or z.dim() != 4 or m.shape[2] != r + 1 or z.shape[1] != r + 1:
+            raise RuntimeError("Evoformer: a non-first block expects padded [1, s, r+1, c] / [1, r+1, r+1, c] "
+                               "inputs, got %s / %s" % (tuple(m.shape), tuple(z.shape)))
+        return m[:, :, :r, :].contiguous(), z[:, :r, :r, :].contiguous()
+
+    def _leave(self, m, z):
+        if self.last_block:
+            return m.squeeze(0), z.squeeze(0)
+        return F.pad(m, (0, 0, 0, 1)), F.pad(z, (0, 0, 0, 1, 0, 1))
+
+    def forward(self, m: torch.Tensor, z: torch.Tensor, msa_mask: torch.Tensor, pair_mask: torch.Tensor,
+                chunk_size: Optional[int] = None, _mask_trans: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+        """``chunk_size`` and ``_mask_trans`` are accepted and ignored, as in the reference
+        (evoformer.py:36-37): chunking is the process-global ``set_chunk_size`` and transitions
+        are never masked."""
+        r = pair_mask.size(-1)
+        m, z = self._enter(m, z, r)
+        m, z = self._core(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0), inplace=not self.first_block)
+        return self._leave(m, z)
+
+    def inplace(self, m, z, msa_mask: torch.Tensor, pair_mask: torch.Tensor, chunk_size: Optional[int] = None,
+                _mask_trans: bool = True):
+        """List-passing variant (evoformer.py:93-152): ``m`` and ``z`` are one-element lists whose
+        tensors are updated / rebound."""
+        r = pair_mask.size(-1)
+        if self.first_block:
+            mm, zz = m[0].unsqueeze(0), z[0].unsqueeze(0)
+            if not mm.is_contiguous() or not zz.is_contiguous():
+                mm, zz = mm.contiguous(), zz.contiguous()
+        else:
+            mm, zz = self._enter(m[0], z[0], r)
+        mm, zz = self._core(mm, zz, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0), inplace=True)
+        m[0], z[0] = self._leave(mm, zz)
+        return m, z
+
+
+class EvoformerStack(nn.Module):
+    """Main Evoformer trunk (Algorithm 6): ``no_blocks`` blocks, then ``s = Linear(c_m, c_s)(m[0])``."""
+
+    def __init__(self, c_m: int, c_z: int, c_s: int, no_blocks: int, blocks_per_ckpt: int,
+                 clear_cache_between_blocks: bool = False, is_multimer: bool = False, **kwargs):
+        super(EvoformerStack, self).__init__()
+        self.blocks_per_ckpt = blocks_per_ckpt
+        self.clear_cache_between_blocks = clear_cache_between_blocks
+        self.blocks = nn.ModuleList()
+        for block_id in range(no_blocks):
+            self.blocks.append(Evoformer(c_m=c_m, c_z=c_z, first_block=(block_id == 0),
+                                         last_block=(block_id == no_blocks - 1), is_multimer=is_multimer))
+        self.linear = Linear(c_m, c_s)
+
+    def _run(self, m, z, msa_mask, pair_mask, inplace_first: bool):
+        mm, zz = m.unsqueeze(0), z.unsqueeze(0)
+        mk, pk = msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)
+        for i, b in enumerate(self.blocks):
+            if self.clear_cache_between_blocks:
+                torch.cuda.empty_cache()
+            mm, zz = b._core(mm.contiguous(), zz.contiguous(), mk, pk, inplace=(inplace_first or i > 0))
+        return mm.squeeze(0), zz.squeeze(0)
+
+    def forward(self, m: torch.Tensor, z: torch.Tensor, msa_mask: torch.Tensor, pair_mask: torch.Tensor,
+                chunk_size: int = None, _mask_trans: bool = True
+                ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+        """
+        m [N_seq, N_res, C_m], z [N_res, N_res, C_z], msa_mask [N_seq, N_res], pair_mask [N_res, N_res]
+        -> (m, z, s [N_res, C_s]).  Inputs are left untouched.
+        """
+        m, z = self._run(m, z, msa_mask, pair_mask, inplace_first=False)
+        s = self.linear(m[..., 0, :, :])
+        return m, z, s
+
+    def inplace(self, m, z, msa_mask: torch.Tensor, pair_mask: torch.Tensor, chunk_size: int = None,
+                _mask_trans: bool = True):
+        """``m`` / ``z`` are one-element lists; their tensors are overwritten (evoformer.py:280-332)."""
+        contiguous = m[0].is_contiguous() and z[0].is_contiguous()
+        mm, zz = self._run(m[0], z[0], msa_mask, pair_mask, inplace_first=contiguous)
+        m[0], z[0] = mm, zz
+        s = self.linear(m[0][..., 0, :, :])
+        return m, z, s

@@ -1,0 +1,414 @@
+"""Evoformer building blocks with the reference's class names, constructor signatures,
+parameter names and call signatures (fastfold/model/fastnn/ops.py), each forward being a
+short sequence of HIP kernel launches (see ``_fused.py``) instead of PyTorch ops.
+
+Differences that do not change results: there is no distributed code (DAP size 1: the
+reference's gather/scatter calls are identities) and chunking (``set_chunk_size``) only
+lowers the scratch-memory budget of the launches, since attention logits and transition /
+outer-product intermediates are already streamed.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from fastfold_amd import _lib
+from fastfold_amd.model.fastnn.kernel import LayerNorm
+from . import _fused as F_
+from .initializer import glorot_uniform_af
+from .kernel import layouts
+
+CHUNK_SIZE = None
+DEBUG = False
+
+
+def set_chunk_size(chunk_size):
+    """Process-global chunk knob (reference: ops.py:31-37)."""
+    global CHUNK_SIZE
+    CHUNK_SIZE = chunk_size
+
+
+def get_chunk_size():
+    global CHUNK_SIZE
+    return CHUNK_SIZE
+
+
+def _budget():
+    return F_._WS_BUDGET_DEFAULT if CHUNK_SIZE is None else F_._WS_BUDGET_CHUNKED
+
+
+class _PackMixin:
+    """Caches kernel-ready copies of the parameters, keyed by dtype/device and rebuilt when a
+    source parameter is modified (``_version``) or moved."""
+
+    def _packed(self, key, params, build):
+        cache = self.__dict__.setdefault("_pack_cache", {})
+        ver = tuple((p.data_ptr(), p._version, p.dtype) for p in params)
+        ent = cache.get(key)
+        if ent is None or ent[0] != ver:
+            with torch.no_grad():
+                ent = (ver, build())
+            cache[key] = ent
+        return ent[1]
+
+
+def _no_grad_guard(module, *tensors):
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise NotImplementedError(
+            "%s: the HIP path implements the forward pass only; run it under torch.no_grad()"
+            % type(module).__name__)
+
+
+def _ln_pair(ln, dtype):
+    return (ln.weight.detach().to(dtype).contiguous(), ln.bias.detach().to(dtype).contiguous())
+
+
+def _mask_like(mask, x):
+    return mask.to(dtype=x.dtype).contiguous()
+
+
+class DropoutRowwise(nn.Module):
+
+    def __init__(self, p):
+        super(DropoutRowwise, self).__init__()
+        self.p = p
+        self.dropout = nn.Dropout(p=p)
+
+    def forward(self, x):
+        dropout_mask = torch.ones_like(x[:, 0:1, :, :])
+        dropout_mask = self.dropout(dropout_mask)
+        return dropout_mask * x
+
+
+class DropoutColumnwise(nn.Module):
+
+    def __init__(self, p):
+        super(DropoutColumnwise, self).__init__()
+        self.p = p
+        self.dropout = nn.Dropout(p=p)
+
+    def forward(self, x):
+        dropout_mask = torch.ones_like(x[:, :, 0:1, :])
+        dropout_mask = self.dropout(dropout_mask)
+        return dropout_mask * x
+
+
+class Linear(nn.Linear, _PackMixin):
+    """nn.Linear with the reference's initialisers (ops.py:229-256): 'linear' = Glorot gain 1,
+    'relu' = gain 2, 'zeros' = zero weight; any other string (the reference's call sites pass
+    'zero') keeps nn.Linear's default init.  The forward is an MFMA GEMM launch."""
+
+    def __init__(self, feature_in: int, feature_out: int, initializer: str = 'linear', use_bias: bool = True,
+                 bias_init: float = 0.):
+        super(Linear, self).__init__(feature_in, feature_out, bias=use_bias)
+        self.use_bias = use_bias
+        if initializer == 'linear':
+            glorot_uniform_af(self.weight, gain=1.0)
+        elif initializer == 'relu':
+            glorot_uniform_af(self.weight, gain=2.0)
+        elif initializer == 'zeros':
+            nn.init.zeros_(self.weight)
+        if self.use_bias:
+            with torch.no_grad():
+                self.bias.fill_(bias_init)
+
+    def _pk(self, dtype, device):
+        params = [self.weight] + ([self.bias] if self.use_bias else [])
+        return self._packed(("lin", dtype, device), params, lambda: (
+            F_.pack_rows([self.weight], dtype, device),
+            F_.pack_vec([self.bias], dtype, device) if self.use_bias else None))
+
+    def forward(self, input):
+        F_.check_cuda(input)
+        _no_grad_guard(self, input)
+        w, b = self._pk(input.dtype, input.device)
+        x2 = input.reshape(-1, self.in_features).contiguous()
+        out = F_.linear(x2, w, b, self.out_features)
+        return out.view(*input.shape[:-1], self.out_features)
+
+
+class Transition(nn.Module, _PackMixin):
+    """src + W2 relu(W1 LN(src) + b1) + b2 (ops.py:71-82); no mask, as in the reference."""
+
+    def __init__(self, d, n=4):
+        super(Transition, self).__init__()
+        self.norm = LayerNorm(d)
+        self.linear1 = Linear(d, n * d, initializer='relu')
+        self.linear2 = Linear(n * d, d, initializer='zeros')
+
+    def _run(self, src, out):
+        F_.check_cuda(src)
+        _no_grad_guard(self, src)
+        dt, dev = src.dtype, src.device
+        d = src.shape[-1]
+        hidden = self.linear1.out_features
+        if not F_.fits_fused(d, dt) or hidden % 128 != 0:
+            raise RuntimeError("Transition: unsupported width %d" % d)
+        w1, b1, w2, b2 = self._packed(("tr", dt, dev), [self.linear1.weight, self.linear1.bias,
+                                                       self.linear2.weight, self.linear2.bias], lambda: (
+            F_.pack_rows([self.linear1.weight], dt, dev), F_.pack_vec([self.linear1.bias], dt, dev),
+            self.linear2.weight.detach().to(dt).contiguous(), self.linear2.bias.detach().to(dt).contiguous()))
+        x = src.view(-1, d)
+        F_.transition(x, out.view(-1, d), ln=_ln_pair(self.norm, dt), w1_pk=w1, b1_pk=b1, w2=w2, b2=b2,
+                      hidden=hidden, budget=_budget())
+        return out
+
+    def forward(self, src):
+        src = src.contiguous()
+        return self._run(src, torch.empty_like(src))
+
+
+class ChunkTransition(Transition):
+    """Same computation (ops.py:85-123); rows are always streamed in bounded chunks."""
+
+    def inplace(self, src):
+        src[0] = src[0].contiguous()
+        self._run(src[0], src[0])
+        return src
+
+
+class OutProductMean(nn.Module, _PackMixin):
+    """Outer-product-mean update of the pair representation (ops.py:126-227)."""
+
+    def __init__(self, n_feat=64, n_feat_out=128, n_feat_proj=32):
+        super(OutProductMean, self).__init__()
+        self.layernormM = LayerNorm(n_feat)
+        self.linear_a = Linear(n_feat, n_feat_proj)
+        self.linear_b = Linear(n_feat, n_feat_proj)
+        self.o_linear = Linear(n_feat_proj * n_feat_proj, n_feat_out, initializer='zero', use_bias=True)
+        self.n_feat_proj = n_feat_proj
+
+    def _run(self, M, M_mask, Z_raw, out):
+        F_.check_cuda(M, M_mask, Z_raw)
+        _no_grad_guard(self, M, Z_raw)
+        if self.n_feat_proj != 32:
+            raise RuntimeError("OutProductMean: the kernel path needs n_feat_proj == 32")
+        dt, dev = M.dtype, M.device
+        if M.dim() == 4:
+            if M.shape[0] != 1:
+                raise RuntimeError("OutProductMean: leading batch dimension must be 1")
+            M, M_mask = M[0], M_mask[0]
+        s, r, C = M.shape
+        Cz = Z_raw.shape[-1]
+        if not F_.fits_fused(C, dt):
+            raise RuntimeError("OutProductMean: unsupported MSA width %d" % C)
+        wab, bab, wo, bo = self._packed(("opm", dt, dev), [self.linear_a.weight, self.linear_a.bias,
+                                                          self.linear_b.weight, self.linear_b.bias,
+                                                          self.o_linear.weight, self.o_linear.bias], lambda: (
+            F_.pack_rows([self.linear_a.weight, self.linear_b.weight], dt, dev),
+            F_.pack_vec([self.linear_a.bias, self.linear_b.bias], dt, dev),
+            self.o_linear.weight.detach().to(dt).contiguous(), self.o_linear.bias.detach().to(dt).contiguous()))
+        F_.outer_product_mean(M.contiguous(), _mask_like(M_mask, M), Z_raw, out, s=s, r=r, C=C, Cz=Cz,
+                              ln=_ln_pair(self.layernormM, dt), wab_pk=wab, bab_pk=bab, wo=wo, bo=bo,
+                              budget=_budget())
+        return out
+
+    def forward(self, M, M_mask, Z_raw):
+        Z_raw = Z_raw.contiguous()
+        return self._run(M, M_mask, Z_raw, torch.empty_like(Z_raw))
+
+    def inplace(self, M, M_mask, Z_raw):
+        Z_raw[0] = Z_raw[0].contiguous()
+        self._run(M, M_mask, Z_raw[0], Z_raw[0])
+        return Z_raw
+
+
+class SelfAttention(nn.Module, _PackMixin):
+    """Multi-head self attention over [batch_size1, batch_size2, len, dim] tensors with gating
+    (ops.py:259-363).  Head dimension ``c`` must be 32 and ``n_head`` a multiple of 4."""
+
+    def __init__(self, qkv_dim, c, n_head, out_dim, gating=True, last_bias_fuse=False):
+        super(SelfAttention, self).__init__()
+        self.qkv_dim = qkv_dim
+        self.c = c
+        self.n_head = n_head
+        self.out_dim = out_dim
+        self.gating = gating
+        self.last_bias_fuse = last_bias_fuse
+        self.scaling = self.c**(-0.5)
+        self.to_qkv = Linear(qkv_dim, 3 * n_head * c, initializer='linear', use_bias=False)
+        if gating:
+            self.gating_bias = nn.parameter.Parameter(data=torch.ones((n_head * c,)))
+            self.gating_linear = Linear(qkv_dim, n_head * c, initializer='zero', use_bias=False)
+        self.o_linear = Linear(n_head * c, out_dim, initializer='zero', use_bias=(not last_bias_fuse))
+
+    def _check(self, dtype):
+        if self.c != 32 or not self.gating:
+            raise RuntimeError("SelfAttention: the kernel path needs head dim 32 and gating=True")
+        if not F_.fits_fused(self.qkv_dim, dtype):
+            raise RuntimeError("SelfAttention: unsupported input width %d" % self.qkv_dim)
+
+    def packed(self, dtype, device, extra_rows=None, extra_params=()):
+        """(w_pk [q;k;v;gate(;extra)], gating_bias_pk, wo_pk)."""
+        key = ("att", dtype, device, extra_rows is not None)
+        params = [self.to_qkv.weight, self.gating_linear.weight, self.gating_bias, self.o_linear.weight]
+        params += list(extra_params)
+
+        def build():
+            mats = [self.to_qkv.weight, self.gating_linear.weight]
+            w = F_.pack_rows(mats, dtype, device)
+            if extra_rows is not None:
+                w = torch.cat([w, F_.pack_rows([extra_rows()], dtype, device)], 0).contiguous()
+            return (w, F_.pack_vec([self.gating_bias], dtype, device), F_.pack_rows([self.o_linear.weight], dtype, device))
+        return self._packed(key, params, build)
+
+    def forward(self, in_data, mask, nonbatched_bias=None):
+        """
+        :param in_data: [batch_size1, batch_size2, len_qkv, qkv_dim]
+        :param mask: None or [batch_size1, batch_size2, len_kv]
+        :param nonbatched_bias: None, or (b [batch_size1, len_q, len_kv, n_head], work), or
+                                (bias [batch_size1, n_head, len_q, len_kv], -1)
+        """
+        F_.check_cuda(in_data, mask)
+        _no_grad_guard(self, in_data)
+        dt, dev = in_data.dtype, in_data.device
+        self._check(dt)
+        if in_data.dim() != 4 or in_data.shape[0] != 1:
+            raise RuntimeError("SelfAttention: expected [1, B2, N, C] input, got %s" % (tuple(in_data.shape),))
+        _, B2, N, C = in_data.shape
+        x = in_data.contiguous()
+        bias_t = None
+        if nonbatched_bias is not None:
+            b = nonbatched_bias[0]
+            if not (isinstance(nonbatched_bias[-1], int) and nonbatched_bias[-1] == -1):
+                b = b.permute(0, 3, 1, 2)                       # 'b q k h -> b h q k'
+            bias_t = layouts.tile_bias(b[0].float() * _lib.LOG2E).to(dt)
+        if mask is None:
+            mk, sb, sn = None, 0, 1
+        else:
+            mk, sb, sn = _mask_like(mask, x)[0], N, 1
+        w_pk, gb_pk, wo_pk = self.packed(dt, dev)
+        ob = None
+        if self.o_linear.use_bias:
+            ob = self._packed(("ob", dt, dev), [self.o_linear.bias], lambda: F_.pack_vec([self.o_linear.bias], dt, dev))
+        out = torch.empty(1, B2, N, self.out_dim, dtype=dt, device=dev)
+        F_.attention(x, out, None, B2=B2, N=N, C=C, H=self.n_head, a_map=(B2 * N, 0, C), ln=None, w_pk=w_pk,
+                     gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob, c_out=self.out_dim, mask=mk, mask_sb=sb,
+                     mask_sn=sn, bias_t=bias_t)
+        return out
+
+
+def permute_final_dims(tensor, inds):
+    zero_index = -1 * len(inds)
+    first_inds = list(range(len(tensor.shape[:zero_index])))
+    return tensor.permute(first_inds + [zero_index + i for i in inds])
+
+
+class _TriangleMultiplication(nn.Module, _PackMixin):
+    _incoming = False
+
+    def __init__(self, d_pair, p_drop, c=128):
+        super().__init__()
+        self.d_pair = d_pair
+        self.c = c
+        self.layernorm1 = LayerNorm(d_pair)
+        self.left_right_projection = Linear(d_pair, 2 * c)
+        self.left_right_gate = Linear(d_pair, 2 * c, initializer='zeros', bias_init=1.)
+        self.output_gate = Linear(d_pair, d_pair, initializer='zeros', bias_init=1.)
+        self.layernorm2 = LayerNorm(c)
+        self.output_projection = Linear(d_pair, d_pair, initializer='zeros', use_bias=False)
+        self.output_bias = nn.parameter.Parameter(data=torch.zeros((d_pair,)), requires_grad=True)
+        self.p_drop = p_drop
+
+    def _run(self, Z_raw, Z_mask, out):
+        F_.check_cuda(Z_raw, Z_mask)
+        _no_grad_guard(self, Z_raw)
+        dt, dev = Z_raw.dtype, Z_raw.device
+        if Z_raw.dim() != 4 or Z_raw.shape[0] != 1 or Z_raw.shape[1] != Z_raw.shape[2]:
+            raise RuntimeError("TriangleMultiplication: expected [1, r, r, C], got %s" % (tuple(Z_raw.shape),))
+        r, C = Z_raw.shape[1], Z_raw.shape[3]
+        if not F_.fits_fused(C, dt) or not F_.fits_fused(self.c, dt):
+            raise RuntimeError("TriangleMultiplication: unsupported widths %d / %d" % (C, self.c))
+        ps = [self.left_right_projection.weight, self.left_right_projection.bias, self.left_right_gate.weight,
+              self.left_right_gate.bias, self.output_gate.weight, self.output_gate.bias,
+              self.output_projection.weight, self.output_bias]
+
+        def build():
+            w, b, n_glu = F_.pack_trimul(self.left_right_projection.weight, self.left_right_projection.bias,
+                                         self.left_right_gate.weight, self.left_right_gate.bias,
+                                         self.output_gate.weight, self.output_gate.bias, self.c, dt, dev)
+            return (w, b, n_glu, F_.pack_rows([self.output_projection.weight], dt, dev),
+                    F_.pack_vec([self.output_bias], dt, dev))
+        w, b, n_glu, wout, bout = self._packed(("tm", dt, dev), ps, build)
+        F_.triangle_multiplication(Z_raw, out, r=r, C=C, c=self.c, incoming=self._incoming,
+                                   ln1=_ln_pair(self.layernorm1, dt), w_pk=w, b_pk=b, n_glu=n_glu,
+                                   ln2=_ln_pair(self.layernorm2, dt), wout_pk=wout, out_bias_pk=bout,
+                                   mask=_mask_like(Z_mask, Z_raw))
+        return out
+
+    def forward(self, Z_raw, Z_mask):
+        Z_raw = Z_raw.contiguous()
+        return self._run(Z_raw, Z_mask, torch.empty_like(Z_raw))
+
+    def inplace(self, Z_raw, Z_mask):
+        Z_raw[0] = Z_raw[0].contiguous()
+        self._run(Z_raw[0], Z_mask, Z_raw[0])
+        return Z_raw
+
+
+class AsyncChunkTriangleMultiplicationOutgoing(_TriangleMultiplication):
+    """Algorithm 11 (ops.py:372-498): p[i,j] = sum_k a[i,k] b[j,k]."""
+    _incoming = False
+
+
+class AsyncChunkTriangleMultiplicationIncoming(_TriangleMultiplication):
+    """Algorithm 12 (ops.py:501-630): p[i,j] = sum_k a[k,i] b[k,j]."""
+    _incoming = True
+
+
+class _TriangleAttention(nn.Module, _PackMixin):
+    _ending = False
+
+    def __init__(self, d_pair, p_drop, c=32, n_head=4):
+        super().__init__()
+        self.d_pair = d_pair
+        self.c = c
+        self.n_head = n_head
+        self.p_drop = p_drop
+        self.layernorm1 = LayerNorm(d_pair)
+        self.linear_b = Linear(d_pair, n_head, initializer='linear', use_bias=False)
+        self.attention = SelfAttention(qkv_dim=d_pair, c=c, n_head=n_head, out_dim=d_pair, gating=True,
+                                       last_bias_fuse=True)
+        self.out_bias = nn.parameter.Parameter(data=torch.zeros((d_pair,)), requires_grad=True)
+
+    def _run(self, Z_raw, Z_mask, out):
+        F_.check_cuda(Z_raw, Z_mask)
+        _no_grad_guard(self, Z_raw)
+        dt, dev = Z_raw.dtype, Z_raw.device
+        self.attention._check(dt)
+        if Z_raw.dim() != 4 or Z_raw.shape[0] != 1 or Z_raw.shape[1] != Z_raw.shape[2]:
+            raise RuntimeError("TriangleAttention: expected [1, r, r, C], got %s" % (tuple(Z_raw.shape),))
+        r, C = Z_raw.shape[1], Z_raw.shape[3]
+        w_pk, gb_pk, wo_pk = self.attention.packed(dt, dev, extra_rows=lambda: self.linear_b.weight,
+                                                  extra_params=[self.linear_b.weight])
+        ob = self._packed(("ob", dt, dev), [self.out_bias], lambda: F_.pack_vec([self.out_bias], dt, dev))
+        NT = (r + 31) // 32
+        bias_t = F_.alloc((self.n_head, NT, NT, 1024), dt, dev, zero=(r % 32) != 0)
+        mask = _mask_like(Z_mask, Z_raw)[0]
+        if self._ending:    # logical row (j, i) reads z[i, j]; keys run along i
+            a_map, sb, sn = (r, C, r * C), 1, r
+        else:
+            a_map, sb, sn = (r * r, 0, C), r, 1
+        F_.attention(Z_raw, out, Z_raw, B2=r, N=r, C=C, H=self.n_head, a_map=a_map,
+                     ln=_ln_pair(self.layernorm1, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
+                     c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=bias_t, bias_in_launch=True)
+        return out
+
+    def forward(self, Z_raw, Z_mask):
+        Z_raw = Z_raw.contiguous()
+        return self._run(Z_raw, Z_mask, torch.empty_like(Z_raw))
+
+    def inplace(self, Z_raw, Z_mask):
+        Z_raw[0] = Z_raw[0].contiguous()
+        self._run(Z_raw[0], Z_mask, Z_raw[0])
+        return Z_raw
+
+
+class ChunkTriangleAttentionStartingNode(_TriangleAttention):
+    """Algorithm 13 (ops.py:633-748): attention along each row of the pair representation."""
+    _ending = False
+
+
+class ChunkTriangleAttentionEndingNode(_TriangleAttention):
+    """Algorithm 14 (ops.py:869-989): attention along each column."""
+    _ending = True

@@ -1,0 +1,43 @@
+"""Pair stack of the Evoformer block (fastfold/model/fastnn/triangle.py:216-271)."""
+import torch
+import torch.nn as nn
+
+from .ops import (AsyncChunkTriangleMultiplicationIncoming, AsyncChunkTriangleMultiplicationOutgoing,
+                  ChunkTransition, ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode)
+
+
+class PairCore(nn.Module):
+
+    def __init__(self, d_pair, p_drop=0.25):
+        super(PairCore, self).__init__()
+        self.d_pair = d_pair
+        self.n_head = 4
+        self.hidden_c = int(d_pair / self.n_head)
+
+        self.TriangleMultiplicationOutgoing = AsyncChunkTriangleMultiplicationOutgoing(d_pair, p_drop=p_drop, c=d_pair)
+        self.TriangleMultiplicationIncoming = AsyncChunkTriangleMultiplicationIncoming(d_pair, p_drop=p_drop, c=d_pair)
+        self.TriangleAttentionStartingNode = ChunkTriangleAttentionStartingNode(d_pair, p_drop=p_drop,
+                                                                                c=self.hidden_c, n_head=self.n_head)
+        self.TriangleAttentionEndingNode = ChunkTriangleAttentionEndingNode(d_pair, p_drop=p_drop,
+                                                                            c=self.hidden_c, n_head=self.n_head)
+        self.PairTransition = ChunkTransition(d=d_pair)
+
+    def forward(self, pair, pair_mask):
+        """pair [1, r, r, d_pair], pair_mask [1, r, r] -> new pair (input untouched)."""
+        pair = pair.contiguous()
+        out = torch.empty_like(pair)
+        self.TriangleMultiplicationOutgoing._run(pair, pair_mask, out)
+        self._rest(out, pair_mask)
+        return out
+
+    def _rest(self, z, pair_mask):
+        self.TriangleMultiplicationIncoming._run(z, pair_mask, z)
+        self.TriangleAttentionStartingNode._run(z, pair_mask, z)
+        self.TriangleAttentionEndingNode._run(z, pair_mask, z)
+        self.PairTransition._run(z, z)
+
+    def inplace(self, pair, pair_mask):
+        pair[0] = pair[0].contiguous()
+        self.TriangleMultiplicationOutgoing._run(pair[0], pair_mask, pair[0])
+        self._rest(pair[0], pair_mask)
+        return pair

@@ -1,0 +1,126 @@
+"""Drop-in seam: swap a model's plain-PyTorch Evoformer (nn layout) for the HIP-backed
+``fastfold_amd.model.fastnn.EvoformerStack`` and re-pack its weights.
+
+Same entry points as the reference's ``fastfold/utils/inject_fastnn.py`` for the Evoformer
+path (``inject_fastnn``, ``inject_evoformer``, ``copy_*``; reference lines 24-152,321-338,
+418-423).  The weight re-layout is:
+  q/k/v weights            -> rows of ``to_qkv.weight`` in that order
+  linear_g.{weight,bias}   -> ``gating_linear.weight`` / ``gating_bias``
+  linear_o.weight          -> ``o_linear.weight``; its bias -> ``out_bias`` (row / triangle
+                              attention) or ``o_linear.bias`` (column attention)
+  linear_z.weight (row)    -> ``linear_b_weights``
+  tri-mul a_p|b_p, a_g|b_g -> ``left_right_projection`` / ``left_right_gate`` (left rows first),
+  linear_g -> ``output_gate``, linear_z.{weight,bias} -> ``output_projection.weight`` / ``output_bias``
+  OPM linear_1/2/out       -> ``linear_a`` / ``linear_b`` / ``o_linear``
+Extra-MSA, template and embedder stages are outside this build and are left as they are.
+"""
+import torch
+
+from fastfold_amd.model.fastnn import EvoformerStack
+
+
+def copy_layernorm(model_fast, model_ori):
+    model_fast.weight.copy_(model_ori.weight)
+    model_fast.bias.copy_(model_ori.bias)
+
+
+def copy_linear(model_fast, model_ori):
+    model_fast.weight.copy_(model_ori.weight)
+    if model_fast.use_bias:
+        model_fast.bias.copy_(model_ori.bias)
+
+
+def copy_qkv_linear(model_fast, ori_q, ori_k, ori_v):
+    model_fast.weight.copy_(torch.cat((ori_q.weight, ori_k.weight, ori_v.weight), dim=0))
+
+
+def copy_attention(model_fast, model_ori):
+    copy_qkv_linear(model_fast.to_qkv, model_ori.linear_q, model_ori.linear_k, model_ori.linear_v)
+    copy_linear(model_fast.gating_linear, model_ori.linear_g)
+    copy_linear(model_fast.o_linear, model_ori.linear_o)
+    if getattr(model_fast, "gating_bias", None) is not None and model_ori.linear_g is not None:
+        model_fast.gating_bias.copy_(model_ori.linear_g.bias)
+
+
+def copy_left_right(model_fast, ori_left, ori_right):
+    model_fast.weight.copy_(torch.cat((ori_left.weight, ori_right.weight), dim=0))
+    model_fast.bias.copy_(torch.cat((ori_left.bias, ori_right.bias), dim=0))
+
+
+def copy_transition(model_fast, model_ori):
+    copy_layernorm(model_fast.norm, model_ori.layer_norm)
+    copy_linear(model_fast.linear1, model_ori.linear_1)
+    copy_linear(model_fast.linear2, model_ori.linear_2)
+
+
+def copy_triangle(model_fast, model_ori):
+    copy_layernorm(model_fast.layernorm1, model_ori.layer_norm_in)
+    copy_layernorm(model_fast.layernorm2, model_ori.layer_norm_out)
+    copy_linear(model_fast.output_projection, model_ori.linear_z)
+    model_fast.output_bias.copy_(model_ori.linear_z.bias)
+    copy_linear(model_fast.output_gate, model_ori.linear_g)
+    copy_left_right(model_fast.left_right_projection, model_ori.linear_a_p, model_ori.linear_b_p)
+    copy_left_right(model_fast.left_right_gate, model_ori.linear_a_g, model_ori.linear_b_g)
+
+
+def copy_triangle_att(model_fast, model_ori):
+    copy_layernorm(model_fast.layernorm1, model_ori.layer_norm)
+    copy_linear(model_fast.linear_b, model_ori.linear)
+    copy_attention(model_fast.attention, model_ori.mha)
+    model_fast.out_bias.copy_(model_ori.mha.linear_o.bias)
+
+
+def copy_evoformer_para(block_fast, block_ori):
+    row_f, row_o = block_fast.msa.MSARowAttentionWithPairBias, block_ori.msa_att_row
+    copy_layernorm(row_f.layernormM, row_o.layer_norm_m)
+    copy_layernorm(row_f.layernormZ, row_o.layer_norm_z)
+    copy_attention(row_f.attention, row_o.mha)
+    row_f.linear_b_weights.copy_(row_o.linear_z.weight)
+    row_f.out_bias.copy_(row_o.mha.linear_o.bias)
+
+    col_f, col_o = block_fast.msa.MSAColumnAttention, block_ori.msa_att_col._msa_att
+    copy_layernorm(col_f.layernormM, col_o.layer_norm_m)
+    copy_attention(col_f.attention, col_o.mha)
+
+    copy_transition(block_fast.msa.MSATransition, block_ori.core.msa_transition)
+
+    opm_f, opm_o = block_fast.communication, block_ori.core.outer_product_mean
+    copy_layernorm(opm_f.layernormM, opm_o.layer_norm)
+    copy_linear(opm_f.linear_a, opm_o.linear_1)
+    copy_linear(opm_f.linear_b, opm_o.linear_2)
+    copy_linear(opm_f.o_linear, opm_o.linear_out)
+
+    copy_triangle(block_fast.pair.TriangleMultiplicationOutgoing, block_ori.core.tri_mul_out)
+    copy_triangle(block_fast.pair.TriangleMultiplicationIncoming, block_ori.core.tri_mul_in)
+    copy_triangle_att(block_fast.pair.TriangleAttentionStartingNode, block_ori.core.tri_att_start)
+    copy_triangle_att(block_fast.pair.TriangleAttentionEndingNode, block_ori.core.tri_att_end)
+    copy_transition(block_fast.pair.PairTransition, block_ori.core.pair_transition)
+
+
+def inject_evoformer(model):
+    with torch.no_grad():
+        target_module = model.evoformer
+        ref_param = next(target_module.parameters())
+        fast_module = EvoformerStack(
+            c_m=target_module.blocks[0].msa_att_row.c_in,
+            c_z=target_module.blocks[0].msa_att_row.c_z,
+            c_s=target_module.linear.out_features,
+            no_blocks=len(target_module.blocks),
+            blocks_per_ckpt=target_module.blocks_per_ckpt,
+            clear_cache_between_blocks=target_module.clear_cache_between_blocks,
+            is_multimer=target_module.blocks[0].is_multimer,
+        ).to(device=ref_param.device, dtype=ref_param.dtype)
+        for target_block, fast_block in zip(target_module.blocks, fast_module.blocks):
+            copy_evoformer_para(fast_block, target_block)
+            if target_block.training is False:
+                fast_block.eval()
+        copy_linear(fast_module.linear, target_module.linear)
+        if target_module.training is False:
+            fast_module.eval()
+        model.evoformer = fast_module
+
+
+def inject_fastnn(model):
+    """Replaces ``model.evoformer``; returns the model (reference: inject_fastnn.py:418-423)."""
+    inject_evoformer(model)
+    return model
