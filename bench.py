@@ -1,0 +1,205 @@
+"""Evoformer hot-path benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4|cfg3] [--no-cpu]
+
+One step = one forward pass of the 48-block Evoformer stack (bf16, N_seq=128, random-init
+weights ~N(0, 0.02^2), inputs ~N(0,1)) with inputs and weights resident in HBM.  The metric is
+the Evoformer-block latency (ms per block = step time / 48).  The same JSON line carries
+  roofline      the dominant kernel (flash attention core with bias: triangle + MSA-row attention),
+                algorithmic FLOPs / HIP-event time of its launches inside the timed region,
+  cpu_baseline  the CPU oracle (plain-PyTorch restatement of the reference's nn Evoformer block)
+                timed on this box's host cores on a bounded sample,
+and the op micro-benchmarks of BASELINE config 2 (fused softmax, LayerNorm: HBM GB/s).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0
+
+WORKLOADS = {
+    "cfg3": dict(n_seq=128, n_res=256, tail=0.0, name="configs[2]: 48-block stack bf16 N_seq=128 N_res=256"),
+    "cfg4": dict(n_seq=128, n_res=1024, tail=0.05,
+                 name="configs[3]: 48-block stack bf16 N_seq=128 N_res=1024, last 5% of residues masked"),
+}
+
+
+def block_gflop(s, r, c_m=256, c_z=128, hm=8, hz=4, d=32, c_opm=32, c_mul=128, n=4):
+    """Algorithmic GFLOP of one block: 2*M*N*K per contraction, un-padded shapes."""
+    row_proj = 2 * s * r * c_m * (3 * hm * d) + 2 * (2 * s * r * c_m * hm * d) + 2 * r * r * c_z * hm
+    row_core = 4 * s * hm * r * r * d
+    col_proj = row_proj - 2 * r * r * c_z * hm
+    col_core = 4 * r * hm * s * s * d
+    mtrans = 4 * s * r * c_m * (n * c_m)
+    opm = 4 * s * r * c_m * c_opm + 2 * r * r * s * c_opm ** 2 + 2 * r * r * c_opm ** 2 * c_z
+    trimul = (2 * (2 * r * r * c_z * 2 * c_mul) + 2 * r * r * c_z * c_z + 2 * r * r * c_mul * c_z) + 2 * c_mul * r ** 3
+    triatt = (2 * r * r * c_z * (3 * hz * d) + 2 * (2 * r * r * c_z * hz * d) + 2 * r * r * c_z * hz) + 4 * r * hz * r * r * d
+    ptrans = 4 * r * r * c_z * (n * c_z)
+    return (row_proj + row_core + col_proj + col_core + mtrans + opm + 2 * trimul + 2 * triatt + ptrans) / 1e9
+
+
+def build_stack(no_blocks, dev, dtype, seed=0):
+    import torch
+    from fastfold_amd.model.fastnn import EvoformerStack
+    from fastfold_amd.synthetic import synth_nn_state
+    from fastfold_amd.utils.inject_fastnn import convert_nn_state_dict
+    st = EvoformerStack(c_m=256, c_z=128, c_s=384, no_blocks=no_blocks, blocks_per_ckpt=1)
+    st.load_state_dict(convert_nn_state_dict(synth_nn_state(seed=seed, no_blocks=no_blocks, std=0.02)), strict=True)
+    return st.to(device=dev, dtype=dtype).eval()
+
+
+def micro_ops(dev):
+    """BASELINE config 2: fused softmax [1,128,8,256,256] bf16 with pair bias and 10% masked keys;
+    LayerNorm over [65536,128] and [32768,256] bf16.  Rotating buffers (> 512 MB) so HBM is touched."""
+    import torch
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel.softmax import _softmax_forward
+    res = {}
+    g = torch.Generator().manual_seed(0)
+    nb = 4
+    xs = [torch.randn(1, 128, 8, 256, 256, device=dev, dtype=torch.bfloat16) for _ in range(nb)]
+    outs = [torch.empty_like(xs[0]) for _ in range(nb)]
+    bias = torch.randn(1, 1, 8, 256, 256, device=dev, dtype=torch.bfloat16)
+    mask = (torch.rand(1, 128, 256, generator=g) > 0.1).to(dev, torch.bfloat16)
+    mask[..., 0] = 1
+
+    def run(name, fn, n, nbytes):
+        for i in range(3):
+            fn(i)
+        torch.cuda.synchronize()
+        rec = _lib.time_kernel(name)
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        _lib.time_kernel(name, enable=False)
+        us = sorted(a.elapsed_time(b) * 1e3 for a, b, _ in rec)
+        med = us[len(us) // 2]
+        return {"us": round(med, 2), "GB/s": round(nbytes / med / 1e3, 1), "frac_of_8TBps": round(nbytes / med / 1e3 / PEAK_HBM_GBPS, 3)}
+
+    res["softmax_bf16_1x128x8x256x256"] = run(
+        "ffk_softmax_fwd", lambda i: _softmax_forward(xs[i % nb], mask, bias, out=outs[i % nb]), 20, 2 * xs[0].numel() * 2)
+    del xs, outs
+    for rows, cols in ((65536, 128), (32768, 256)):
+        nb = 20
+        xs = [torch.randn(rows, cols, device=dev, dtype=torch.bfloat16) for _ in range(nb)]
+        os_ = [torch.empty_like(xs[0]) for _ in range(nb)]
+        gam = (1 + 0.1 * torch.randn(cols, generator=g)).to(dev, torch.bfloat16)
+        bet = (0.1 * torch.randn(cols, generator=g)).to(dev, torch.bfloat16)
+
+        def f(i):
+            _lib.call("ffk_layernorm_fwd", os_[i % nb].data_ptr(), None, None, xs[i % nb].data_ptr(), gam.data_ptr(),
+                      bet.data_ptr(), rows, cols, 1e-5, _lib.FFK_BF16, _lib.stream_ptr())
+        res["layernorm_bf16_%dx%d" % (rows, cols)] = run("ffk_layernorm_fwd", f, 60, 2 * rows * cols * 2)
+        del xs, os_
+    return res
+
+
+def cpu_baseline(threads):
+    """The CPU oracle timed on the host cores: one fp32 block at N_seq=128, N_res=256."""
+    import numpy as np
+    import torch
+    from fastfold_amd.synthetic import synth_inputs, synth_nn_state
+    from oracle.evoformer_ref import EvoformerStack as OracleStack
+    torch.set_num_threads(threads)
+    st = OracleStack(no_blocks=1).eval()
+    st.load_state_dict({k: torch.from_numpy(v) for k, v in synth_nn_state(seed=0, no_blocks=1).items()})
+    m, z, mm, pm = (torch.from_numpy(t) for t in synth_inputs(0, 128, 256))
+    ts = []
+    with torch.no_grad():
+        st(m, z, mm, pm, _mask_trans=False)
+        t_end = time.time() + 20.0
+        while len(ts) < 5 and (time.time() < t_end or len(ts) < 2):
+            t0 = time.time()
+            st(m, z, mm, pm, _mask_trans=False)
+            ts.append((time.time() - t0) * 1e3)
+    return {"value": round(float(np.median(ts)), 2), "unit": "ms/block", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "1 Evoformer block, fp32, N_seq=128 N_res=256 (configs[2] shape), oracle/evoformer_ref.py, "
+                      "median of %d runs after 1 warm-up" % len(ts)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--blocks", type=int, default=48)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-micro", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the Evoformer on ONE GPU (DAP size 1, no collectives); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from fastfold_amd import _lib
+    from fastfold_amd.synthetic import synth_inputs
+    _lib.load()
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS[args.workload]
+    s, r = wl["n_seq"], wl["n_res"]
+    stack = build_stack(args.blocks, dev, torch.bfloat16)
+    m, z, mm, pm = (torch.from_numpy(t).to(dev, torch.bfloat16) for t in synth_inputs(0, s, r, mask_tail_frac=wl["tail"]))
+
+    def step():
+        with torch.no_grad():
+            return stack(m, z, mm, pm, chunk_size=None)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    rec = _lib.time_kernel("ffk_attention_fwd")
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    _lib.time_kernel("ffk_attention_fwd", enable=False)
+    assert all(bool(torch.isfinite(t.float()).all()) for t in out), "non-finite output"
+
+    # dominant kernel: attention core launches that carry a bias (MSA row + triangle start/end)
+    flops, ms, n = 0.0, 0.0, 0
+    for e0, e1, a in rec:
+        if a[4] is None:       # bias_t == NULL: column attention (other kernel instantiation)
+            continue
+        B2, H, Nq, Nk = a[7], a[8], a[9], a[10]
+        flops += 4.0 * B2 * H * Nq * Nk * 32
+        ms += e0.elapsed_time(e1)
+        n += 1
+    ach = flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+    roofline = {"bound": "mfma", "kernel": "attention_kernel<bf16, bias> (ffk_attention_fwd)",
+                "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "launches": n, "avg_launch_ms": round(ms / max(n, 1), 4),
+                "flops_per_launch_avg": round(flops / max(n, 1) / 1e9, 2)}
+
+    line = {
+        "metric": "Evoformer-block latency, bf16, N_seq=%d, N_res=%d (stack of %d blocks)" % (s, r, args.blocks),
+        "value": round(ms_per_step / args.blocks, 4), "unit": "ms/block",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": wl["name"], "blocks": args.blocks, "n_seq": s, "n_res": r,
+                   "block_gflop": round(block_gflop(s, r), 1),
+                   "stack_tflops": round(block_gflop(s, r) * args.blocks / ms_per_step, 1)},
+        "roofline": roofline,
+    }
+    del stack, out
+    torch.cuda.empty_cache()
+    if not args.no_micro:
+        line["ops"] = micro_ops(dev)
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

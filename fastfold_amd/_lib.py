@@ -89,10 +89,32 @@ def check_device(*tensors):
             raise RuntimeError("fastfold_amd: tensor must be contiguous")
 
 
+# Optional per-launch timing: name -> list of (start_event, end_event, args).  Events are recorded
+# on torch's current stream, which is the stream every kernel is launched on.
+_TIMED = {}
+
+
+def time_kernel(name, enable=True):
+    """Starts (or stops) recording HIP events around every launch of entry point ``name``;
+    returns the list the records go to: tuples (start_event, end_event, args)."""
+    if enable:
+        _TIMED[name] = []
+        return _TIMED[name]
+    return _TIMED.pop(name, None)
+
+
 def call(name: str, *args):
     """Calls an entry point; raises RuntimeError with the library's message on failure."""
     lib = load()
-    rc = getattr(lib, name)(*args)
+    rec = _TIMED.get(name)
+    if rec is not None:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        rc = getattr(lib, name)(*args)
+        e1.record()
+        rec.append((e0, e1, args))
+    else:
+        rc = getattr(lib, name)(*args)
     if rc != 0:
         msg = lib.ffk_last_error_string()
         raise RuntimeError("%s failed (status %d): %s" % (name, rc, msg.decode() if msg else "?"))

@@ -124,3 +124,72 @@ def inject_fastnn(model):
     """Replaces ``model.evoformer``; returns the model (reference: inject_fastnn.py:418-423)."""
     inject_evoformer(model)
     return model
+
+
+def convert_nn_state_dict(sd):
+    """nn-layout state dict of an Evoformer stack (``blocks.N.msa_att_row...``) -> fastnn-layout
+    state dict (``blocks.N.msa.MSARowAttentionWithPairBias...``) by the same re-layout as
+    ``copy_evoformer_para``; values may be tensors or numpy arrays."""
+    import numpy as np
+
+    def T(x):
+        return x if isinstance(x, torch.Tensor) else torch.from_numpy(np.ascontiguousarray(x))
+
+    out = {}
+    blocks = sorted({int(k.split(".")[1]) for k in sd if k.startswith("blocks.")})
+
+    def ln(dst, src):
+        out[dst + ".weight"], out[dst + ".bias"] = T(sd[src + ".weight"]), T(sd[src + ".bias"])
+
+    def lin(dst, src, bias=True):
+        out[dst + ".weight"] = T(sd[src + ".weight"])
+        if bias:
+            out[dst + ".bias"] = T(sd[src + ".bias"])
+
+    def att(dst, src, fused_out_bias):
+        out[dst + ".attention.to_qkv.weight"] = torch.cat([T(sd[src + ".linear_%s.weight" % n]) for n in "qkv"], 0)
+        out[dst + ".attention.gating_linear.weight"] = T(sd[src + ".linear_g.weight"])
+        out[dst + ".attention.gating_bias"] = T(sd[src + ".linear_g.bias"])
+        out[dst + ".attention.o_linear.weight"] = T(sd[src + ".linear_o.weight"])
+        if fused_out_bias:
+            out[dst + ".out_bias"] = T(sd[src + ".linear_o.bias"])
+        else:
+            out[dst + ".attention.o_linear.bias"] = T(sd[src + ".linear_o.bias"])
+
+    for i in blocks:
+        s, d = "blocks.%d." % i, "blocks.%d." % i
+        row = d + "msa.MSARowAttentionWithPairBias"
+        ln(row + ".layernormM", s + "msa_att_row.layer_norm_m")
+        ln(row + ".layernormZ", s + "msa_att_row.layer_norm_z")
+        out[row + ".linear_b_weights"] = T(sd[s + "msa_att_row.linear_z.weight"])
+        att(row, s + "msa_att_row.mha", True)
+        col = d + "msa.MSAColumnAttention"
+        ln(col + ".layernormM", s + "msa_att_col._msa_att.layer_norm_m")
+        att(col, s + "msa_att_col._msa_att.mha", False)
+        for dst, src in ((d + "msa.MSATransition", s + "core.msa_transition"),
+                         (d + "pair.PairTransition", s + "core.pair_transition")):
+            ln(dst + ".norm", src + ".layer_norm")
+            lin(dst + ".linear1", src + ".linear_1")
+            lin(dst + ".linear2", src + ".linear_2")
+        ln(d + "communication.layernormM", s + "core.outer_product_mean.layer_norm")
+        lin(d + "communication.linear_a", s + "core.outer_product_mean.linear_1")
+        lin(d + "communication.linear_b", s + "core.outer_product_mean.linear_2")
+        lin(d + "communication.o_linear", s + "core.outer_product_mean.linear_out")
+        for dst, src in ((d + "pair.TriangleMultiplicationOutgoing", s + "core.tri_mul_out"),
+                         (d + "pair.TriangleMultiplicationIncoming", s + "core.tri_mul_in")):
+            ln(dst + ".layernorm1", src + ".layer_norm_in")
+            ln(dst + ".layernorm2", src + ".layer_norm_out")
+            for nm, a, b in ((".left_right_projection", ".linear_a_p", ".linear_b_p"),
+                             (".left_right_gate", ".linear_a_g", ".linear_b_g")):
+                out[dst + nm + ".weight"] = torch.cat([T(sd[src + a + ".weight"]), T(sd[src + b + ".weight"])], 0)
+                out[dst + nm + ".bias"] = torch.cat([T(sd[src + a + ".bias"]), T(sd[src + b + ".bias"])], 0)
+            lin(dst + ".output_gate", src + ".linear_g")
+            out[dst + ".output_projection.weight"] = T(sd[src + ".linear_z.weight"])
+            out[dst + ".output_bias"] = T(sd[src + ".linear_z.bias"])
+        for dst, src in ((d + "pair.TriangleAttentionStartingNode", s + "core.tri_att_start"),
+                         (d + "pair.TriangleAttentionEndingNode", s + "core.tri_att_end")):
+            ln(dst + ".layernorm1", src + ".layer_norm")
+            out[dst + ".linear_b.weight"] = T(sd[src + ".linear.weight"])
+            att(dst, src + ".mha", True)
+    lin("linear", "linear")
+    return out
