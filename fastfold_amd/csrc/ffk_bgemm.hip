@@ -12,10 +12,6 @@ namespace {
 constexpr int BT = 128;
 constexpr int THREADS = 256;
 
-__device__ __forceinline__ long row_off(long m, int inner, long so, long si) {
-    return (m / inner) * so + (m % inner) * si;
-}
-
 template <typename T, typename OT>
 __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc d) {
     typedef Mma<T> MM;
@@ -54,22 +50,26 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
             if (ma >= M) ma = M - 1;
             long nb = n0 + r;
             if (nb >= N) nb = N - 1;
-            if (k < K) {
-                ra[i] = ld16(A + ma * d.lda + k);
-                rb[i] = ld16(B + nb * d.ldb + k);
-            } else {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) ra[i].e[e] = rb[i].e[e] = DT<T>::from_f(0.0f);
-            }
+            // branch-free: clamp the K offset to the last full vector; the K tail is zeroed when the
+            // registers are committed to LDS (touching them here would serialise the loads)
+            const int kk = k < K ? k : K - VEC;
+            ra[i] = ld16(A + ma * d.lda + kk);
+            rb[i] = ld16(B + nb * d.ldb + kk);
         }
     };
-    auto commit = [&](int slot) {
+    auto commit = [&](int slot, int kc) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int v = tid + THREADS * i;
             const int r = v / (BK / VEC), c = v % (BK / VEC);
-            *reinterpret_cast<Vec16<T>*>(sA + slot * SLOT + r * P + c * 16) = ra[i];
-            *reinterpret_cast<Vec16<T>*>(sB + slot * SLOT + r * P + c * 16) = rb[i];
+            const bool tail = kc * BK + c * VEC >= K;
+            Vec16<T> xa = ra[i], xb = rb[i];
+            if (tail) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) xa.e[e] = xb.e[e] = DT<T>::from_f(0.0f);
+            }
+            *reinterpret_cast<Vec16<T>*>(sA + slot * SLOT + r * P + c * 16) = xa;
+            *reinterpret_cast<Vec16<T>*>(sB + slot * SLOT + r * P + c * 16) = xb;
         }
     };
 
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     fetch(0);
     for (int kc = 0; kc < kchunks; ++kc) {
         const int slot = kc & 1;
-        commit(slot);
+        commit(slot, kc);
         __syncthreads();
         if (kc + 1 < kchunks) fetch(kc + 1);
         const unsigned char* pa = sA + slot * SLOT + (wm * 64 + l32) * P + half * (MM::KLANE * ES);
@@ -106,14 +106,38 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     }
     __syncthreads();
 
+    // row offsets of this tile, one integer division per row (kept in LDS for phase 2)
+    __shared__ long s_off[BT];
+    if (tid < BT) {
+        long m = m0 + tid;
+        if (m >= M) m = M - 1;
+        const unsigned hi = (unsigned)m / (unsigned)d.inner;
+        const unsigned lo = (unsigned)m - hi * (unsigned)d.inner;
+        s_off[tid] = (long)hi * d.s_o + (long)lo * d.s_i;
+    }
+
     // ---- phase 1: registers -> staged tile [m][n] (values after bias / act / scale / rowdiv) ----
+    // (bias / rowdiv are fetched with clamped indices, i.e. without per-lane branches, so the loads
+    // are issued back to back; out-of-range values are computed but never stored)
     const T* bias = (const T*)d.bias;
+    float bv[2][4][4];
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                long n = n0 + wn * 64 + ni * 32 + 8 * g + 4 * half + e;
+                n = n < N ? n : N - 1;
+                bv[ni][g][e] = bias ? DT<T>::to_f(bias[n]) : 0.0f;
+            }
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
         const int mr = wm * 64 + mi * 32 + l32;
-        const long m = m0 + mr;
+        long m = m0 + mr;
+        m = m < M ? m : M - 1;
         float rdiv = 1.0f;
-        if (d.rowdiv && m < M) rdiv = 1.0f / (d.rowdiv[(long)bz * M + m] + d.div_eps);
+        if (d.rowdiv) rdiv = 1.0f / (d.rowdiv[(long)bz * M + m] + d.div_eps);
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni) {
 #pragma unroll
@@ -122,8 +146,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
                 OT* dst = reinterpret_cast<OT*>(sC + mr * CP + nc * OES);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float x = acc[ni][mi][4 * g + e];
-                    if (bias && n0 + nc + e < N) x += DT<T>::to_f(bias[n0 + nc + e]);
+                    float x = acc[ni][mi][4 * g + e] + bv[ni][g][e];
                     if (d.act == FFK_ACT_RELU) x = fmaxf(x, 0.0f);
                     else if (d.act == FFK_ACT_SIGMOID) x = sigmoid_f(x);
                     dst[e] = DT<OT>::from_f(x * d.scale * rdiv);
@@ -138,25 +161,48 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     const OT* resid = d.resid ? (const OT*)d.resid + (long)bz * d.o_bs : nullptr;
     if (d.s_d == 1) {
         constexpr int VPR = BT / OVEC;
-        for (int v = tid; v < BT * VPR; v += THREADS) {
-            const int r = v / VPR, c = (v % VPR) * OVEC;
-            const long m = m0 + r, n = n0 + c;
-            if (m >= M || n >= N) continue;
-            Vec16<OT> x = *reinterpret_cast<const Vec16<OT>*>(sC + r * CP + c * OES);
-            const long o = row_off(m, d.inner, d.s_o, d.s_i) + (n >> 5) * d.s_h + (n & 31);
-            if (n + OVEC <= N && ((reinterpret_cast<uintptr_t>(out + o) & 15u) == 0)) {
-                if (resid) {
-                    Vec16<OT> rv = ld16(resid + o);
+        constexpr int N_IT = BT * VPR / THREADS;
+        // vector path when every row pitch / base keeps 16-byte alignment and N is a multiple of the vector
+        const bool vec_ok = (N % OVEC) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 &&
+                            (!resid || (reinterpret_cast<uintptr_t>(resid) & 15u) == 0) && (d.s_o % OVEC) == 0 &&
+                            (d.s_i % OVEC) == 0 && (d.s_h % OVEC) == 0;
+        if (vec_ok) {
+            const long n_last = N - OVEC;
+#pragma unroll 1
+            for (int i0 = 0; i0 < N_IT; i0 += 4) {
+                Vec16<OT> x[4], rv[4];
+                long o[4];
 #pragma unroll
-                    for (int e = 0; e < OVEC; ++e) x.e[e] = DT<OT>::from_f(DT<OT>::to_f(x.e[e]) + DT<OT>::to_f(rv.e[e]));
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int r = v / VPR, c = (v % VPR) * OVEC;
+                    long n = n0 + c;
+                    n = n <= n_last ? n : n_last;
+                    o[j] = s_off[r] + (n >> 5) * d.s_h + (n & 31);
+                    x[j] = *reinterpret_cast<const Vec16<OT>*>(sC + r * CP + c * OES);
+                    if (resid) rv[j] = ld16(resid + o[j]);
                 }
-                st16(out + o, x);
-            } else {
-                for (int e = 0; e < OVEC && n + e < N; ++e) {
-                    float y = DT<OT>::to_f(x.e[e]);
-                    if (resid) y += DT<OT>::to_f(resid[o + e]);
-                    out[o + e] = DT<OT>::from_f(y);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int r = v / VPR, c = (v % VPR) * OVEC;
+                    if (resid) {
+#pragma unroll
+                        for (int e = 0; e < OVEC; ++e)
+                            x[j].e[e] = DT<OT>::from_f(DT<OT>::to_f(x[j].e[e]) + DT<OT>::to_f(rv[j].e[e]));
+                    }
+                    if (m0 + r < M && n0 + c < N) st16(out + o[j], x[j]);
                 }
+            }
+        } else {
+            for (int v = tid; v < BT * BT; v += THREADS) {
+                const int r = v / BT, c = v % BT;
+                const long m = m0 + r, n = n0 + c;
+                if (m >= M || n >= N) continue;
+                const long o = s_off[r] + (n >> 5) * d.s_h + (n & 31);
+                float y = DT<OT>::to_f(*reinterpret_cast<const OT*>(sC + r * CP + c * OES));
+                if (resid) y += DT<OT>::to_f(resid[o]);
+                out[o] = DT<OT>::from_f(y);
             }
         }
     } else {
@@ -164,7 +210,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
             const int c = v / BT, r = v % BT;           // consecutive threads -> consecutive rows m
             const long m = m0 + r, n = n0 + c;
             if (m >= M || n >= N) continue;
-            const long o = row_off(m, d.inner, d.s_o, d.s_i) + (n >> 5) * d.s_h + (n & 31) * d.s_d;
+            const long o = s_off[r] + (n >> 5) * d.s_h + (n & 31) * d.s_d;
             float y = DT<OT>::to_f(*reinterpret_cast<const OT*>(sC + r * CP + c * OES));
             if (resid) y += DT<OT>::to_f(resid[o]);
             out[o] = DT<OT>::from_f(y);

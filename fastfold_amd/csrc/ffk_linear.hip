@@ -19,7 +19,7 @@ constexpr int THREADS = 256;
 
 template <typename T> struct LinCfg;
 template <> struct LinCfg<bf16_t> {
-    static constexpr int BM = 128, WM = 4, WN = 1, BK = 64;
+    static constexpr int BM = 64, WM = 2, WN = 2, BK = 32;
 };
 template <> struct LinCfg<float> {
     static constexpr int BM = 64, WM = 2, WN = 2, BK = 32;
@@ -29,12 +29,30 @@ struct LinArgs {
     ffk_linear_desc d;
 };
 
-__device__ __forceinline__ long row_off(long m, int inner, long so, long si) {
-    return (m / inner) * so + (m % inner) * si;
+// Row tables.  Splitting a logical row into (hi, lo) = divmod(m, inner) needs an integer
+// division; it is done once per row of the slab (by one thread per row) and kept in LDS, so
+// the streaming loops below contain no divisions.
+struct RowTab {
+    long off[128];   // hi * s_o + lo * s_i
+    int hi[128];
+    int lo[128];
+};
+
+__device__ __forceinline__ void fill_rowtab(RowTab& tab, int tid, int BM, long m0, int M, int inner, long so, long si) {
+    if (tid < BM) {
+        long m = m0 + tid;
+        if (m >= M) m = M - 1;
+        const unsigned mu = (unsigned)m;
+        const unsigned hi = mu / (unsigned)inner;
+        const unsigned lo = mu - hi * (unsigned)inner;
+        tab.hi[tid] = (int)hi;
+        tab.lo[tid] = (int)lo;
+        tab.off[tid] = (long)hi * so + (long)lo * si;
+    }
 }
 
 template <typename T>
-__global__ __launch_bounds__(THREADS) void fused_linear_kernel(const LinArgs args) {
+__global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs args) {
     typedef LinCfg<T> Cfg;
     typedef Mma<T> MM;
     constexpr int BM = Cfg::BM, WM = Cfg::WM, WN = Cfg::WN, BK = Cfg::BK;
@@ -47,11 +65,13 @@ __global__ __launch_bounds__(THREADS) void fused_linear_kernel(const LinArgs arg
     constexpr int CPT = BM * ES + 16;              // staged C pitch, [channel][row]
     static_assert(BM * CP <= 2 * WBUF, "C staging must fit in the weight ring");
     static_assert(NT * CPT <= 2 * WBUF + 4096, "transposed C staging");
+    (void)WM;
 
     const ffk_linear_desc& d = args.d;
     const int K = d.K, M = d.M;
     const int AP = K * ES + 16;                    // A slab row pitch (bytes)
     extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ RowTab tab;
     unsigned char* sA = smem;
     unsigned char* sW = smem + (size_t)BM * AP;
     unsigned char* sC = sW;                        // aliases the ring between tiles
@@ -69,7 +89,7 @@ __global__ __launch_bounds__(THREADS) void fused_linear_kernel(const LinArgs arg
     const int kchunks = K / BK;
     const int total_chunks = d.n_tiles * kchunks;
     auto w_fetch = [&](int chunk) {
-        const int nt = chunk / kchunks, kc = chunk % kchunks;
+        const int nt = chunk / kchunks, kc = chunk - nt * kchunks;
 #pragma unroll
         for (int i = 0; i < WVEC; ++i) {
             const int v = tid + THREADS * i;
@@ -87,45 +107,66 @@ __global__ __launch_bounds__(THREADS) void fused_linear_kernel(const LinArgs arg
     };
     w_fetch(0);
 
-    // ---- stage the A slab ----
+    // ---- stage the A slab (loads issued four at a time so their latencies overlap) ----
+    fill_rowtab(tab, tid, BM, m0, M, d.a_inner, d.a_so, d.a_si);
+    __syncthreads();
+    // Loads below are unconditional (row / column indices are clamped to valid ones instead of
+    // being predicated) so that a batch of four is in flight at once; only the LDS stores are guarded.
+    // Rows beyond M hold a copy of row M-1: their results are never stored.
     if (!d.a_chanmajor) {
-        const int vpr = K / VEC;
-        for (int v = tid; v < BM * vpr; v += THREADS) {
-            const int r = v / vpr, c = v % vpr;
-            const long m = m0 + r;
-            Vec16<T> x;
-            if (m < M) {
-                x = ld16(A + row_off(m, d.a_inner, d.a_so, d.a_si) + c * VEC);
-            } else {
+        const int vpr = K / VEC;                   // 16-byte vectors per row
+        int cs = 3;
+        while ((1 << cs) < vpr) ++cs;              // lanes per row rounded up to a power of two
+        const int c_raw = tid & ((1 << cs) - 1);
+        const int c = c_raw < vpr ? c_raw : vpr - 1;
+        const int r_first = tid >> cs, rstep = THREADS >> cs;
+        const int n_it = BM / rstep;
+        for (int i0 = 0; i0 < n_it; i0 += 4) {
+            Vec16<T> buf[4];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) x.e[e] = DT<T>::from_f(0.0f);
+            for (int j = 0; j < 4; ++j) {
+                int r = r_first + (i0 + j) * rstep;
+                r = r < BM ? r : BM - 1;
+                buf[j] = ld16(A + tab.off[r] + c * VEC);
             }
-            *reinterpret_cast<Vec16<T>*>(sA + r * AP + c * 16) = x;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = r_first + (i0 + j) * rstep;
+                if (r < BM && c_raw < vpr) *reinterpret_cast<Vec16<T>*>(sA + r * AP + c * 16) = buf[j];
+            }
         }
     } else {
         // element (m, k) at a + k * a_cs + rowoff(m): read runs of VEC rows, scatter into [row][k]
-        const int rpv = BM / VEC;
-        for (int v = tid; v < K * rpv; v += THREADS) {
-            const int k = v / rpv, r0 = (v % rpv) * VEC;
-            const long m = m0 + r0;
-            T vals[VEC];
-            const long o0 = m < M ? row_off(m, d.a_inner, d.a_so, d.a_si) : 0;
-            const long mlast = m + VEC - 1;
-            bool contig = mlast < M && d.a_si == 1 && (m % d.a_inner) + VEC - 1 < d.a_inner;
-            const T* src = A + (long)k * d.a_cs + o0;
-            contig = contig && ((reinterpret_cast<uintptr_t>(src) & 15u) == 0);
-            if (contig) {
-                Vec16<T> x = ld16(src);
+        constexpr int RPV = BM / VEC;              // VEC-row runs per channel (a power of two)
+        const int n_it = K * RPV / THREADS;        // K % 32 == 0  =>  a multiple of 4 (bf16) / 2... see below
+        // uniform fast-path test: every run of VEC rows of this slab is contiguous and 16-byte aligned
+        const bool fast = d.a_si == 1 && m0 + BM <= M && (d.a_inner % VEC) == 0 && (d.a_so % VEC) == 0 &&
+                          (d.a_cs % VEC) == 0 && (m0 % VEC) == 0;
+        if (fast) {
+            for (int i0 = 0; i0 < n_it; i0 += 4) {
+                Vec16<T> buf[4];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) vals[e] = x.e[e];
-            } else {
+                for (int j = 0; j < 4; ++j) {
+                    int v = tid + THREADS * (i0 + j);
+                    v = v < K * RPV ? v : K * RPV - 1;
+                    const int k = v / RPV, r0 = (v % RPV) * VEC;
+                    buf[j] = ld16(A + (long)k * d.a_cs + tab.off[r0]);
+                }
 #pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    vals[e] = (m + e < M) ? A[(long)k * d.a_cs + row_off(m + e, d.a_inner, d.a_so, d.a_si)]
-                                          : DT<T>::from_f(0.0f);
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int k = v / RPV, r0 = (v % RPV) * VEC;
+                    if (v < K * RPV) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) *reinterpret_cast<T*>(sA + (r0 + e) * AP + k * ES) = buf[j].e[e];
+                    }
+                }
             }
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) *reinterpret_cast<T*>(sA + (r0 + e) * AP + k * ES) = vals[e];
+        } else {
+            for (int v = tid; v < K * BM; v += THREADS) {
+                const int k = v / BM, r = v % BM;
+                *reinterpret_cast<T*>(sA + r * AP + k * ES) = A[(long)k * d.a_cs + tab.off[r]];
+            }
         }
     }
     __syncthreads();
@@ -202,9 +243,13 @@ __global__ __launch_bounds__(THREADS) void fused_linear_kernel(const LinArgs arg
         const int prow = wm * 32 + l32;                         // row within the slab
         const long mrow = m0 + prow;
         float rmask = 1.0f;
-        if (t.rowmask && mrow < M)
-            rmask = DT<T>::to_f(((const T*)t.rowmask)[row_off(mrow, t.inner, t.m_so, t.m_si)]);
+        if (t.rowmask && mrow < M) {
+            const unsigned hi = (unsigned)mrow / (unsigned)t.inner;
+            const unsigned lo = (unsigned)mrow - hi * (unsigned)t.inner;
+            rmask = DT<T>::to_f(((const T*)t.rowmask)[(long)hi * t.m_so + (long)lo * t.m_si]);
+        }
         __syncthreads();                                        // all waves done with the ring
+        fill_rowtab(tab, tid, BM, m0, M, t.inner, t.s_o, t.s_i);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             if (t.glu && (ct & 1)) continue;
@@ -243,63 +288,91 @@ __global__ __launch_bounds__(THREADS) void fused_linear_kernel(const LinArgs arg
         const int ncols = t.ncols;
         if (mode_c) {
             constexpr int VPR = NT / VEC;
-            for (int v = tid; v < BM * VPR; v += THREADS) {
-                const int r = v / VPR, c = (v % VPR) * VEC;
-                const long m = m0 + r;
-                if (m >= M || c >= ncols) continue;
-                Vec16<T> x = *reinterpret_cast<const Vec16<T>*>(sC + r * CP + c * ES);
-                long o;
-                if (t.kind == FFK_TILE_QK) {
-                    const long b2 = m / t.inner;
-                    const int n = (int)(m % t.inner);
-                    o = b2 * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 + qk_tile_off(n & 31, c & 31);
-                } else {
-                    o = row_off(m, t.inner, t.s_o, t.s_i) + (long)(c >> 5) * t.s_h + (c & 31);
-                }
-                if (t.gate) {
-                    Vec16<T> gv = ld16((const T*)t.gate + m * t.gate_ld + c);
+            constexpr int N_IT = BM * VPR / THREADS;             // = 8
+            const bool qk = t.kind == FFK_TILE_QK;
+            const T* gate = (const T*)t.gate;
+            const T* resid = (const T*)t.resid;
+            const int c_last = ncols >= VEC ? ((ncols - VEC) / VEC) * VEC : 0;   // last full vector column
+#pragma unroll 1
+            for (int i0 = 0; i0 < N_IT; i0 += 4) {
+                Vec16<T> x[4], gv[4], rv[4];
+                long o[4];
+                // issue every load of the batch first (clamped, branch-free), then combine and store
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) x.e[e] = DT<T>::from_f(DT<T>::to_f(x.e[e]) * DT<T>::to_f(gv.e[e]));
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int r = v / VPR;
+                    int c = (v % VPR) * VEC;
+                    c = c + VEC <= ncols ? c : c_last;
+                    if (qk) {
+                        const int n = tab.lo[r];
+                        o[j] = (long)tab.hi[r] * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 +
+                               qk_tile_off(n & 31, c & 31);
+                    } else {
+                        o[j] = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
+                    }
+                    x[j] = *reinterpret_cast<const Vec16<T>*>(sC + r * CP + c * ES);
+                    long mr = m0 + r;
+                    mr = mr < M ? mr : M - 1;
+                    if (gate) gv[j] = ld16(gate + mr * t.gate_ld + c);
+                    if (resid) rv[j] = ld16(resid + o[j]);
                 }
-                if (c + VEC <= ncols) {
-                    if (t.resid) {
-                        Vec16<T> rv = ld16((const T*)t.resid + o);
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) x.e[e] = DT<T>::from_f(DT<T>::to_f(x.e[e]) + DT<T>::to_f(rv.e[e]));
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int r = v / VPR, c = (v % VPR) * VEC;
+                    if (gate) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) * DT<T>::to_f(gv[j].e[e]));
                     }
-                    st16(out + o, x);
-                } else {
-                    for (int e = 0; e < VEC && c + e < ncols; ++e) {
-                        float y = DT<T>::to_f(x.e[e]);
-                        if (t.resid) y += DT<T>::to_f(((const T*)t.resid)[o + e]);
-                        out[o + e] = DT<T>::from_f(y);
+                    if (resid) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) + DT<T>::to_f(rv[j].e[e]));
                     }
+                    if (m0 + r < M && c + VEC <= ncols) st16(out + o[j], x[j]);
+                }
+            }
+            if (ncols % VEC != 0) {
+                // ragged tail (fewer than VEC channels left): element-wise, rare
+                const int c0 = (ncols / VEC) * VEC, nrem = ncols - c0;
+                for (int v = tid; v < BM * nrem; v += THREADS) {
+                    const int r = v / nrem, c = c0 + v % nrem;
+                    if (m0 + r >= M) continue;
+                    float y = DT<T>::to_f(*reinterpret_cast<const T*>(sC + r * CP + c * ES));
+                    long oo;
+                    if (qk) {
+                        const int n = tab.lo[r];
+                        oo = (long)tab.hi[r] * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 + qk_tile_off(n & 31, c & 31);
+                    } else {
+                        oo = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
+                    }
+                    if (gate) y = DT<T>::to_f(DT<T>::from_f(y * DT<T>::to_f(gate[(m0 + r) * t.gate_ld + c])));
+                    if (resid) y += DT<T>::to_f(resid[oo]);
+                    out[oo] = DT<T>::from_f(y);
                 }
             }
         } else {
             constexpr int QPR = BM / 4;                         // 4-row runs per channel
             for (int v = tid; v < ncols * QPR; v += THREADS) {
                 const int c = v / QPR, r = (v % QPR) * 4;
-                const long m = m0 + r;
-                if (m >= M) continue;
+                if (m0 + r >= M) continue;
                 const T* src = reinterpret_cast<const T*>(sC + c * CPT + r * ES);
                 long o[4];
                 bool ok[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const long me = m + e;
-                    ok[e] = me < M;
-                    const long mm = ok[e] ? me : m;
-                    const long hi = mm / t.inner;
-                    const int lo = (int)(mm % t.inner);
+                    ok[e] = m0 + r + e < M;
+                    const int hi = tab.hi[r + e], lo = tab.lo[r + e];
                     if (t.kind == FFK_TILE_V) {
-                        o[e] = hi * t.s_o + (long)(c >> 5) * t.s_h + (long)(lo >> 5) * 1024 + acc_tile_off(lo & 31, c & 31);
+                        o[e] = (long)hi * t.s_o + (long)(c >> 5) * t.s_h + (long)(lo >> 5) * 1024 + acc_tile_off(lo & 31, c & 31);
                     } else if (t.kind == FFK_TILE_BIAS) {
                         // logical row = (query hi, key lo); channel = head
-                        o[e] = (long)c * t.s_h + (hi >> 5) * t.s_o + (long)(lo >> 5) * 1024 +
-                               acc_tile_off(lo & 31, (int)(hi & 31));
+                        o[e] = (long)c * t.s_h + (long)(hi >> 5) * t.s_o + (long)(lo >> 5) * 1024 +
+                               acc_tile_off(lo & 31, hi & 31);
                     } else {
-                        o[e] = hi * t.s_o + lo * t.s_i + (long)(c >> 5) * t.s_h + (long)(c & 31) * t.s_d;
+                        o[e] = tab.off[r + e] + (long)(c >> 5) * t.s_h + (long)(c & 31) * t.s_d;
                     }
                 }
                 const bool run = ok[3] && o[1] == o[0] + 1 && o[2] == o[0] + 2 && o[3] == o[0] + 3 &&
@@ -350,7 +423,7 @@ int launch_linear(const ffk_linear_desc& d, hipStream_t st) {
 extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
     FFK_REQUIRE(d, FFK_ERR_NULL, "ffk_fused_linear: null descriptor");
     FFK_REQUIRE(d->a && d->w, FFK_ERR_NULL, "ffk_fused_linear: null operand");
-    const int bk = d->dtype == FFK_F32 ? 32 : 64;
+    const int bk = 32;
     FFK_REQUIRE(d->M > 0 && d->K >= bk && d->K <= 256 && d->K % bk == 0, FFK_ERR_SHAPE,
                 "ffk_fused_linear: need M > 0 and K <= 256, a multiple of %d; got M=%d K=%d", bk, d->M, d->K);
     FFK_REQUIRE(d->n_tiles >= 1 && d->n_tiles <= FFK_MAX_TILES, FFK_ERR_SHAPE,

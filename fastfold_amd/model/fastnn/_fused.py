@@ -58,8 +58,7 @@ def check_cuda(*ts):
 
 
 def fits_fused(K, dtype):
-    bk = 32 if dtype == torch.float32 else 64
-    return K <= 256 and K % bk == 0
+    return K <= 256 and K % 32 == 0
 
 
 # ------------------------------------------------------------------------- linear ----
