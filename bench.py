@@ -171,7 +171,7 @@ def main():
     for e0, e1, a in rec:
         if a[4] is None:       # bias_t == NULL: column attention (other kernel instantiation)
             continue
-        B2, H, Nq, Nk = a[7], a[8], a[9], a[10]
+        B2, H, Nq, Nk = a[8], a[9], a[10], a[11]
         flops += 4.0 * B2 * H * Nq * Nk * 32
         ms += e0.elapsed_time(e1)
         n += 1

@@ -209,8 +209,8 @@ class BgemmDesc(ctypes.Structure):
 
 
 SIGNATURES["ffk_bgemm_nt"] = [ctypes.POINTER(BgemmDesc), _P]
-SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _I, _P]
-SIGNATURES["ffk_key_bias"] = [_P, _P, _L, _L, _L, _L, _I, _P]
+SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _I, _P]
+SIGNATURES["ffk_key_bias"] = [_P, _P, _P, _L, _L, _L, _L, _I, _P]
 
 
 def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, inner=None, s_o=0, s_i=None,
@@ -230,11 +230,12 @@ def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, i
     call("ffk_bgemm_nt", ctypes.byref(d), stream_ptr())
 
 
-def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, gate, *, B2, H, Nq, Nk):
-    call("ffk_attention_fwd", ptr(out), ptr(q_t), ptr(k_t), ptr(v_t), ptr(bias_t), ptr(keybias), ptr(gate),
+def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H, Nq, Nk):
+    call("ffk_attention_fwd", ptr(out), ptr(q_t), ptr(k_t), ptr(v_t), ptr(bias_t), ptr(keybias), ptr(tileflags),
+         ptr(gate),
          B2, H, Nq, Nk, dtype_tag(q_t.dtype), stream_ptr())
 
 
-def key_bias(keybias, mask, *, B, N, mask_sb=0, mask_sn=1):
-    call("ffk_key_bias", ptr(keybias), ptr(mask), B, N, mask_sb, mask_sn,
+def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):
+    call("ffk_key_bias", ptr(keybias), ptr(tileflags), ptr(mask), B, N, mask_sb, mask_sn,
          dtype_tag(mask.dtype) if mask is not None else FFK_F32, stream_ptr())

@@ -142,7 +142,8 @@ __host__ __device__ __forceinline__ int qk_tile_off(int n32, int d) { return (d 
 //  accumulator-order tile: element (row, col) of a 32x32 tile whose column is the lane's
 //  (l & 31) and whose rows are spread over (l >> 5, register) as in the MFMA accumulator:
 //  lane = ((row & 7) >> 2) * 32 + col,  register = 4 * (row >> 3) + (row & 3).
-//  Used for v (row = key, col = head-dim index) and for the bias (row = key, col = query).
+//  Used for v (row = key, col = head-dim index).  The additive bias uses the q/k order with
+//  rows = keys and the 32 queries of the tile in place of the head dim.
 __host__ __device__ __forceinline__ int acc_tile_off(int row, int col) {
     return ((((row & 7) >> 2) * 32 + col) << 4) + 4 * (row >> 3) + (row & 3);
 }

@@ -370,7 +370,7 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
                     } else if (t.kind == FFK_TILE_BIAS) {
                         // logical row = (query hi, key lo); channel = head
                         o[e] = (long)c * t.s_h + (long)(hi >> 5) * t.s_o + (long)(lo >> 5) * 1024 +
-                               acc_tile_off(lo & 31, hi & 31);
+                               qk_tile_off(lo & 31, hi & 31);
                     } else {
                         o[e] = tab.off[r + e] + (long)(c >> 5) * t.s_h + (long)(c & 31) * t.s_d;
                     }

@@ -150,9 +150,10 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     a_inner, a_so, a_si = a_map
     _lib.fused_linear(x, w_pk, tiles, M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln)
     kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
-    _lib.key_bias(kb, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
+    flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
+    _lib.key_bias(kb, flags, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
     o = torch.empty(M, HC, dtype=dt, device=dev)
-    _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, gate, B2=B2, H=H, Nq=N, Nk=N)
+    _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, flags, gate, B2=B2, H=H, Nq=N, Nk=N)
     del q_t, k_t, v_t, gate
     tiles = []
     for t in range((c_out + 127) // 128):

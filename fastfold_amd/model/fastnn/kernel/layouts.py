@@ -63,15 +63,16 @@ def untile_v(t, N):
 
 
 def tile_bias(b, scale=1.0):
-    """[H, Nq, Nk] -> [H, QT, KT, 2, 32, 4, 4]  (key = row, query = column of each tile), times scale."""
+    """[H, Nq, Nk] -> [H, QT, KT, 2, 32, 16]: element (k, q) of a tile at [q%32 // 16, k%32, q%16]
+    (an MFMA operand with rows = keys and the tile's 32 queries as the reduction dim), times scale."""
     H, Nq, Nk = b.shape
     b = _pad_to(_pad_to(b, 1, 32), 2, 32) * scale
     qt, kt = b.shape[1] // 32, b.shape[2] // 32
-    x = b.view(H, qt, 32, kt, 4, 2, 4)                        # [h, qt, q32, kt, a, kg, b]
-    return x.permute(0, 1, 3, 5, 2, 4, 6).contiguous()        # [h, qt, kt, kg, q32, a, b]
+    x = b.view(H, qt, 2, 16, kt, 32)                          # [h, qt, qhi, qlo, kt, k32]
+    return x.permute(0, 1, 4, 2, 5, 3).contiguous()           # [h, qt, kt, qhi, k32, qlo]
 
 
 def untile_bias(t, Nq, Nk):
     H, qt, kt = t.shape[:3]
-    x = t.permute(0, 1, 4, 2, 5, 3, 6)                        # [h, qt, q32, kt, a, kg, b]
+    x = t.permute(0, 1, 3, 5, 2, 4)                           # [h, qt, qhi, qlo, kt, k32]
     return x.reshape(H, qt * 32, kt * 32)[:, :Nq, :Nk]

@@ -212,8 +212,10 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  * ffk_fused_linear tile kinds):
  *   q_t, k_t : [B2][H][ceil(N/32)][1024]   FFK_TILE_QK order
  *   v_t      : [B2][H][ceil(Nk/32)][1024]  FFK_TILE_V  order
- *   bias_t   : [H][ceil(Nq/32)][ceil(Nk/32)][1024]  FFK_TILE_BIAS order, or NULL
+ *   bias_t   : [H][ceil(Nq/32)][ceil(Nk/32)][1024]  FFK_TILE_BIAS order (keys x queries as an
+ *              MFMA operand: element (k, q) at (q%32/16)*512 + (k%32)*16 + q%16), or NULL
  *   keybias  : [B2][ceil(Nk/32)*32] fp32
+ *   tileflags: [B2][ceil(Nk/32)] int32 per 32-key tile: 0 all keys valid, 1 mixed, 2 all masked
  *   gate     : [B2*Nq, H*32] row-major multiplicative gate (already sigmoid-ed), or NULL
  *   out      : [B2*Nq, H*32] row-major
  * Replaces: the matmul / fused_softmax / matmul (+ bias_sigmod_ele) chain of
@@ -221,15 +223,16 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  * fused_attention_core (kernel/attention_core.py:17-52, kernel/triton/attention_core.py:12-190).
  */
 int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t,
-                      const void* bias_t, const float* keybias, const void* gate,
+                      const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
                       int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int dtype, void* stream);
 
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the
- * given dtype, or NULL (all keys valid).  Replaces the `1e9 * (mask - 1)` key-padding term of
+ * given dtype, or NULL (all keys valid).  tileflags[b, k/32] classifies each 32-key tile (see
+ * ffk_attention_fwd).  Replaces the `1e9 * (mask - 1)` key-padding term of
  * the reference (ops.py:313, kernel/triton/softmax.py:17-19). */
-int ffk_key_bias(float* keybias, const void* mask, int64_t B, int64_t N, int64_t mask_sb,
-                 int64_t mask_sn, int dtype, void* stream);
+int ffk_key_bias(float* keybias, int32_t* tileflags, const void* mask, int64_t B, int64_t N,
+                 int64_t mask_sb, int64_t mask_sn, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -40,10 +40,14 @@ def test_attention_core(dev, dtype, tol, B2, H, N, use_bias, use_gate):
     bt = layouts.tile_bias((bias[0].float() * LOG2E).to(dtype)) if use_bias else None
     NT = layouts.n_tiles(N)
     kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
-    _lib.key_bias(kb, mask[0], B=B2, N=N, mask_sb=N, mask_sn=1)
+    fl = torch.empty(B2, NT, dtype=torch.int32, device=dev)
+    _lib.key_bias(kb, fl, mask[0], B=B2, N=N, mask_sb=N, mask_sn=1)
     assert float(kb[:, :N][mask[0] != 0].abs().max()) == 0.0 and float(kb[:, :N][mask[0] == 0].max()) < -1e9
+    bad = torch.nn.functional.pad(mask[0].float(), (0, NT * 32 - N)).view(B2, NT, 32) == 0
+    want = torch.where(bad.all(-1), 2, torch.where(bad.any(-1), 1, 0)).to(torch.int32)
+    assert torch.equal(fl, want)
     out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
-    _lib.attention_fwd(out, qt, kt, vt, bt, kb, gate, B2=B2, H=H, Nq=N, Nk=N)
+    _lib.attention_fwd(out, qt, kt, vt, bt, kb, fl, gate, B2=B2, H=H, Nq=N, Nk=N)
     # oracle on exactly the operands the kernel saw (q rounded after scaling, bias rounded after log2e)
     q_eff = _np(qs) / scale * math.sqrt(32) / math.sqrt(32)
     b_eff = _np((bias[0].float() * LOG2E).to(dtype))[None] / LOG2E if use_bias else None
@@ -64,23 +68,25 @@ def test_attention_tiling_invariance_and_masked_keys(dev, dtype, tol):
     mask = torch.ones(B2, N, device=dev, dtype=dtype)
     mask[:, 90:] = 0
     kb = torch.empty(B2, 128, dtype=torch.float32, device=dev)
-    _lib.key_bias(kb, mask, B=B2, N=N, mask_sb=N, mask_sn=1)
+    fl = torch.empty(B2, 4, dtype=torch.int32, device=dev)
+    _lib.key_bias(kb, fl, mask, B=B2, N=N, mask_sb=N, mask_sn=1)
     outs = []
     for delta in (0.0, 5.0):
         k2, v2 = k.clone(), v.clone()
         k2[:, :, 90:] += delta
         v2[:, :, 90:] -= delta
         out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
-        _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k2), layouts.tile_v(v2), None, kb, None,
+        _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k2), layouts.tile_v(v2), None, kb, fl, None,
                            B2=B2, H=H, Nq=N, Nk=N)
         outs.append(_np(out))
     assert np.abs(outs[0] - outs[1]).max() == 0.0
     # same as attending over the first 90 keys only
     kb90 = torch.empty(B2, 96, dtype=torch.float32, device=dev)
-    _lib.key_bias(kb90, None, B=B2, N=90)
+    fl90 = torch.empty(B2, 3, dtype=torch.int32, device=dev)
+    _lib.key_bias(kb90, fl90, None, B=B2, N=90)
     out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
     _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k[:, :, :90].contiguous()),
-                       layouts.tile_v(v[:, :, :90].contiguous()), None, kb90, None, B2=B2, H=H, Nq=N, Nk=90)
+                       layouts.tile_v(v[:, :, :90].contiguous()), None, kb90, fl90, None, B2=B2, H=H, Nq=N, Nk=90)
     assert _rel(_np(out), outs[0]) < tol
 
 

@@ -171,7 +171,7 @@ def test_bias_tiles(dev, dtype, r, H):
     bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
     T = layouts.n_tiles(r)
     for transposed in (False, True):
-        bt = torch.zeros(H, T, T, 2, 32, 4, 4, dtype=dtype, device=dev)
+        bt = torch.zeros(H, T, T, 2, 32, 16, dtype=dtype, device=dev)
         tile = _lib.make_tile(bt, kind=_lib.FFK_TILE_BIAS, inner=r, s_o=T * 1024, s_h=T * T * 1024, ncols=H, scale=_lib.LOG2E)
         kw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else {}
         _lib.fused_linear(z, _pack(wb, 1), [tile], M=r * r, K=C, ln=(gam, bet), **kw)
