@@ -86,7 +86,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     for (int kc = 0; kc < kchunks; ++kc) {
         const int slot = kc & 1;
         commit(slot, kc);
-        __syncthreads();
+        lds_barrier();
         if (kc + 1 < kchunks) fetch(kc + 1);
         const unsigned char* pa = sA + slot * SLOT + (wm * 64 + l32) * P + half * (MM::KLANE * ES);
         const unsigned char* pb = sB + slot * SLOT + (wn * 64 + l32) * P + half * (MM::KLANE * ES);
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
                 for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     // row offsets of this tile, one integer division per row (kept in LDS for phase 2)
     __shared__ long s_off[BT];
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     // ---- phase 2: staged tile -> global ----
     OT* out = (OT*)d.out + (long)bz * d.o_bs;

@@ -80,6 +80,12 @@ __device__ __forceinline__ float group_max(float v, int width) {
     return v;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load / store of the wave (vmcnt(0)), which would serialise the register
+// prefetches and the fire-and-forget output stores of the streaming kernels with each barrier.
+// No kernel here communicates between waves through global memory, so LDS ordering suffices.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ------------------------------------------------------------ fast math ----
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
