@@ -191,7 +191,6 @@ def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanma
                            % (128 * len(tiles), K, a.dtype, tuple(w.shape), w.dtype))
     for i, t in enumerate(tiles):
         d.tiles[i] = t
-    d.reserved = int(os.environ.get('FFK_DBG', '0'))
     call("ffk_fused_linear", ctypes.byref(d), stream_ptr())
 
 

@@ -66,7 +66,7 @@ __device__ __forceinline__ typename Mma<T>::Frag identity_frag(int i, int l32, i
 }
 
 template <typename T, bool HAS_BIAS>
-__global__ __launch_bounds__(THREADS, 2) void attention_kernel(T* __restrict__ out, const T* __restrict__ q_t,
+__global__ __launch_bounds__(THREADS, sizeof(T) == 2 ? 3 : 2) void attention_kernel(T* __restrict__ out, const T* __restrict__ q_t,
                                                               const T* __restrict__ k_t, const T* __restrict__ v_t,
                                                               const T* __restrict__ bias_t,
                                                               const float* __restrict__ keybias,
@@ -117,10 +117,21 @@ __global__ __launch_bounds__(THREADS, 2) void attention_kernel(T* __restrict__ o
         for (int i = 0; i < NF; ++i) ident[i] = identity_frag<T>(i, l32, half);
     }
 
-    f32x16 o_acc;
+    // Online softmax with a lazily updated reference.  Instead of subtracting the running row maximum
+    // from every score on the vector pipe, the negated reference  -m_ref[q]  is the C operand of the
+    // first MFMA of each tile, so the accumulator already holds  s - m_ref  and exp2 is applied to it
+    // directly.  m_ref is only moved (and O / l rescaled) when a tile contains a score more than
+    // REF_SLACK above it, which bounds  p = exp2(s - m_ref) <= 2^REF_SLACK;  the first tile always
+    // sets it.  The row sum l is accumulated on the matrix pipe as well (ones . P^T).
+    constexpr float REF_SLACK = 20.0f;
+    constexpr float REF_FLOOR = -1.0e4f;          // keeps m_ref small when the first tile is fully masked
+    f32x16 o_acc, l_acc, negm;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) o_acc[v] = 0.0f;
-    float m_run = NEG_BIG, l_run = 0.0f;
+    for (int v = 0; v < 16; ++v) o_acc[v] = l_acc[v] = negm[v] = 0.0f;
+    bool first = true;
+    Frag ones;
+#pragma unroll
+    for (int t = 0; t < MM::KLANE; ++t) ones[t] = (T)1.0f;
 
     auto load_tile = [&](int kt, Ops16<T>& kk, Ops16<T>& vv, Ops16<T>& bb) {
         kk.load(kp + ((long)kt << 10));
@@ -129,10 +140,8 @@ __global__ __launch_bounds__(THREADS, 2) void attention_kernel(T* __restrict__ o
     };
 
     auto process = [&](int kt, const Ops16<T>& kc, const Ops16<T>& vc, const Ops16<T>& bc) {
-        // S^T = K . Q^T + Bias^T . I   (rows: keys, columns: queries)
-        f32x16 s;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.0f;
+        // S^T - m_ref = K . Q^T + Bias^T . I + (-m_ref)   (rows: keys, columns: queries)
+        f32x16 s = negm;
 #pragma unroll
         for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
         if (HAS_BIAS) {
@@ -151,26 +160,30 @@ __global__ __launch_bounds__(THREADS, 2) void attention_kernel(T* __restrict__ o
         float mt = fmaxf(s[0], s[1]);
 #pragma unroll
         for (int v = 2; v < 16; ++v) mt = fmaxf(mt, s[v]);
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m_run, mt);
+        if (first || __builtin_amdgcn_ballot_w64(mt > REF_SLACK) != 0) {
+            // move the reference of every row of this wave to its running maximum
+            const float mfull = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float delta = first ? fmaxf(mfull, REF_FLOOR) : fmaxf(mfull, 0.0f);
+            const float alpha = first ? 1.0f : fast_exp2(-delta);   // nothing accumulated before the first tile
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                s[v] -= delta;
+                negm[v] -= delta;
+                o_acc[v] *= alpha;
+            }
+            l_acc[0] *= alpha;
+            first = false;
+        }
         float p[16];
-        float ls = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            p[v] = fast_exp2(s[v] - m_new);
-            ls += p[v];
+        for (int v = 0; v < 16; ++v) p[v] = fast_exp2(s[v]);
+        // O^T += V^T . P^T  and  l += 1 . P^T   (rows: head dim, columns: queries)
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+            const Frag pf = PFrag<T>::make(p + i * MM::KLANE);
+            MM::mma(o_acc, vc.frag(i), pf);
+            MM::mma(l_acc, ones, pf);
         }
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {     // rescale only when some row's max moved
-            const float alpha = fast_exp2(m_run - m_new);
-            l_run *= alpha;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o_acc[v] *= alpha;
-            m_run = m_new;
-        }
-        l_run += ls;
-        // O^T += V^T . P^T   (rows: head dim, columns: queries)
-#pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(o_acc, vc.frag(i), PFrag<T>::make(p + i * MM::KLANE));
     };
 
     // Software pipeline over two register sets used alternately (no copies).  Every prefetch is
@@ -188,8 +201,10 @@ __global__ __launch_bounds__(THREADS, 2) void attention_kernel(T* __restrict__ o
     }
     if (kt_end & 1) process(last, ka, va, ba);
 
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / l_tot;
+    // every row of l_acc holds the full row sum (the MFMA already summed both lane halves); rows whose
+    // keys are all masked have l == 0 and produce zeros
+    const float l_tot = l_acc[0];
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     if (q < Nq) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {

@@ -20,6 +20,8 @@ int ffk_fail(int code, const char* fmt, ...);
         if (!(cond)) return ffk_fail((code), __VA_ARGS__); \
     } while (0)
 
+int ffk_linear_slab_launch(const ffk_linear_desc* d, hipStream_t st);   // ffk_linear_slab.hip
+
 static inline bool ffk_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Checks the launch that was just issued on this thread.
@@ -67,6 +69,14 @@ template <typename T> __device__ __forceinline__ Vec16<T> ld16(const T* p) {
 }
 template <typename T> __device__ __forceinline__ void st16(T* p, const Vec16<T>& v) {
     *reinterpret_cast<Vec16<T>*>(p) = v;
+}
+// Streaming (non-temporal) variants for data that is touched exactly once.
+template <typename T> __device__ __forceinline__ Vec16<T> ld16_nt(const T* p) {
+    u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return *reinterpret_cast<Vec16<T>*>(&r);
+}
+template <typename T> __device__ __forceinline__ void st16_nt(T* p, const Vec16<T>& v) {
+    __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&v), reinterpret_cast<u32x4*>(p));
 }
 
 // ------------------------------------------------------- wave reductions ----

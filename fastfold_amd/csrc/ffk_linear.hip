@@ -1,12 +1,10 @@
 // Fused linear layer for the Evoformer projections (see ffk_fused_linear in include/ffk.h).
 //
-// Persistent workgroups (4 wavefronts) walk over slabs of BM = 64 rows of A.  The whole
-// [BM x K] slab (K <= 256) is staged in LDS once - read from HBM exactly once - optionally
-// LayerNorm-ed in place, and then multiplied against every 128-row tile of the weight matrix.
-// The next slab is prefetched into registers while the current one is being processed, and
-// each weight tile (128 rows x 256 bytes of K) is prefetched into registers during the MFMAs
-// and epilogue of the previous tile; weights are a few hundred KB and stay in L2.  All global
-// loads are issued without per-lane branches (indices are clamped) so they overlap.
+// One workgroup (4 wavefronts) owns BM rows of A.  The whole [BM x K] slab (K <= 256) is
+// staged in LDS once - read from HBM exactly once - optionally LayerNorm-ed in place, and
+// then multiplied against every 128-row tile of the weight matrix.  Weight tiles stream
+// through a double-buffered LDS ring in K-chunks (register prefetch of the next chunk
+// overlaps the MFMAs of the current one); weights are a few hundred KB and stay in L2.
 // The 32x32 MFMA computes C^T: the weight fragment is the M-operand (rows = output
 // channels) and the activation fragment the N-operand (columns = rows of A), so a lane
 // ends up with 4 consecutive output channels of one row.  Results are staged through LDS
@@ -21,14 +19,10 @@ constexpr int THREADS = 256;
 
 template <typename T> struct LinCfg;
 template <> struct LinCfg<bf16_t> {
-    static constexpr int BM = 128;                  // rows of A per slab
-    static constexpr int WM = 4, WN = 1;            // wave grid: 32 rows x 128 channels per wave
-    static constexpr int KC = 128;                  // K elements per weight chunk (256 bytes per row)
+    static constexpr int BM = 64, WM = 2, WN = 2, BK = 32;
 };
 template <> struct LinCfg<float> {
-    static constexpr int BM = 64;
-    static constexpr int WM = 2, WN = 2;            // 32 rows x 64 channels per wave
-    static constexpr int KC = 64;
+    static constexpr int BM = 64, WM = 2, WN = 2, BK = 32;
 };
 
 struct LinArgs {
@@ -96,23 +90,21 @@ __device__ __forceinline__ void stage_tile(const f32x16 (&acc)[CT], const T (&bv
     }
 }
 
-// NA: 16-byte vectors of A each thread prefetches for the next slab (8), or 0 = the slab is
-// loaded at the start of its own iteration (channel-major A, or rows too long to keep in registers).
-template <typename T, int NA>
-__global__ __launch_bounds__(THREADS, 2) void fused_linear_kernel(const LinArgs args) {
+template <typename T>
+__global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs args) {
     typedef LinCfg<T> Cfg;
     typedef Mma<T> MM;
-    constexpr int BM = Cfg::BM, WN = Cfg::WN, KC = Cfg::KC;
-    constexpr int CT = NT / (WN * 32);             // 32-channel MFMA tiles per wave (= 2)
+    constexpr int BM = Cfg::BM, WM = Cfg::WM, WN = Cfg::WN, BK = Cfg::BK;
+    constexpr int CT = NT / (WN * 32);             // 32-channel MFMA tiles per wave
     constexpr int VEC = DT<T>::VEC;
     constexpr int ES = sizeof(T);
-    constexpr int WP = KC * ES + 16;               // weight chunk row pitch (bytes)
-    constexpr int WBUF = NT * WP;
+    constexpr int WP = BK * ES + 16;               // weight ring row pitch (bytes)
+    constexpr int WBUF = NT * WP;                  // one ring slot
     constexpr int CP = NT * ES + 16;               // staged C pitch, [row][channel]
     constexpr int CPT = BM * ES + 16;              // staged C pitch, [channel][row]
-    constexpr int WV = NT * (KC / VEC) / THREADS;  // weight vectors per thread per chunk (= 8)
-    constexpr int NAR = NA > 0 ? NA : 1;
-    static_assert(BM * CP <= WBUF && NT * CPT <= WBUF, "C staging must fit in the weight buffer");
+    static_assert(BM * CP <= 2 * WBUF, "C staging must fit in the weight ring");
+    static_assert(NT * CPT <= 2 * WBUF + 4096, "transposed C staging");
+    (void)WM;
 
     const ffk_linear_desc& d = args.d;
     const int K = d.K, M = d.M;
@@ -121,383 +113,339 @@ __global__ __launch_bounds__(THREADS, 2) void fused_linear_kernel(const LinArgs 
     __shared__ RowTab tab;
     unsigned char* sA = smem;
     unsigned char* sW = smem + (size_t)BM * AP;
-    unsigned char* sC = sW;                        // the staged output tile aliases the weight buffer
+    unsigned char* sC = sW;                        // aliases the ring between tiles
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, half = lane >> 5;
+    const long m0 = (long)blockIdx.x * BM;
     const T* A = (const T*)d.a;
     const T* W = (const T*)d.w;
-    const int n_slabs = (M + BM - 1) / BM;
 
-    // ---- weight chunks: whole 128 x KC chunk prefetched into registers ----
-    const int n_kc = (K + KC - 1) / KC;
-    const int chunks_per_slab = d.n_tiles * n_kc;
-    Vec16<T> wreg[WV];
-    // Workgroups that share a CU would otherwise run the same phase (load, MFMA, store) at the same
-    // time; odd workgroups walk the N-tiles starting from the middle so that their phases interleave.
-    const int rot = (blockIdx.x & 1) ? d.n_tiles / 2 : 0;
-    auto w_fetch = [&](int chunk) {                // chunk index within a slab
-        int nt = chunk / n_kc;
-        const int kc = chunk - nt * n_kc;
-        nt = nt + rot < d.n_tiles ? nt + rot : nt + rot - d.n_tiles;
-        const int kv = (K - kc * KC < KC ? K - kc * KC : KC) / VEC;   // vectors per row in this chunk
+    // ---- weight chunk prefetch (registers) ----
+    constexpr int WVEC = NT * BK / VEC / THREADS;  // 16-byte vectors per thread per chunk (= 4)
+    Vec16<T> wreg[WVEC];
+    const int kchunks = K / BK;
+    const int total_chunks = d.n_tiles * kchunks;
+    auto w_fetch = [&](int chunk) {
+        const int nt = chunk / kchunks, kc = chunk - nt * kchunks;
 #pragma unroll
-        for (int i = 0; i < WV; ++i) {
+        for (int i = 0; i < WVEC; ++i) {
             const int v = tid + THREADS * i;
-            const int r = v / (KC / VEC);
-            int c = v % (KC / VEC);
-            c = c < kv ? c : kv - 1;
-            wreg[i] = ld16(W + ((long)nt * NT + r) * K + kc * KC + c * VEC);
+            const int r = v / (BK / VEC), c = v % (BK / VEC);
+            wreg[i] = ld16(W + ((long)nt * NT + r) * K + kc * BK + c * VEC);
         }
     };
-    auto w_commit = [&](int kc) {
-        const int kv = (K - kc * KC < KC ? K - kc * KC : KC) / VEC;
+    auto w_commit = [&](int slot) {
 #pragma unroll
-        for (int i = 0; i < WV; ++i) {
+        for (int i = 0; i < WVEC; ++i) {
             const int v = tid + THREADS * i;
-            const int r = v / (KC / VEC), c = v % (KC / VEC);
-            if (c < kv) *reinterpret_cast<Vec16<T>*>(sW + r * WP + c * 16) = wreg[i];
+            const int r = v / (BK / VEC), c = v % (BK / VEC);
+            *reinterpret_cast<Vec16<T>*>(sW + slot * WBUF + r * WP + c * 16) = wreg[i];
         }
     };
-
-    // ---- A slab: row-major rows are prefetched one slab ahead into registers ----
-    const int vpr = K / VEC;                       // 16-byte vectors per row
-    int cs = 3;
-    while ((1 << cs) < vpr) ++cs;                  // lanes per row rounded up to a power of two
-    const int a_c_raw = tid & ((1 << cs) - 1);
-    const int a_c = a_c_raw < vpr ? a_c_raw : vpr - 1;
-    const int a_r_first = tid >> cs, a_rstep = THREADS >> cs;
-    const bool a_plain = d.a_inner >= M;           // one contiguous group: no division needed
-    Vec16<T> areg[NAR];
-    auto a_fetch = [&](int slab) {
-#pragma unroll
-        for (int i = 0; i < NAR; ++i) {
-            int r = a_r_first + i * a_rstep;
-            r = r < BM ? r : BM - 1;
-            long m = (long)slab * BM + r;
-            m = m < M ? m : M - 1;
-            long off;
-            if (a_plain) {
-                off = m * d.a_si;
-            } else {
-                const unsigned hi = (unsigned)m / (unsigned)d.a_inner;
-                const unsigned lo = (unsigned)m - hi * (unsigned)d.a_inner;
-                off = (long)hi * d.a_so + (long)lo * d.a_si;
-            }
-            areg[i] = ld16(A + off + a_c * VEC);
-        }
-    };
-    auto a_commit = [&]() {
-#pragma unroll
-        for (int i = 0; i < NAR; ++i) {
-            const int r = a_r_first + i * a_rstep;
-            if (r < BM && a_c_raw < vpr) *reinterpret_cast<Vec16<T>*>(sA + r * AP + a_c * 16) = areg[i];
-        }
-    };
-
-    if (NA > 0) a_fetch(blockIdx.x);
     w_fetch(0);
 
-    for (int slab = blockIdx.x; slab < n_slabs; slab += gridDim.x) {
-        const long m0 = (long)slab * BM;
-        lds_barrier();                           // previous slab completely finished (sA, sC, tab free)
-        if (NA > 0) {
-            a_commit();
-            if (slab + (int)gridDim.x < n_slabs) a_fetch(slab + gridDim.x);
+    // ---- stage the A slab (loads issued four at a time so their latencies overlap) ----
+    fill_rowtab(tab, tid, BM, m0, M, d.a_inner, d.a_so, d.a_si);
+    lds_barrier();
+    // Loads below are unconditional (row / column indices are clamped to valid ones instead of
+    // being predicated) so that a batch of four is in flight at once; only the LDS stores are guarded.
+    // Rows beyond M hold a copy of row M-1: their results are never stored.
+    if (!d.a_chanmajor) {
+        const int vpr = K / VEC;                   // 16-byte vectors per row
+        int cs = 3;
+        while ((1 << cs) < vpr) ++cs;              // lanes per row rounded up to a power of two
+        const int c_raw = tid & ((1 << cs) - 1);
+        const int c = c_raw < vpr ? c_raw : vpr - 1;
+        const int r_first = tid >> cs, rstep = THREADS >> cs;
+        const int n_it = BM / rstep;
+        for (int i0 = 0; i0 < n_it; i0 += 4) {
+            Vec16<T> buf[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int r = r_first + (i0 + j) * rstep;
+                r = r < BM ? r : BM - 1;
+                buf[j] = ld16(A + tab.off[r] + c * VEC);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = r_first + (i0 + j) * rstep;
+                if (r < BM && c_raw < vpr) *reinterpret_cast<Vec16<T>*>(sA + r * AP + c * 16) = buf[j];
+            }
+        }
+    } else {
+        // element (m, k) at a + k * a_cs + rowoff(m): read runs of VEC rows, scatter into [row][k]
+        constexpr int RPV = BM / VEC;              // VEC-row runs per channel (a power of two)
+        const int n_it = K * RPV / THREADS;        // K % 32 == 0  =>  a multiple of 4 (bf16) / 2... see below
+        // uniform fast-path test: every run of VEC rows of this slab is contiguous and 16-byte aligned
+        const bool fast = d.a_si == 1 && m0 + BM <= M && (d.a_inner % VEC) == 0 && (d.a_so % VEC) == 0 &&
+                          (d.a_cs % VEC) == 0 && (m0 % VEC) == 0;
+        if (fast) {
+            for (int i0 = 0; i0 < n_it; i0 += 4) {
+                Vec16<T> buf[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    int v = tid + THREADS * (i0 + j);
+                    v = v < K * RPV ? v : K * RPV - 1;
+                    const int k = v / RPV, r0 = (v % RPV) * VEC;
+                    buf[j] = ld16(A + (long)k * d.a_cs + tab.off[r0]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int k = v / RPV, r0 = (v % RPV) * VEC;
+                    if (v < K * RPV) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) *reinterpret_cast<T*>(sA + (r0 + e) * AP + k * ES) = buf[j].e[e];
+                    }
+                }
+            }
         } else {
-            fill_rowtab(tab, tid, BM, m0, M, d.a_inner, d.a_so, d.a_si);
+            for (int v = tid; v < K * BM; v += THREADS) {
+                const int k = v / BM, r = v % BM;
+                *reinterpret_cast<T*>(sA + r * AP + k * ES) = A[(long)k * d.a_cs + tab.off[r]];
+            }
+        }
+    }
+    lds_barrier();
+
+    // ---- LayerNorm prologue, in place ----
+    if (d.ln_gamma) {
+        constexpr int TPR = THREADS / BM;          // threads per row (adjacent lanes)
+        const int r = tid / TPR, j = tid % TPR;
+        const int vpr = K / VEC;
+        const T* gam = (const T*)d.ln_gamma;
+        const T* bet = (const T*)d.ln_beta;
+        unsigned char* rowp = sA + r * AP;
+        float s = 0.0f;
+        for (int c = j; c < vpr; c += TPR) {
+            Vec16<T> x = *reinterpret_cast<Vec16<T>*>(rowp + c * 16);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s += DT<T>::to_f(x.e[e]);
+        }
+        const float mu = group_sum(s, TPR) / (float)K;
+        float q = 0.0f;
+        for (int c = j; c < vpr; c += TPR) {
+            Vec16<T> x = *reinterpret_cast<Vec16<T>*>(rowp + c * 16);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float dd = DT<T>::to_f(x.e[e]) - mu;
+                q += dd * dd;
+            }
+        }
+        const float rs = rsqrtf(group_sum(q, TPR) / (float)K + d.ln_eps);
+        for (int c = j; c < vpr; c += TPR) {
+            Vec16<T> x = *reinterpret_cast<Vec16<T>*>(rowp + c * 16);
+            Vec16<T> g = ld16(gam + c * VEC), b = ld16(bet + c * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                x.e[e] = DT<T>::from_f((DT<T>::to_f(x.e[e]) - mu) * rs * DT<T>::to_f(g.e[e]) + DT<T>::to_f(b.e[e]));
+            *reinterpret_cast<Vec16<T>*>(rowp + c * 16) = x;
+        }
+        // visibility to the other waves is ensured by the barrier of the first weight chunk
+    }
+
+    // ---- main loop over N-tiles ----
+    const unsigned char* a_frag_base = sA + (wm * 32 + l32) * AP + half * (MM::KLANE * ES);
+    int chunk = 0;
+    for (int nt = 0; nt < d.n_tiles; ++nt) {
+        f32x16 acc[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[ct][v] = 0.0f;
+
+        for (int kc = 0; kc < kchunks; ++kc, ++chunk) {
+            const int slot = chunk & 1;
+            w_commit(slot);
             lds_barrier();
-            if (!d.a_chanmajor) {
-                const int n_it = BM / a_rstep;
-                for (int i0 = 0; i0 < n_it; i0 += 4) {
-                    Vec16<T> buf[4];
+            if (chunk + 1 < total_chunks) w_fetch(chunk + 1);
+            const unsigned char* wb = sW + slot * WBUF + (wn * CT * 32 + l32) * WP + half * (MM::KLANE * ES);
+            const unsigned char* ab = a_frag_base + kc * BK * ES;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        int r = a_r_first + (i0 + j) * a_rstep;
-                        r = r < BM ? r : BM - 1;
-                        buf[j] = ld16(A + tab.off[r] + a_c * VEC);
-                    }
+            for (int ks = 0; ks < BK / MM::KSTEP; ++ks) {
+                typename MM::Frag fx = *reinterpret_cast<const typename MM::Frag*>(ab + ks * MM::KSTEP * ES);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int r = a_r_first + (i0 + j) * a_rstep;
-                        if (r < BM && a_c_raw < vpr) *reinterpret_cast<Vec16<T>*>(sA + r * AP + a_c * 16) = buf[j];
-                    }
+                for (int ct = 0; ct < CT; ++ct) {
+                    typename MM::Frag fw =
+                        *reinterpret_cast<const typename MM::Frag*>(wb + ct * 32 * WP + ks * MM::KSTEP * ES);
+                    MM::mma(acc[ct], fw, fx);
                 }
+            }
+        }
+
+        // ---- epilogue of this tile ----
+        const ffk_tile& t = d.tiles[nt];
+        const bool mode_c = (t.kind == FFK_TILE_STRIDED && t.s_d == 1) || t.kind == FFK_TILE_QK;
+        const int prow = wm * 32 + l32;                         // row within the slab
+        const long mrow = m0 + prow;
+        T bv[CT][4][4];
+        if (t.bias) {
+            const T* bias = (const T*)t.bias;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const T* bp = bias + (wn * CT + ct) * 32 + 8 * g + 4 * half;
+                    if (ES == 2) *reinterpret_cast<u32x2*>(&bv[ct][g][0]) = *reinterpret_cast<const u32x2*>(bp);
+                    else *reinterpret_cast<u32x4*>(&bv[ct][g][0]) = *reinterpret_cast<const u32x4*>(bp);
+                }
+        } else {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) bv[ct][g][e] = DT<T>::from_f(0.0f);
+        }
+        float rmask = 1.0f;
+        if (t.rowmask) {
+            long mr = mrow < M ? mrow : M - 1;
+            const unsigned hi = (unsigned)mr / (unsigned)t.inner;
+            const unsigned lo = (unsigned)mr - hi * (unsigned)t.inner;
+            rmask = DT<T>::to_f(((const T*)t.rowmask)[(long)hi * t.m_so + (long)lo * t.m_si]);
+        }
+        lds_barrier();                                        // all waves done with the ring
+        fill_rowtab(tab, tid, BM, m0, M, t.inner, t.s_o, t.s_i);
+        {
+            const float scl = t.scale * rmask;
+            unsigned char* crow = mode_c ? sC + prow * CP : sC + prow * ES;
+            const int chan0 = wn * CT * 32 + 4 * half;
+            if (t.glu) {
+                stage_tile<T, CT, 1, 0>(acc, bv, scl, crow, mode_c, wn * CT * 16 + 4 * half, CPT);
+            } else if (t.act == FFK_ACT_RELU) {
+                stage_tile<T, CT, 0, FFK_ACT_RELU>(acc, bv, scl, crow, mode_c, chan0, CPT);
+            } else if (t.act == FFK_ACT_SIGMOID) {
+                stage_tile<T, CT, 0, FFK_ACT_SIGMOID>(acc, bv, scl, crow, mode_c, chan0, CPT);
             } else {
-                // element (m, k) at a + k * a_cs + rowoff(m): read runs of VEC rows, scatter into [row][k]
-                constexpr int RPV = BM / VEC;
-                const int n_it = (K * RPV + THREADS - 1) / THREADS;
-                const bool fast = d.a_si == 1 && m0 + BM <= M && (d.a_inner % VEC) == 0 && (d.a_so % VEC) == 0 &&
-                                  (d.a_cs % VEC) == 0 && (m0 % VEC) == 0;
-                if (fast) {
-                    for (int i0 = 0; i0 < n_it; i0 += 4) {
-                        Vec16<T> buf[4];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            int v = tid + THREADS * (i0 + j);
-                            v = v < K * RPV ? v : K * RPV - 1;
-                            const int k = v / RPV, r0 = (v % RPV) * VEC;
-                            buf[j] = ld16(A + (long)k * d.a_cs + tab.off[r0]);
-                        }
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int v = tid + THREADS * (i0 + j);
-                            const int k = v / RPV, r0 = (v % RPV) * VEC;
-                            if (v < K * RPV) {
-#pragma unroll
-                                for (int e = 0; e < VEC; ++e)
-                                    *reinterpret_cast<T*>(sA + (r0 + e) * AP + k * ES) = buf[j].e[e];
-                            }
-                        }
-                    }
-                } else {
-                    for (int v = tid; v < K * BM; v += THREADS) {
-                        const int k = v / BM, r = v % BM;
-                        *reinterpret_cast<T*>(sA + r * AP + k * ES) = A[(long)k * d.a_cs + tab.off[r]];
-                    }
-                }
+                stage_tile<T, CT, 0, FFK_ACT_NONE>(acc, bv, scl, crow, mode_c, chan0, CPT);
             }
         }
         lds_barrier();
 
-        // ---- LayerNorm prologue, in place ----
-        if (d.ln_gamma) {
-            constexpr int TPR = THREADS / BM;      // threads per row (adjacent lanes)
-            const int r = tid / TPR, j = tid % TPR;
-            const T* gam = (const T*)d.ln_gamma;
-            const T* bet = (const T*)d.ln_beta;
-            unsigned char* rowp = sA + r * AP;
-            float s = 0.0f;
-            for (int c = j; c < vpr; c += TPR) {
-                Vec16<T> x = *reinterpret_cast<Vec16<T>*>(rowp + c * 16);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) s += DT<T>::to_f(x.e[e]);
-            }
-            const float mu = group_sum(s, TPR) / (float)K;
-            float q = 0.0f;
-            for (int c = j; c < vpr; c += TPR) {
-                Vec16<T> x = *reinterpret_cast<Vec16<T>*>(rowp + c * 16);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const float dd = DT<T>::to_f(x.e[e]) - mu;
-                    q += dd * dd;
-                }
-            }
-            const float rs = rsqrtf(group_sum(q, TPR) / (float)K + d.ln_eps);
-            for (int c = j; c < vpr; c += TPR) {
-                Vec16<T> x = *reinterpret_cast<Vec16<T>*>(rowp + c * 16);
-                Vec16<T> g = ld16(gam + c * VEC), b = ld16(bet + c * VEC);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    x.e[e] = DT<T>::from_f((DT<T>::to_f(x.e[e]) - mu) * rs * DT<T>::to_f(g.e[e]) + DT<T>::to_f(b.e[e]));
-                *reinterpret_cast<Vec16<T>*>(rowp + c * 16) = x;
-            }
-            // made visible to the other waves by the first barrier of the tile loop
-        }
-
-        // ---- N-tiles ----
-        const unsigned char* a_frag_base = sA + (wm * 32 + l32) * AP + half * (MM::KLANE * ES);
-        const unsigned char* w_frag_base = sW + (wn * CT * 32 + l32) * WP + half * (MM::KLANE * ES);
-        int chunk = 0;
-        for (int nt0 = 0; nt0 < d.n_tiles; ++nt0) {
-            const int nt = nt0 + rot < d.n_tiles ? nt0 + rot : nt0 + rot - d.n_tiles;
-            const ffk_tile& t = d.tiles[nt];
-            const bool mode_c = (t.kind == FFK_TILE_STRIDED && t.s_d == 1) || t.kind == FFK_TILE_QK;
-            const int prow = wm * 32 + l32;                     // row within the slab
-            // bias (4 consecutive channels per load) and row mask of this lane, fetched ahead of use
-            T bv[CT][4][4];
-            if (t.bias) {
-                const T* bias = (const T*)t.bias;
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const T* bp = bias + (wn * CT + ct) * 32 + 8 * g + 4 * half;
-                        if (ES == 2) *reinterpret_cast<u32x2*>(&bv[ct][g][0]) = *reinterpret_cast<const u32x2*>(bp);
-                        else *reinterpret_cast<u32x4*>(&bv[ct][g][0]) = *reinterpret_cast<const u32x4*>(bp);
-                    }
-            } else {
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) bv[ct][g][e] = DT<T>::from_f(0.0f);
-            }
-            float rmask = 1.0f;
-            if (t.rowmask) {
-                long mrow = m0 + prow;
-                mrow = mrow < M ? mrow : M - 1;
-                const unsigned hi = (unsigned)mrow / (unsigned)t.inner;
-                const unsigned lo = (unsigned)mrow - hi * (unsigned)t.inner;
-                rmask = DT<T>::to_f(((const T*)t.rowmask)[(long)hi * t.m_so + (long)lo * t.m_si]);
-            }
-
-            f32x16 acc[CT];
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[ct][v] = 0.0f;
-
-            for (int kc = 0; kc < n_kc; ++kc, ++chunk) {
-                lds_barrier();                   // consumers of the weight buffer / staged tile are done
-                w_commit(kc);
-                lds_barrier();
-                {   // prefetch the next chunk (wraps to chunk 0 for the next slab: same weights)
-                    const int nxt = chunk + 1 < chunks_per_slab ? chunk + 1 : 0;
-                    w_fetch(nxt);
-                }
-                const int ksteps = (K - kc * KC < KC ? K - kc * KC : KC) / MM::KSTEP;
-                const unsigned char* ab = a_frag_base + kc * KC * ES;
-                for (int ks = 0; ks < (d.reserved >= 3 ? 0 : ksteps); ++ks) {
-                    typename MM::Frag fx = *reinterpret_cast<const typename MM::Frag*>(ab + ks * MM::KSTEP * ES);
-#pragma unroll
-                    for (int ct = 0; ct < CT; ++ct) {
-                        typename MM::Frag fw =
-                            *reinterpret_cast<const typename MM::Frag*>(w_frag_base + ct * 32 * WP + ks * MM::KSTEP * ES);
-                        MM::mma(acc[ct], fw, fx);
-                    }
-                }
-            }
-
-            // ---- epilogue of this tile ----
-            lds_barrier();                                    // all waves done with the weight buffer
-            if (d.reserved >= 2) continue;
-            fill_rowtab(tab, tid, BM, m0, M, t.inner, t.s_o, t.s_i);
-            // the activation variant is selected once per tile; each variant is straight-line code
-            {
-                const float scl = t.scale * rmask;
-                unsigned char* crow = mode_c ? sC + prow * CP : sC + prow * ES;
-                const int chan0 = wn * CT * 32 + 4 * half;
-                if (t.glu) {        // pairs of MFMA tiles collapse to one: half as many output channels
-                    stage_tile<T, CT, 1, 0>(acc, bv, scl, crow, mode_c, wn * CT * 16 + 4 * half, CPT);
-                } else if (t.act == FFK_ACT_RELU) {
-                    stage_tile<T, CT, 0, FFK_ACT_RELU>(acc, bv, scl, crow, mode_c, chan0, CPT);
-                } else if (t.act == FFK_ACT_SIGMOID) {
-                    stage_tile<T, CT, 0, FFK_ACT_SIGMOID>(acc, bv, scl, crow, mode_c, chan0, CPT);
-                } else {
-                    stage_tile<T, CT, 0, FFK_ACT_NONE>(acc, bv, scl, crow, mode_c, chan0, CPT);
-                }
-            }
-            lds_barrier();
-
-            T* out = (T*)t.out;
-            const int ncols = t.ncols;
-            if (d.reserved == 1) continue;
-            if (mode_c) {
-                constexpr int VPR = NT / VEC;
-                constexpr int N_IT = BM * VPR / THREADS;
-                const bool qk = t.kind == FFK_TILE_QK;
-                const T* gate = (const T*)t.gate;
-                const T* resid = (const T*)t.resid;
-                const int c_last = ncols >= VEC ? ((ncols - VEC) / VEC) * VEC : 0;   // last full vector column
+        T* out = (T*)t.out;
+        const int ncols = t.ncols;
+        if (mode_c) {
+            constexpr int VPR = NT / VEC;
+            constexpr int N_IT = BM * VPR / THREADS;             // = 8
+            const bool qk = t.kind == FFK_TILE_QK;
+            const T* gate = (const T*)t.gate;
+            const T* resid = (const T*)t.resid;
+            const int c_last = ncols >= VEC ? ((ncols - VEC) / VEC) * VEC : 0;   // last full vector column
 #pragma unroll 1
-                for (int i0 = 0; i0 < N_IT; i0 += 4) {
-                    Vec16<T> x[4], gv[4], rv[4];
-                    long o[4];
-                    // issue every load of the batch first (clamped, branch-free), then combine and store
+            for (int i0 = 0; i0 < N_IT; i0 += 4) {
+                Vec16<T> x[4], gv[4], rv[4];
+                long o[4];
+                // issue every load of the batch first (clamped, branch-free), then combine and store
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int v = tid + THREADS * (i0 + j);
-                        const int r = v / VPR;
-                        int c = (v % VPR) * VEC;
-                        c = c + VEC <= ncols ? c : c_last;
-                        if (qk) {
-                            const int n = tab.lo[r];
-                            o[j] = (long)tab.hi[r] * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 +
-                                   qk_tile_off(n & 31, c & 31);
-                        } else {
-                            o[j] = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
-                        }
-                        x[j] = *reinterpret_cast<const Vec16<T>*>(sC + r * CP + c * ES);
-                        long mr = m0 + r;
-                        mr = mr < M ? mr : M - 1;
-                        if (gate) gv[j] = ld16(gate + mr * t.gate_ld + c);
-                        if (resid) rv[j] = ld16(resid + o[j]);
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int v = tid + THREADS * (i0 + j);
-                        const int r = v / VPR, c = (v % VPR) * VEC;
-                        if (gate) {
-#pragma unroll
-                            for (int e = 0; e < VEC; ++e)
-                                x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) * DT<T>::to_f(gv[j].e[e]));
-                        }
-                        if (resid) {
-#pragma unroll
-                            for (int e = 0; e < VEC; ++e)
-                                x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) + DT<T>::to_f(rv[j].e[e]));
-                        }
-                        if (m0 + r < M && c + VEC <= ncols) st16(out + o[j], x[j]);
-                    }
-                }
-                if (ncols % VEC != 0) {
-                    // ragged tail (fewer than VEC channels left): element-wise, rare
-                    const int c0 = (ncols / VEC) * VEC, nrem = ncols - c0;
-                    for (int v = tid; v < BM * nrem; v += THREADS) {
-                        const int r = v / nrem, c = c0 + v % nrem;
-                        if (m0 + r >= M) continue;
-                        float y = DT<T>::to_f(*reinterpret_cast<const T*>(sC + r * CP + c * ES));
-                        long oo;
-                        if (qk) {
-                            const int n = tab.lo[r];
-                            oo = (long)tab.hi[r] * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 + qk_tile_off(n & 31, c & 31);
-                        } else {
-                            oo = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
-                        }
-                        if (gate) y = DT<T>::to_f(DT<T>::from_f(y * DT<T>::to_f(gate[(m0 + r) * t.gate_ld + c])));
-                        if (resid) y += DT<T>::to_f(resid[oo]);
-                        out[oo] = DT<T>::from_f(y);
-                    }
-                }
-            } else {
-                constexpr int QPR = BM / 4;                         // 4-row runs per channel
-                for (int v = tid; v < ncols * QPR; v += THREADS) {
-                    const int c = v / QPR, r = (v % QPR) * 4;
-                    if (m0 + r >= M) continue;
-                    const T* src = reinterpret_cast<const T*>(sC + c * CPT + r * ES);
-                    long o[4];
-                    bool ok[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        ok[e] = m0 + r + e < M;
-                        const int hi = tab.hi[r + e], lo = tab.lo[r + e];
-                        if (t.kind == FFK_TILE_V) {
-                            o[e] = (long)hi * t.s_o + (long)(c >> 5) * t.s_h + (long)(lo >> 5) * 1024 + acc_tile_off(lo & 31, c & 31);
-                        } else if (t.kind == FFK_TILE_BIAS) {
-                            // logical row = (query hi, key lo); channel = head
-                            o[e] = (long)c * t.s_h + (long)(hi >> 5) * t.s_o + (long)(lo >> 5) * 1024 +
-                                   qk_tile_off(lo & 31, hi & 31);
-                        } else {
-                            o[e] = tab.off[r + e] + (long)(c >> 5) * t.s_h + (long)(c & 31) * t.s_d;
-                        }
-                    }
-                    const bool run = ok[3] && o[1] == o[0] + 1 && o[2] == o[0] + 2 && o[3] == o[0] + 3 &&
-                                     ((reinterpret_cast<uintptr_t>(out + o[0]) & (4 * ES - 1)) == 0);
-                    if (run) {
-                        if (ES == 2) {
-                            *reinterpret_cast<u32x2*>(out + o[0]) = *reinterpret_cast<const u32x2*>(src);
-                        } else {
-                            *reinterpret_cast<u32x4*>(out + o[0]) = *reinterpret_cast<const u32x4*>(src);
-                        }
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int r = v / VPR;
+                    int c = (v % VPR) * VEC;
+                    c = c + VEC <= ncols ? c : c_last;
+                    if (qk) {
+                        const int n = tab.lo[r];
+                        o[j] = (long)tab.hi[r] * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 +
+                               qk_tile_off(n & 31, c & 31);
                     } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (ok[e]) out[o[e]] = src[e];
+                        o[j] = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
                     }
+                    x[j] = *reinterpret_cast<const Vec16<T>*>(sC + r * CP + c * ES);
+                    long mr = m0 + r;
+                    mr = mr < M ? mr : M - 1;
+                    if (gate) gv[j] = ld16(gate + mr * t.gate_ld + c);
+                    if (resid) rv[j] = ld16(resid + o[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int v = tid + THREADS * (i0 + j);
+                    const int r = v / VPR, c = (v % VPR) * VEC;
+                    if (gate) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) * DT<T>::to_f(gv[j].e[e]));
+                    }
+                    if (resid) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) + DT<T>::to_f(rv[j].e[e]));
+                    }
+                    if (m0 + r < M && c + VEC <= ncols) st16(out + o[j], x[j]);
+                }
+            }
+            if (ncols % VEC != 0) {
+                // ragged tail (fewer than VEC channels left): element-wise, rare
+                const int c0 = (ncols / VEC) * VEC, nrem = ncols - c0;
+                for (int v = tid; v < BM * nrem; v += THREADS) {
+                    const int r = v / nrem, c = c0 + v % nrem;
+                    if (m0 + r >= M) continue;
+                    float y = DT<T>::to_f(*reinterpret_cast<const T*>(sC + r * CP + c * ES));
+                    long oo;
+                    if (qk) {
+                        const int n = tab.lo[r];
+                        oo = (long)tab.hi[r] * t.s_o + (long)(c >> 5) * t.s_h + (long)(n >> 5) * 1024 + qk_tile_off(n & 31, c & 31);
+                    } else {
+                        oo = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
+                    }
+                    if (gate) y = DT<T>::to_f(DT<T>::from_f(y * DT<T>::to_f(gate[(m0 + r) * t.gate_ld + c])));
+                    if (resid) y += DT<T>::to_f(resid[oo]);
+                    out[oo] = DT<T>::from_f(y);
+                }
+            }
+        } else {
+            constexpr int QPR = BM / 4;                         // 4-row runs per channel
+            for (int v = tid; v < ncols * QPR; v += THREADS) {
+                const int c = v / QPR, r = (v % QPR) * 4;
+                if (m0 + r >= M) continue;
+                const T* src = reinterpret_cast<const T*>(sC + c * CPT + r * ES);
+                long o[4];
+                bool ok[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ok[e] = m0 + r + e < M;
+                    const int hi = tab.hi[r + e], lo = tab.lo[r + e];
+                    if (t.kind == FFK_TILE_V) {
+                        o[e] = (long)hi * t.s_o + (long)(c >> 5) * t.s_h + (long)(lo >> 5) * 1024 + acc_tile_off(lo & 31, c & 31);
+                    } else if (t.kind == FFK_TILE_BIAS) {
+                        // logical row = (query hi, key lo); channel = head
+                        o[e] = (long)c * t.s_h + (long)(hi >> 5) * t.s_o + (long)(lo >> 5) * 1024 +
+                               qk_tile_off(lo & 31, hi & 31);
+                    } else {
+                        o[e] = tab.off[r + e] + (long)(c >> 5) * t.s_h + (long)(c & 31) * t.s_d;
+                    }
+                }
+                const bool run = ok[3] && o[1] == o[0] + 1 && o[2] == o[0] + 2 && o[3] == o[0] + 3 &&
+                                 ((reinterpret_cast<uintptr_t>(out + o[0]) & (4 * ES - 1)) == 0);
+                if (run) {
+                    if (ES == 2) {
+                        *reinterpret_cast<u32x2*>(out + o[0]) = *reinterpret_cast<const u32x2*>(src);
+                    } else {
+                        *reinterpret_cast<u32x4*>(out + o[0]) = *reinterpret_cast<const u32x4*>(src);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (ok[e]) out[o[e]] = src[e];
                 }
             }
         }
+        lds_barrier();                                        // staging area is the ring again
     }
 }
 
-template <typename T, int NA>
-int launch_linear_na(const ffk_linear_desc& d, size_t smem, hipStream_t st) {
+template <typename T>
+int launch_linear(const ffk_linear_desc& d, hipStream_t st) {
+    typedef LinCfg<T> Cfg;
+    constexpr int ES = sizeof(T);
+    constexpr int WP = Cfg::BK * ES + 16;
+    size_t ring = 2 * (size_t)NT * WP;
+    size_t ct = (size_t)NT * (Cfg::BM * ES + 16);
+    if (ct > ring) ring = ct;
+    const size_t smem = (size_t)Cfg::BM * (d.K * ES + 16) + ring;
     static size_t configured = 0;
     if (smem > configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<T, NA>,
+        hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<T>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem,
                                              hipGetErrorString(e));
@@ -505,27 +453,9 @@ int launch_linear_na(const ffk_linear_desc& d, size_t smem, hipStream_t st) {
     }
     LinArgs a;
     a.d = d;
-    const int n_slabs = ffk_cdiv(d.M, LinCfg<T>::BM);
-    // persistent workgroups: as many as can be resident (LDS-limited), each walks slabs with stride gridDim
-    const int per_cu = (int)(160 * 1024 / (smem + 2048));
-    int resident = 256 * (per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu));   // 2 waves per SIMD (register budget)
-    dim3 grid(n_slabs < resident ? n_slabs : resident);
-    fused_linear_kernel<T, NA><<<grid, THREADS, smem, st>>>(a);
+    dim3 grid(ffk_cdiv(d.M, Cfg::BM));
+    fused_linear_kernel<T><<<grid, THREADS, smem, st>>>(a);
     return ffk_check_launch("ffk_fused_linear");
-}
-
-template <typename T>
-int launch_linear(const ffk_linear_desc& d, hipStream_t st) {
-    typedef LinCfg<T> Cfg;
-    constexpr int ES = sizeof(T);
-    const size_t smem = (size_t)Cfg::BM * (d.K * ES + 16) + (size_t)NT * (Cfg::KC * ES + 16);
-    // vectors of A per thread for a one-slab-ahead prefetch
-    const int vpr = d.K / (16 / ES);
-    int cs = 3;
-    while ((1 << cs) < vpr) ++cs;
-    const int n_it = Cfg::BM / (THREADS >> cs);
-    if (d.a_chanmajor || n_it > 8) return launch_linear_na<T, 0>(d, smem, st);
-    return launch_linear_na<T, 8>(d, smem, st);
 }
 
 }  // namespace
@@ -563,6 +493,17 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
                         "ffk_fused_linear: tile %d: gate alignment", i);
         }
     }
+    // Two kernel variants.  Launches whose tiles are all stored channel-contiguous (plain, gated,
+    // residual and q/k tiles) use the slab-persistent kernel (128-row slabs, register prefetch of the
+    // next slab and of whole weight tiles); launches with row-contiguous tiles (v / bias tiles,
+    // channel-major stores) use the 64-row kernel below, whose smaller LDS footprint keeps four
+    // workgroups per CU in flight and hides the longer store phase of those tiles.
+    bool all_c = d->dtype == FFK_BF16 && !d->a_chanmajor;
+    for (int i = 0; i < d->n_tiles; ++i) {
+        const ffk_tile& t = d->tiles[i];
+        all_c = all_c && ((t.kind == FFK_TILE_STRIDED && t.s_d == 1) || t.kind == FFK_TILE_QK);
+    }
+    if (all_c) return ffk_linear_slab_launch(d, (hipStream_t)stream);
     switch (d->dtype) {
         case FFK_BF16: return launch_linear<bf16_t>(*d, (hipStream_t)stream);
         case FFK_F32: return launch_linear<float>(*d, (hipStream_t)stream);

@@ -5,6 +5,7 @@
 // 16-byte vectors: each wave-level access covers whole 128-byte lines.  Reductions are
 // xor-shuffles inside the lane group; all arithmetic is fp32.
 #include "ffk_common.h"
+#include <stdlib.h>
 
 thread_local char ffk_err_buf[512] = "";
 
@@ -30,9 +31,15 @@ constexpr float MASK_FILL = -1e9f;
 struct RowGeom {
     int lpr, vpl;
 };
+static int env_int(const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : dflt;
+}
 static bool row_geom(long nvec, RowGeom* g) {
-    int lpr = 8;   // >= 8 lanes x 16 B: every wave-level access covers whole 128-byte lines
-    while (lpr < 64 && (long)lpr * 2 < nvec) lpr <<= 1;
+    static const int min_lpr = env_int("FFK_ROW_LPR", 8);
+    static const int tgt_vpl = env_int("FFK_ROW_VPL", 4);
+    int lpr = min_lpr;   // >= 8 lanes x 16 B: every wave-level access covers whole 128-byte lines
+    while (lpr < 64 && (long)lpr * tgt_vpl < nvec) lpr <<= 1;
     long vpl = (nvec + lpr - 1) / lpr;
     int v = 1;
     while (v < vpl) v <<= 1;
@@ -45,12 +52,12 @@ static bool row_geom(long nvec, RowGeom* g) {
 static int row_grid(long rows, int lpr) {
     long rows_per_block = (long)WAVES_PER_BLOCK * (64 / lpr);
     long blocks = (rows + rows_per_block - 1) / rows_per_block;
-    const long cap = 256L * 16;   // 256 CUs, up to 16 resident blocks each; grid-stride beyond
+    static const long cap = 256L * env_int("FFK_ROW_CAP", 16);   // 256 CUs x resident blocks; grid-stride beyond
     return (int)(blocks < cap ? blocks : cap);
 }
 
 // ------------------------------------------------------------------ softmax ----
-template <typename T, int VPL>
+template <typename T, int VPL, bool NTS>
 __global__ __launch_bounds__(BLOCK) void softmax_vec_kernel(T* out, const T* x,   // out may alias x
                                                            const T* __restrict__ mask,
                                                            const T* __restrict__ bias, long rows, int cols,
@@ -74,7 +81,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_vec_kernel(T* out, const T* x, 
         for (int i = 0; i < VPL; ++i) {
             const int vi = j + i * lpr;
             if (valid && vi < nvec) {
-                Vec16<T> xv = ld16(xr + vi * VEC);
+                Vec16<T> xv = NTS ? ld16_nt(xr + vi * VEC) : ld16(xr + vi * VEC);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) v[i][e] = DT<T>::to_f(xv.e[e]);
                 if (br) {
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_vec_kernel(T* out, const T* x, 
                 Vec16<T> ov;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) ov.e[e] = DT<T>::from_f(v[i][e] * inv);
-                st16(orow + vi * VEC, ov);
+                if (NTS) st16_nt(orow + vi * VEC, ov); else st16(orow + vi * VEC, ov);
             }
         }
     }
@@ -180,12 +187,13 @@ int softmax_launch(T* out, const T* x, const T* mask, const T* bias, long rows, 
                         (!mask || ffk_aligned16(mask)) && (!bias || ffk_aligned16(bias)) &&
                         row_geom(cols / VEC, &g);
     if (vec_ok) {
+        static const bool nts = env_int("FFK_ROW_NT", 1) != 0;
         dim3 grid(row_grid(rows, g.lpr));
         switch (g.vpl) {
-            case 1: softmax_vec_kernel<T, 1><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
-            case 2: softmax_vec_kernel<T, 2><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
-            case 4: softmax_vec_kernel<T, 4><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
-            default: softmax_vec_kernel<T, 8><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq); break;
+            case 1: (nts ? softmax_vec_kernel<T, 1, true><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq) : softmax_vec_kernel<T, 1, false><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq)); break;
+            case 2: (nts ? softmax_vec_kernel<T, 2, true><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq) : softmax_vec_kernel<T, 2, false><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq)); break;
+            case 4: (nts ? softmax_vec_kernel<T, 4, true><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq) : softmax_vec_kernel<T, 4, false><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq)); break;
+            default: (nts ? softmax_vec_kernel<T, 8, true><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq) : softmax_vec_kernel<T, 8, false><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq)); break;
         }
     } else {
         dim3 grid(row_grid(rows, 64));
@@ -195,7 +203,7 @@ int softmax_launch(T* out, const T* x, const T* mask, const T* bias, long rows, 
 }
 
 // ---------------------------------------------------------------- LayerNorm ----
-template <typename T, int VPL>
+template <typename T, int VPL, bool NTS>
 __global__ __launch_bounds__(BLOCK) void layernorm_vec_kernel(T* __restrict__ out, float* __restrict__ mean_o,
                                                              float* __restrict__ rstd_o, const T* __restrict__ x,
                                                              const T* __restrict__ gamma,
@@ -237,7 +245,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_vec_kernel(T* __restrict__ ou
         for (int i = 0; i < VPL; ++i) {
             const int vi = j + i * lpr;
             if (valid && vi < nvec) {
-                Vec16<T> xv = ld16(xr + vi * VEC);
+                Vec16<T> xv = NTS ? ld16_nt(xr + vi * VEC) : ld16(xr + vi * VEC);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     v[i][e] = DT<T>::to_f(xv.e[e]);
@@ -271,7 +279,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_vec_kernel(T* __restrict__ ou
                 Vec16<T> ov;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) ov.e[e] = DT<T>::from_f((v[i][e] - mu) * rs * gm[i][e] + bt[i][e]);
-                st16(orow + vi * VEC, ov);
+                if (NTS) st16_nt(orow + vi * VEC, ov); else st16(orow + vi * VEC, ov);
             }
         }
         if (valid && j == 0) {
@@ -375,12 +383,13 @@ int layernorm_launch(T* out, float* mean, float* rstd, const T* x, const T* gamm
     const bool vec_ok = cols % VEC == 0 && ffk_aligned16(out) && ffk_aligned16(x) && ffk_aligned16(gamma) &&
                         ffk_aligned16(beta) && row_geom(cols / VEC, &g);
     if (vec_ok) {
+        static const bool nts = env_int("FFK_ROW_NT", 1) != 0;
         dim3 grid(row_grid(rows, g.lpr));
         switch (g.vpl) {
-            case 1: layernorm_vec_kernel<T, 1><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
-            case 2: layernorm_vec_kernel<T, 2><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
-            case 4: layernorm_vec_kernel<T, 4><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
-            default: layernorm_vec_kernel<T, 8><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps); break;
+            case 1: (nts ? layernorm_vec_kernel<T, 1, true><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps) : layernorm_vec_kernel<T, 1, false><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps)); break;
+            case 2: (nts ? layernorm_vec_kernel<T, 2, true><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps) : layernorm_vec_kernel<T, 2, false><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps)); break;
+            case 4: (nts ? layernorm_vec_kernel<T, 4, true><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps) : layernorm_vec_kernel<T, 4, false><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps)); break;
+            default: (nts ? layernorm_vec_kernel<T, 8, true><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps) : layernorm_vec_kernel<T, 8, false><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps)); break;
         }
     } else {
         dim3 grid(row_grid(rows, 64));
