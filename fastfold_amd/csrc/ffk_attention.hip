@@ -1,10 +1,9 @@
 // Flash-style attention for head dimension 32 (see ffk_attention_fwd in include/ffk.h).
 //
-// One wavefront owns 32 queries of one (b2, head) and walks the keys 32 at a time; the
-// four waves of a workgroup take consecutive query tiles of the same (b2, head), so their
-// K / V tile reads hit the same lines.  There is no LDS and no barrier: every operand is
-// stored in HBM in exactly the order a wave consumes it (1024-element tiles, 16 contiguous
-// elements per lane).
+// One wavefront owns 32 queries of one (b2, head) and walks the keys 32 at a time.  Every
+// operand is stored in HBM in exactly the order a wave consumes it (1024-element tiles, 16
+// contiguous elements per lane); the eight waves of a workgroup share their operand tiles
+// through a double-buffered LDS stage (see attention_kernel).
 //
 // The score tile is computed transposed, S^T = K . Q^T (rows = keys, columns = queries):
 // a lane then holds 16 keys of ONE query, so the running max / sum are per-lane scalars
@@ -65,31 +64,67 @@ __device__ __forceinline__ typename Mma<T>::Frag identity_frag(int i, int l32, i
     return f;
 }
 
+// Workgroup = 8 wavefronts = 2 batch rows x 4 query tiles of one head.  Per 32-key step the
+// workgroup needs the K and V tiles of its two batch rows and the bias tiles of its four query
+// tiles: 8 operand tiles, each consumed by 4 (K, V) or 2 (bias) waves.  They are fetched from
+// global memory once per workgroup (two 16-byte loads per thread), double-buffered in LDS, and read
+// from there by the waves in exactly the lane order of the MFMA operands, which divides the
+// traffic through the vector memory path by three compared with per-wave global loads.
+constexpr int ATT_WAVES = 8;
+constexpr int ATT_THREADS = 64 * ATT_WAVES;
+
 template <typename T, bool HAS_BIAS>
-__global__ __launch_bounds__(THREADS, sizeof(T) == 2 ? 3 : 2) void attention_kernel(T* __restrict__ out, const T* __restrict__ q_t,
-                                                              const T* __restrict__ k_t, const T* __restrict__ v_t,
-                                                              const T* __restrict__ bias_t,
-                                                              const float* __restrict__ keybias,
-                                                              const int* __restrict__ tileflags,
-                                                              const T* __restrict__ gate, int H, int Nq, int Nk) {
+__global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention_kernel(
+    T* __restrict__ out, const T* __restrict__ q_t, const T* __restrict__ k_t, const T* __restrict__ v_t,
+    const T* __restrict__ bias_t, const float* __restrict__ keybias, const int* __restrict__ tileflags,
+    const T* __restrict__ gate, int B2, int H, int Nq, int Nk) {
     typedef Mma<T> MM;
     typedef typename MM::Frag Frag;
     constexpr int NF = 16 / MM::KLANE;            // fragments per 16-element lane slice (bf16 2, fp32 4)
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int VEC = DT<T>::VEC;
+    constexpr int NTILES = HAS_BIAS ? 8 : 4;      // operand tiles per key step: K0 K1 V0 V1 [B0 B1 B2 B3]
+    constexpr int TILE_VECS = 1024 / VEC;         // 16-byte vectors per tile
+    constexpr int NVL = (NTILES * TILE_VECS + ATT_THREADS - 1) / ATT_THREADS;   // vectors per thread per step
+    extern __shared__ __align__(16) unsigned char att_smem[];
+    T* lds = reinterpret_cast<T*>(att_smem);      // [2][NTILES][1024]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
+    const int bsel = wave >> 2, qsel = wave & 3;
     const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
-    const int qt = blockIdx.x * 4 + wave;
-    if (qt >= QT) return;
-    const int h = blockIdx.y, b2 = blockIdx.z;
+    const int h = blockIdx.y;
+    const int b2_raw = blockIdx.z * 2 + bsel, qt_raw = blockIdx.x * 4 + qsel;
+    const bool live = b2_raw < B2 && qt_raw < QT;      // dead waves still help loading and keep the barriers
+    const int b2 = b2_raw < B2 ? b2_raw : B2 - 1;
+    const int qt = qt_raw < QT ? qt_raw : QT - 1;
     const long bh = (long)b2 * H + h;
 
     Ops16<T> qf;
     qf.load(q_t + ((bh * QT + qt) << 10) + lane * 16);
-    const T* kp = k_t + ((bh * KT) << 10) + lane * 16;
-    const T* vp = v_t + ((bh * KT) << 10) + lane * 16;
-    const T* bp = HAS_BIAS ? bias_t + ((((long)h * QT + qt) * KT) << 10) + lane * 16 : nullptr;
     const float* mp = keybias + (long)b2 * KT * 32 + 4 * half;
     const int* fl = tileflags + (long)b2 * KT;
+
+    // cooperative operand fetch: vector slot v = tid + i * ATT_THREADS -> (tile, vector in tile)
+    const T* src[NVL];
+    int dst[NVL];
+#pragma unroll
+    for (int i = 0; i < NVL; ++i) {
+        int v = tid + i * ATT_THREADS;
+        v = v < NTILES * TILE_VECS ? v : NTILES * TILE_VECS - 1;
+        const int tile = v / TILE_VECS, wv = v % TILE_VECS;
+        const T* base;
+        if (tile < 4) {
+            int bb = blockIdx.z * 2 + (tile & 1);
+            bb = bb < B2 ? bb : B2 - 1;
+            base = (tile < 2 ? k_t : v_t) + ((((long)bb * H + h) * KT) << 10);
+        } else {
+            int qq = blockIdx.x * 4 + (tile - 4);
+            qq = qq < QT ? qq : QT - 1;
+            base = bias_t + ((((long)h * QT + qq) * KT) << 10);
+        }
+        src[i] = base + wv * VEC;
+        dst[i] = tile * 1024 + wv * VEC;
+    }
 
     // gate values of this lane's 16 outputs, fetched now so that their latency is hidden by the loop
     const int q = qt * 32 + l32;
@@ -107,9 +142,13 @@ __global__ __launch_bounds__(THREADS, sizeof(T) == 2 ? 3 : 2) void attention_ker
         }
     }
 
-    // trailing key tiles that are completely masked (sequence padding) contribute exactly zero
+    // trailing key tiles that are completely masked in both batch rows contribute exactly zero
     int kt_end = KT;
-    while (kt_end > 1 && fl[kt_end - 1] == 2) --kt_end;
+    {
+        const int* f0 = tileflags + (long)(blockIdx.z * 2 < B2 ? blockIdx.z * 2 : B2 - 1) * KT;
+        const int* f1 = tileflags + (long)(blockIdx.z * 2 + 1 < B2 ? blockIdx.z * 2 + 1 : B2 - 1) * KT;
+        while (kt_end > 1 && f0[kt_end - 1] == 2 && f1[kt_end - 1] == 2) --kt_end;
+    }
 
     Frag ident[NF];
     if (HAS_BIAS) {
@@ -122,24 +161,39 @@ __global__ __launch_bounds__(THREADS, sizeof(T) == 2 ? 3 : 2) void attention_ker
     // first MFMA of each tile, so the accumulator already holds  s - m_ref  and exp2 is applied to it
     // directly.  m_ref is only moved (and O / l rescaled) when a tile contains a score more than
     // REF_SLACK above it, which bounds  p = exp2(s - m_ref) <= 2^REF_SLACK;  the first tile always
-    // sets it.  The row sum l is accumulated on the matrix pipe as well (ones . P^T).
+    // sets it.
     constexpr float REF_SLACK = 20.0f;
     constexpr float REF_FLOOR = -1.0e4f;          // keeps m_ref small when the first tile is fully masked
-    f32x16 o_acc, l_acc, negm;
+    f32x16 o_acc, negm;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) o_acc[v] = l_acc[v] = negm[v] = 0.0f;
+    for (int v = 0; v < 16; ++v) o_acc[v] = negm[v] = 0.0f;
+    float l_run = 0.0f;                           // partial row sum of this lane's 16 keys per tile
     bool first = true;
-    Frag ones;
-#pragma unroll
-    for (int t = 0; t < MM::KLANE; ++t) ones[t] = (T)1.0f;
 
-    auto load_tile = [&](int kt, Ops16<T>& kk, Ops16<T>& vv, Ops16<T>& bb) {
-        kk.load(kp + ((long)kt << 10));
-        vv.load(vp + ((long)kt << 10));
-        if (HAS_BIAS) bb.load(bp + ((long)kt << 10));
+    Vec16<T> pre[NVL];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < NVL; ++i) pre[i] = ld16(src[i] + ((long)kt << 10));
+    };
+    auto commit = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < NVL; ++i)
+            if (tid + i * ATT_THREADS < NTILES * TILE_VECS)
+                *reinterpret_cast<Vec16<T>*>(lds + slot * NTILES * 1024 + dst[i]) = pre[i];
     };
 
-    auto process = [&](int kt, const Ops16<T>& kc, const Ops16<T>& vc, const Ops16<T>& bc) {
+    fetch(0);
+    commit(0);
+    for (int kt = 0; kt < kt_end; ++kt) {
+        lds_barrier();                            // tile kt is in LDS; nobody still reads the other slot
+        const int nxt = kt + 1 < kt_end ? kt + 1 : kt;
+        fetch(nxt);                               // in flight during the MFMAs below
+        const T* buf = lds + (kt & 1) * NTILES * 1024;
+        Ops16<T> kc, vc, bc;
+        kc.load(buf + bsel * 1024 + lane * 16);
+        vc.load(buf + (2 + bsel) * 1024 + lane * 16);
+        if (HAS_BIAS) bc.load(buf + (4 + qsel) * 1024 + lane * 16);
+
         // S^T - m_ref = K . Q^T + Bias^T . I + (-m_ref)   (rows: keys, columns: queries)
         f32x16 s = negm;
 #pragma unroll
@@ -171,41 +225,28 @@ __global__ __launch_bounds__(THREADS, sizeof(T) == 2 ? 3 : 2) void attention_ker
                 negm[v] -= delta;
                 o_acc[v] *= alpha;
             }
-            l_acc[0] *= alpha;
+            l_run *= alpha;
             first = false;
         }
         float p[16];
+        float ls = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) p[v] = fast_exp2(s[v]);
-        // O^T += V^T . P^T  and  l += 1 . P^T   (rows: head dim, columns: queries)
-#pragma unroll
-        for (int i = 0; i < NF; ++i) {
-            const Frag pf = PFrag<T>::make(p + i * MM::KLANE);
-            MM::mma(o_acc, vc.frag(i), pf);
-            MM::mma(l_acc, ones, pf);
+        for (int v = 0; v < 16; ++v) {
+            p[v] = fast_exp2(s[v]);
+            ls += p[v];
         }
-    };
+        l_run += ls;
+        // O^T += V^T . P^T   (rows: head dim, columns: queries)
+#pragma unroll
+        for (int i = 0; i < NF; ++i) MM::mma(o_acc, vc.frag(i), PFrag<T>::make(p + i * MM::KLANE));
 
-    // Software pipeline over two register sets used alternately (no copies).  Every prefetch is
-    // unconditional (the tile index is clamped instead), which keeps the loop free of branches
-    // around loads so the compiler can wait for exactly the tile it needs.
-    Ops16<T> ka, va, ba, kb, vb, bb;
-    const int last = kt_end - 1;
-    const int n2 = kt_end & ~1;
-    load_tile(0, ka, va, ba);
-    for (int kt = 0; kt < n2; kt += 2) {
-        load_tile(kt + 1, kb, vb, bb);
-        process(kt, ka, va, ba);
-        load_tile(kt + 2 < last ? kt + 2 : last, ka, va, ba);
-        process(kt + 1, kb, vb, bb);
+        commit((kt + 1) & 1);                     // the slot last read in step kt - 1
     }
-    if (kt_end & 1) process(last, ka, va, ba);
 
-    // every row of l_acc holds the full row sum (the MFMA already summed both lane halves); rows whose
-    // keys are all masked have l == 0 and produce zeros
-    const float l_tot = l_acc[0];
+    // rows whose keys are all masked have l == 0 and produce zeros
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    if (q < Nq) {
+    if (live && q < Nq) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             T r4[4];
@@ -244,17 +285,30 @@ __global__ void key_bias_kernel(float* kb, int* flags, const T* mask, long N, lo
     }
 }
 
+template <typename T, bool HAS_BIAS>
+int launch_attention_b(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
+                       const int* flags, const void* gate, long B2, long H, long Nq, long Nk, hipStream_t st) {
+    const size_t smem = 2 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 * sizeof(T);
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)attention_kernel<T, HAS_BIAS>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_attention_fwd: cannot reserve %zu B of LDS: %s", smem,
+                                             hipGetErrorString(e));
+        configured = true;
+    }
+    dim3 grid(ffk_cdiv((Nq + 31) / 32, 4), (unsigned)H, (unsigned)ffk_cdiv(B2, 2));
+    attention_kernel<T, HAS_BIAS><<<grid, ATT_THREADS, smem, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
+                                                                  (const T*)bias, kb, flags, (const T*)gate, (int)B2,
+                                                                  (int)H, (int)Nq, (int)Nk);
+    return ffk_check_launch("ffk_attention_fwd");
+}
+
 template <typename T>
 int launch_attention(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
                      const int* flags, const void* gate, long B2, long H, long Nq, long Nk, hipStream_t st) {
-    dim3 grid(ffk_cdiv((Nq + 31) / 32, 4), (unsigned)H, (unsigned)B2);
-    if (bias)
-        attention_kernel<T, true><<<grid, THREADS, 0, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
-                                                          (const T*)bias, kb, flags, (const T*)gate, (int)H, (int)Nq, (int)Nk);
-    else
-        attention_kernel<T, false><<<grid, THREADS, 0, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v, nullptr,
-                                                           kb, flags, (const T*)gate, (int)H, (int)Nq, (int)Nk);
-    return ffk_check_launch("ffk_attention_fwd");
+    return bias ? launch_attention_b<T, true>(out, q, k, v, bias, kb, flags, gate, B2, H, Nq, Nk, st)
+                : launch_attention_b<T, false>(out, q, k, v, nullptr, kb, flags, gate, B2, H, Nq, Nk, st);
 }
 
 }  // namespace
@@ -263,7 +317,7 @@ extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, co
                                  const float* keybias, const int32_t* tileflags, const void* gate, int64_t B2, int64_t H, int64_t Nq,
                                  int64_t Nk, int dtype, void* stream) {
     FFK_REQUIRE(out && q_t && k_t && v_t && keybias && tileflags, FFK_ERR_NULL, "ffk_attention_fwd: null pointer");
-    FFK_REQUIRE(B2 > 0 && B2 < 65536 && H > 0 && H < 65536 && Nq > 0 && Nk > 0 && Nq < (1 << 24) && Nk < (1 << 24),
+    FFK_REQUIRE(B2 > 0 && B2 < 131072 && H > 0 && H < 65536 && Nq > 0 && Nk > 0 && Nq < (1 << 24) && Nk < (1 << 24),
                 FFK_ERR_SHAPE, "ffk_attention_fwd: bad shape B2=%ld H=%ld Nq=%ld Nk=%ld", (long)B2, (long)H, (long)Nq,
                 (long)Nk);
     FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(q_t) && ffk_aligned16(k_t) && ffk_aligned16(v_t) &&
