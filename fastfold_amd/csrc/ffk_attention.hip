@@ -42,6 +42,18 @@ template <> struct PFrag<bf16_t> {
         for (int t = 0; t < 8; ++t) r[t] = (bf16_t)p[t];
         return r;
     }
+    // acc + sum of the eight rounded probabilities (the values the PV product really uses), two
+    // per instruction
+    static __device__ __forceinline__ float add_sum(const bf16x8& f, float acc) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const bf16x2 pr = {f[2 * t], f[2 * t + 1]};
+            acc = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, acc, false);
+        }
+        return acc;
+    }
 };
 template <> struct PFrag<float> {
     static __device__ __forceinline__ f32x4 make(const float* p) {
@@ -49,6 +61,9 @@ template <> struct PFrag<float> {
 #pragma unroll
         for (int t = 0; t < 4; ++t) r[t] = p[t];
         return r;
+    }
+    static __device__ __forceinline__ float add_sum(const f32x4& f, float acc) {
+        return acc + ((f[0] + f[1]) + (f[2] + f[3]));
     }
 };
 
@@ -92,8 +107,17 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     const int l32 = lane & 31, half = lane >> 5;
     const int bsel = wave >> 2, qsel = wave & 3;
     const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
-    const int h = blockIdx.y;
-    const int b2_raw = blockIdx.z * 2 + bsel, qt_raw = blockIdx.x * 4 + qsel;
+    // Workgroup -> work mapping.  The hardware hands consecutive workgroup ids to the eight XCDs in
+    // turn, and each XCD has its own L2.  Logical work items are ordered (head, batch-row pair,
+    // query group) and every XCD takes one contiguous eighth of that order, so that the query groups
+    // that share a K / V pair and the batch rows that share a head's bias run behind the same L2.
+    const int NQG = (QT + 3) >> 2, NZ = (B2 + 1) >> 1;
+    const unsigned total = (unsigned)NQG * H * NZ, per_xcd = (total + 7) >> 3;
+    const unsigned item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (item >= total) return;                    // whole workgroup leaves together
+    const int wg_q = item % NQG, wg_z = (item / NQG) % NZ;
+    const int h = (item / NQG) / NZ;
+    const int b2_raw = wg_z * 2 + bsel, qt_raw = wg_q * 4 + qsel;
     const bool live = b2_raw < B2 && qt_raw < QT;      // dead waves still help loading and keep the barriers
     const int b2 = b2_raw < B2 ? b2_raw : B2 - 1;
     const int qt = qt_raw < QT ? qt_raw : QT - 1;
@@ -114,11 +138,11 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
         const int tile = v / TILE_VECS, wv = v % TILE_VECS;
         const T* base;
         if (tile < 4) {
-            int bb = blockIdx.z * 2 + (tile & 1);
+            int bb = wg_z * 2 + (tile & 1);
             bb = bb < B2 ? bb : B2 - 1;
             base = (tile < 2 ? k_t : v_t) + ((((long)bb * H + h) * KT) << 10);
         } else {
-            int qq = blockIdx.x * 4 + (tile - 4);
+            int qq = wg_q * 4 + (tile - 4);
             qq = qq < QT ? qq : QT - 1;
             base = bias_t + ((((long)h * QT + qq) * KT) << 10);
         }
@@ -145,8 +169,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     // trailing key tiles that are completely masked in both batch rows contribute exactly zero
     int kt_end = KT;
     {
-        const int* f0 = tileflags + (long)(blockIdx.z * 2 < B2 ? blockIdx.z * 2 : B2 - 1) * KT;
-        const int* f1 = tileflags + (long)(blockIdx.z * 2 + 1 < B2 ? blockIdx.z * 2 + 1 : B2 - 1) * KT;
+        const int* f0 = tileflags + (long)(wg_z * 2 < B2 ? wg_z * 2 : B2 - 1) * KT;
+        const int* f1 = tileflags + (long)(wg_z * 2 + 1 < B2 ? wg_z * 2 + 1 : B2 - 1) * KT;
         while (kt_end > 1 && f0[kt_end - 1] == 2 && f1[kt_end - 1] == 2) --kt_end;
     }
 
@@ -184,10 +208,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
 
     fetch(0);
     commit(0);
+    int flag_nxt = fl[0];
     for (int kt = 0; kt < kt_end; ++kt) {
+        // the tile's mask flag was fetched one step ahead, so that its latency is never exposed
+        const int flag = __builtin_amdgcn_readfirstlane(flag_nxt);
         lds_barrier();                            // tile kt is in LDS; nobody still reads the other slot
         const int nxt = kt + 1 < kt_end ? kt + 1 : kt;
         fetch(nxt);                               // in flight during the MFMAs below
+        flag_nxt = fl[nxt];
         const T* buf = lds + (kt & 1) * NTILES * 1024;
         Ops16<T> kc, vc, bc;
         kc.load(buf + bsel * 1024 + lane * 16);
@@ -202,7 +230,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
 #pragma unroll
             for (int i = 0; i < NF; ++i) MM::mma(s, bc.frag(i), ident[i]);
         }
-        if (fl[kt] != 0) {           // some key of this tile is masked or padding: add the key bias
+        if (flag != 0) {             // some key of this tile is masked or padding: add the key bias
             f32x4 mk[4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) mk[g] = *reinterpret_cast<const f32x4*>(mp + kt * 32 + 8 * g);
@@ -229,16 +257,15 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
             first = false;
         }
         float p[16];
-        float ls = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            p[v] = fast_exp2(s[v]);
-            ls += p[v];
-        }
-        l_run += ls;
+        for (int v = 0; v < 16; ++v) p[v] = fast_exp2(s[v]);
         // O^T += V^T . P^T   (rows: head dim, columns: queries)
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(o_acc, vc.frag(i), PFrag<T>::make(p + i * MM::KLANE));
+        for (int i = 0; i < NF; ++i) {
+            const Frag pf = PFrag<T>::make(p + i * MM::KLANE);
+            l_run = PFrag<T>::add_sum(pf, l_run);
+            MM::mma(o_acc, vc.frag(i), pf);
+        }
 
         commit((kt + 1) & 1);                     // the slot last read in step kt - 1
     }
@@ -297,7 +324,9 @@ int launch_attention_b(void* out, const void* q, const void* k, const void* v, c
                                              hipGetErrorString(e));
         configured = true;
     }
-    dim3 grid(ffk_cdiv((Nq + 31) / 32, 4), (unsigned)H, (unsigned)ffk_cdiv(B2, 2));
+    const long items = (long)ffk_cdiv((Nq + 31) / 32, 4) * H * ffk_cdiv(B2, 2);
+    FFK_REQUIRE(items < (1L << 31) - 8, FFK_ERR_SHAPE, "ffk_attention_fwd: %ld workgroups exceed the grid limit", items);
+    dim3 grid((unsigned)(8 * ffk_cdiv(items, 8)));
     attention_kernel<T, HAS_BIAS><<<grid, ATT_THREADS, smem, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
                                                                   (const T*)bias, kb, flags, (const T*)gate, (int)B2,
                                                                   (int)H, (int)Nq, (int)Nk);
