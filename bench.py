@@ -24,10 +24,16 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
 
+# "attn_traffic": HBM bytes per launch of the biased attention kernel, averaged over the launches the
+# roofline object covers (2 triangle : 1 MSA-row per block).  It comes from rocprofv3 --pmc FETCH_SIZE
+# and WRITE_SIZE runs of this script (profiles/evoformer_blocks_cfg4_hbm_traffic.txt: counters scaled by
+# 2.0 / 1.0 after calibration on a plain streaming kernel); counters cannot be read inside a timed run.
 WORKLOADS = {
-    "cfg3": dict(n_seq=128, n_res=256, tail=0.0, name="configs[2]: 48-block stack bf16 N_seq=128 N_res=256"),
+    "cfg3": dict(n_seq=128, n_res=256, tail=0.0, name="configs[2]: 48-block stack bf16 N_seq=128 N_res=256",
+                 attn_traffic=None),
     "cfg4": dict(n_seq=128, n_res=1024, tail=0.05,
-                 name="configs[3]: 48-block stack bf16 N_seq=128 N_res=1024, last 5% of residues masked"),
+                 name="configs[3]: 48-block stack bf16 N_seq=128 N_res=1024, last 5% of residues masked",
+                 attn_traffic=1.785e9),
 }
 
 
@@ -198,7 +204,8 @@ def main():
     ach = flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
     roofline = {"bound": "mfma", "kernel": "attention_kernel<bf16, bias> (ffk_attention_fwd)",
                 "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": wl["attn_traffic"],
+                "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, see profiles/)",
                 "launches": n, "avg_launch_ms": round(ms / max(n, 1), 4),
                 "flops_per_launch_avg": round(flops / max(n, 1) / 1e9, 2)}
 
