@@ -1,0 +1,60 @@
+"""``fused_attention_core`` with the reference's interface
+(fastfold/model/fastnn/kernel/attention_core.py:17-52):
+
+    softmax(q * d**-0.5 @ k^T + bias + BIG * (mask - 1)) @ v   ->   [b1, b2, n, h*d]
+
+for q, k, v ``[b1, b2, h, n, d]``, mask ``[b1, b2, n]`` (0/1, over keys) and bias ``[b1, h, n, n]``.
+The logits are never materialised: the operands are re-tiled into the 32x32 MFMA order and handed to
+the flash attention kernel (``ffk_attention_fwd``).  Forward only, like the reference.  The kernel is
+specialised for the Evoformer's head dim (32); other head dims raise ``RuntimeError``.
+"""
+import math
+
+import torch
+
+from .... import _lib
+from . import layouts
+
+
+def _attention_core(q, k, v, mask=None, bias=None):
+    _lib.check_device(q, k, v, mask, bias)
+    if q.dim() != 5 or q.shape != k.shape or q.shape != v.shape:
+        raise RuntimeError("fused_attention_core: q, k, v must be [b1, b2, h, n, d] of one shape, got %s %s %s"
+                           % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    b1, b2, h, n, d = q.shape
+    if d != 32:
+        raise RuntimeError("fused_attention_core: head dim %d is not supported (the kernel is built for 32)" % d)
+    if mask is not None and tuple(mask.shape) != (b1, b2, n):
+        raise RuntimeError("fused_attention_core: mask must be [b1, b2, n], got %s" % (tuple(mask.shape),))
+    if bias is not None and tuple(bias.shape) != (b1, h, n, n):
+        raise RuntimeError("fused_attention_core: bias must be [b1, h, n, n], got %s" % (tuple(bias.shape),))
+    out = torch.empty(b1, b2, n, h * d, dtype=q.dtype, device=q.device)
+    if out.numel() == 0:
+        return out
+    nt = layouts.n_tiles(n)
+    scale = _lib.LOG2E / math.sqrt(d)            # the kernel exponentiates in base 2
+    kb = torch.empty(b2, nt * 32, dtype=torch.float32, device=q.device)
+    fl = torch.empty(b2, nt, dtype=torch.int32, device=q.device)
+    for i in range(b1):
+        mk = mask[i].to(q.dtype).contiguous() if mask is not None else torch.ones(b2, n, dtype=q.dtype, device=q.device)
+        _lib.key_bias(kb, fl, mk, B=b2, N=n, mask_sb=n, mask_sn=1)
+        qt = layouts.tile_qk((q[i].float() * scale).to(q.dtype))
+        bt = layouts.tile_bias((bias[i].float() * _lib.LOG2E).to(q.dtype)) if bias is not None else None
+        _lib.attention_fwd(out[i].view(b2 * n, h * d), qt, layouts.tile_qk(k[i]), layouts.tile_v(v[i]), bt, kb, fl,
+                           None, B2=b2, H=h, Nq=n, Nk=n)
+    return out
+
+
+class FusedAttenionCoreFunc(torch.autograd.Function):
+    """Name (including its spelling) as in the reference (attention_core.py:34)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, mask=None, bias=None):
+        return _attention_core(q, k, v, mask, bias)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("fused_attention_core is forward-only, as in the reference")
+
+
+fused_attention_core = FusedAttenionCoreFunc.apply

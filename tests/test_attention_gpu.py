@@ -144,3 +144,24 @@ def test_bgemm_outer_product_and_projection(dev, dtype, tol, s, r):
     nrm = torch.empty(r, r, dtype=torch.float32, device=dev)
     _lib.bgemm_nt(mk, mk, nrm, M=r, N=r, K=spad, lda=spad, ldb=spad, out_f32=True)
     assert np.array_equal(_np(nrm), _np(mk) @ _np(mk).T)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("b1,b2,h,n", [(1, 3, 4, 77), (2, 2, 8, 64)])
+def test_fused_attention_core_op(dev, dtype, tol, b1, b2, h, n):
+    """The exported op against the textbook formula the reference tests it with
+    (tests/test_fastnn/test_attention_core.py:16-31)."""
+    from fastfold_amd.model.fastnn.kernel import fused_attention_core
+    g = torch.Generator().manual_seed(b2 * n)
+    q, k, v = (torch.randn(b1, b2, h, n, 32, generator=g).to(dev, dtype) for _ in range(3))
+    bias = torch.randn(b1, h, n, n, generator=g).to(dev, dtype)
+    mask = (torch.rand(b1, b2, n, generator=g) > 0.25).to(dev, dtype)
+    mask[..., 0] = 1
+    out = fused_attention_core(q, k, v, mask, bias)
+    assert out.shape == (b1, b2, n, h * 32) and out.dtype == dtype
+    ref = ops_np.attention_core(_np(q), _np(k), _np(v), _np(mask), _np(bias))
+    assert _rel(_np(out), ref) < tol
+    with pytest.raises(RuntimeError):
+        fused_attention_core(q[..., :16].contiguous(), k[..., :16].contiguous(), v[..., :16].contiguous(), mask, bias)
+    with pytest.raises(RuntimeError):
+        fused_attention_core(q.cpu(), k.cpu(), v.cpu(), mask.cpu(), bias.cpu())
