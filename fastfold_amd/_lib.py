@@ -121,7 +121,7 @@ def call(name: str, *args):
 
 
 # ------------------------------------------------------------------ fused linear ----
-FFK_TILE_STRIDED, FFK_TILE_QK, FFK_TILE_V, FFK_TILE_BIAS = 0, 1, 2, 3
+FFK_TILE_STRIDED, FFK_TILE_QK, FFK_TILE_V, FFK_TILE_BIAS, FFK_TILE_ACC = 0, 1, 2, 3, 4
 FFK_ACT_NONE, FFK_ACT_RELU, FFK_ACT_SIGMOID = 0, 1, 2
 FFK_MAX_TILES = 10
 LOG2E = 1.4426950408889634
@@ -209,7 +209,7 @@ class BgemmDesc(ctypes.Structure):
 
 
 SIGNATURES["ffk_bgemm_nt"] = [ctypes.POINTER(BgemmDesc), _P]
-SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _I, _P]
+SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P]
 SIGNATURES["ffk_key_bias"] = [_P, _P, _P, _L, _L, _L, _L, _I, _P]
 
 
@@ -230,10 +230,13 @@ def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, i
     call("ffk_bgemm_nt", ctypes.byref(d), stream_ptr())
 
 
-def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H, Nq, Nk):
+FFK_ATT_GATE_TILED = 1
+
+
+def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H, Nq, Nk, gate_tiled=False):
     call("ffk_attention_fwd", ptr(out), ptr(q_t), ptr(k_t), ptr(v_t), ptr(bias_t), ptr(keybias), ptr(tileflags),
          ptr(gate),
-         B2, H, Nq, Nk, dtype_tag(q_t.dtype), stream_ptr())
+         B2, H, Nq, Nk, FFK_ATT_GATE_TILED if gate_tiled else 0, dtype_tag(q_t.dtype), stream_ptr())
 
 
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):

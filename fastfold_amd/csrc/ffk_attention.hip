@@ -92,7 +92,7 @@ template <typename T, bool HAS_BIAS>
 __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention_kernel(
     T* __restrict__ out, const T* __restrict__ q_t, const T* __restrict__ k_t, const T* __restrict__ v_t,
     const T* __restrict__ bias_t, const float* __restrict__ keybias, const int* __restrict__ tileflags,
-    const T* __restrict__ gate, int B2, int H, int Nq, int Nk) {
+    const T* __restrict__ gate, int B2, int H, int Nq, int Nk, int flags) {
     typedef Mma<T> MM;
     typedef typename MM::Frag Frag;
     constexpr int NF = 16 / MM::KLANE;            // fragments per 16-element lane slice (bf16 2, fp32 4)
@@ -156,12 +156,24 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     const long rowo = ((long)b2 * Nq + qc) * (H * 32) + h * 32 + 4 * half;
     T gv[4][4];
     if (gate) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
+        if (flags & FFK_ATT_GATE_TILED) {
+            // accumulator-order tile: this lane's 16 values are contiguous
+            const T* gp = gate + ((bh * QT + qt) << 10) + lane * 16;
             if (sizeof(T) == 2) {
-                *reinterpret_cast<u32x2*>(&gv[g][0]) = *reinterpret_cast<const u32x2*>(gate + rowo + 8 * g);
+                *reinterpret_cast<u32x4*>(&gv[0][0]) = *reinterpret_cast<const u32x4*>(gp);
+                *reinterpret_cast<u32x4*>(&gv[2][0]) = *reinterpret_cast<const u32x4*>(gp + 8);
             } else {
-                *reinterpret_cast<u32x4*>(&gv[g][0]) = *reinterpret_cast<const u32x4*>(gate + rowo + 8 * g);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) *reinterpret_cast<u32x4*>(&gv[g][0]) = *reinterpret_cast<const u32x4*>(gp + 4 * g);
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                if (sizeof(T) == 2) {
+                    *reinterpret_cast<u32x2*>(&gv[g][0]) = *reinterpret_cast<const u32x2*>(gate + rowo + 8 * g);
+                } else {
+                    *reinterpret_cast<u32x4*>(&gv[g][0]) = *reinterpret_cast<const u32x4*>(gate + rowo + 8 * g);
+                }
             }
         }
     }
@@ -314,7 +326,7 @@ __global__ void key_bias_kernel(float* kb, int* flags, const T* mask, long N, lo
 
 template <typename T, bool HAS_BIAS>
 int launch_attention_b(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
-                       const int* flags, const void* gate, long B2, long H, long Nq, long Nk, hipStream_t st) {
+                       const int* flags, const void* gate, long B2, long H, long Nq, long Nk, int aflags, hipStream_t st) {
     const size_t smem = 2 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 * sizeof(T);
     static bool configured = false;
     if (!configured) {
@@ -329,22 +341,22 @@ int launch_attention_b(void* out, const void* q, const void* k, const void* v, c
     dim3 grid((unsigned)(8 * ffk_cdiv(items, 8)));
     attention_kernel<T, HAS_BIAS><<<grid, ATT_THREADS, smem, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
                                                                   (const T*)bias, kb, flags, (const T*)gate, (int)B2,
-                                                                  (int)H, (int)Nq, (int)Nk);
+                                                                  (int)H, (int)Nq, (int)Nk, aflags);
     return ffk_check_launch("ffk_attention_fwd");
 }
 
 template <typename T>
 int launch_attention(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
-                     const int* flags, const void* gate, long B2, long H, long Nq, long Nk, hipStream_t st) {
-    return bias ? launch_attention_b<T, true>(out, q, k, v, bias, kb, flags, gate, B2, H, Nq, Nk, st)
-                : launch_attention_b<T, false>(out, q, k, v, nullptr, kb, flags, gate, B2, H, Nq, Nk, st);
+                     const int* flags, const void* gate, long B2, long H, long Nq, long Nk, int aflags, hipStream_t st) {
+    return bias ? launch_attention_b<T, true>(out, q, k, v, bias, kb, flags, gate, B2, H, Nq, Nk, aflags, st)
+                : launch_attention_b<T, false>(out, q, k, v, nullptr, kb, flags, gate, B2, H, Nq, Nk, aflags, st);
 }
 
 }  // namespace
 
 extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t, const void* bias_t,
                                  const float* keybias, const int32_t* tileflags, const void* gate, int64_t B2, int64_t H, int64_t Nq,
-                                 int64_t Nk, int dtype, void* stream) {
+                                 int64_t Nk, int flags, int dtype, void* stream) {
     FFK_REQUIRE(out && q_t && k_t && v_t && keybias && tileflags, FFK_ERR_NULL, "ffk_attention_fwd: null pointer");
     FFK_REQUIRE(B2 > 0 && B2 < 131072 && H > 0 && H < 65536 && Nq > 0 && Nk > 0 && Nq < (1 << 24) && Nk < (1 << 24),
                 FFK_ERR_SHAPE, "ffk_attention_fwd: bad shape B2=%ld H=%ld Nq=%ld Nk=%ld", (long)B2, (long)H, (long)Nq,
@@ -354,8 +366,8 @@ extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, co
                 FFK_ERR_ALIGN, "ffk_attention_fwd: buffers must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
-        case FFK_BF16: return launch_attention<bf16_t>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, B2, H, Nq, Nk, st);
-        case FFK_F32: return launch_attention<float>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, B2, H, Nq, Nk, st);
+        case FFK_BF16: return launch_attention<bf16_t>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, B2, H, Nq, Nk, flags, st);
+        case FFK_F32: return launch_attention<float>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, B2, H, Nq, Nk, flags, st);
         default: return ffk_fail(FFK_ERR_DTYPE, "ffk_attention_fwd: unsupported dtype tag %d", dtype);
     }
 }

@@ -33,9 +33,21 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, half = lane >> 5;
-    const long m0 = (long)blockIdx.x * BT, n0 = (long)blockIdx.y * BT;
-    const int bz = blockIdx.z;
     const int M = d.M, N = d.N, K = d.K;
+    // Workgroup -> tile.  Consecutive workgroup ids go to the eight XCDs in turn, each with its own L2.
+    // With at least eight batches every XCD takes a contiguous eighth of the (batch, n-tile, m-tile)
+    // order, so that all tiles of one batch matrix pair run behind one L2 and A / B are fetched from
+    // HBM once instead of once per XCD.  With fewer batches the plain order is kept: tiles that run
+    // together then share their operand panels across the XCDs' row / column residues.
+    const unsigned tiles_m = (M + BT - 1) / BT, tiles_n = (N + BT - 1) / BT;
+    unsigned item = blockIdx.x;
+    if (d.batch >= 8) {
+        const unsigned total = tiles_m * tiles_n * (unsigned)d.batch, per_xcd = (total + 7) >> 3;
+        item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (item >= total) return;
+    }
+    const long m0 = (long)(item % tiles_m) * BT, n0 = (long)((item / tiles_m) % tiles_n) * BT;
+    const int bz = (item / tiles_m) / tiles_n;
     const T* A = (const T*)d.a + (long)bz * d.a_bs;
     const T* B = (const T*)d.b + (long)bz * d.b_bs;
 
@@ -231,7 +243,9 @@ int launch_bgemm(const ffk_bgemm_desc& d, hipStream_t st) {
                                              hipGetErrorString(e));
         configured = true;
     }
-    dim3 grid(ffk_cdiv(d.M, BT), ffk_cdiv(d.N, BT), d.batch);
+    const long tiles = (long)ffk_cdiv(d.M, BT) * ffk_cdiv(d.N, BT) * d.batch;
+    FFK_REQUIRE(tiles < (1L << 31) - 8, FFK_ERR_SHAPE, "ffk_bgemm_nt: %ld output tiles exceed the grid limit", tiles);
+    dim3 grid((unsigned)(d.batch >= 8 ? 8 * ffk_cdiv(tiles, 8) : tiles));
     bgemm_nt_kernel<T, OT><<<grid, THREADS, smem, st>>>(d);
     return ffk_check_launch("ffk_bgemm_nt");
 }
@@ -246,7 +260,6 @@ extern "C" int ffk_bgemm_nt(const ffk_bgemm_desc* d, void* stream) {
     FFK_REQUIRE(d->M > 0 && d->N > 0 && d->K > 0 && d->batch > 0 && d->batch < 65536 && d->inner > 0, FFK_ERR_SHAPE,
                 "ffk_bgemm_nt: bad shape M=%d N=%d K=%d batch=%d inner=%d", d->M, d->N, d->K, d->batch, d->inner);
     FFK_REQUIRE(d->K % vec == 0, FFK_ERR_SHAPE, "ffk_bgemm_nt: K=%d must be a multiple of %d", d->K, vec);
-    FFK_REQUIRE(ffk_cdiv(d->N, BT) < 65536, FFK_ERR_SHAPE, "ffk_bgemm_nt: N too large");
     FFK_REQUIRE(ffk_aligned16(d->a) && ffk_aligned16(d->b) && d->lda % vec == 0 && d->ldb % vec == 0 &&
                     d->a_bs % vec == 0 && d->b_bs % vec == 0,
                 FFK_ERR_ALIGN, "ffk_bgemm_nt: operand rows must be 16-byte aligned");

@@ -407,6 +407,8 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
                     const int hi = tab.hi[r + e], lo = tab.lo[r + e];
                     if (t.kind == FFK_TILE_V) {
                         o[e] = (long)hi * t.s_o + (long)(c >> 5) * t.s_h + (long)(lo >> 5) * 1024 + acc_tile_off(lo & 31, c & 31);
+                    } else if (t.kind == FFK_TILE_ACC) {
+                        o[e] = (long)hi * t.s_o + (long)(c >> 5) * t.s_h + (long)(lo >> 5) * 1024 + acc_tile_off(c & 31, lo & 31);
                     } else if (t.kind == FFK_TILE_BIAS) {
                         // logical row = (query hi, key lo); channel = head
                         o[e] = (long)c * t.s_h + (long)(hi >> 5) * t.s_o + (long)(lo >> 5) * 1024 +
@@ -480,7 +482,7 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
         FFK_REQUIRE(t.out, FFK_ERR_NULL, "ffk_fused_linear: tile %d has no output", i);
         FFK_REQUIRE(t.inner > 0 && t.ncols > 0 && t.ncols <= (t.glu ? 64 : 128), FFK_ERR_SHAPE,
                     "ffk_fused_linear: tile %d: bad inner/ncols (%d, %d)", i, t.inner, t.ncols);
-        FFK_REQUIRE(t.kind >= FFK_TILE_STRIDED && t.kind <= FFK_TILE_BIAS, FFK_ERR_UNSUPPORTED,
+        FFK_REQUIRE(t.kind >= FFK_TILE_STRIDED && t.kind <= FFK_TILE_ACC, FFK_ERR_UNSUPPORTED,
                     "ffk_fused_linear: tile %d: unknown kind %d", i, t.kind);
         const bool mode_c = (t.kind == FFK_TILE_STRIDED && t.s_d == 1) || t.kind == FFK_TILE_QK;
         FFK_REQUIRE(mode_c || (!t.resid && !t.gate), FFK_ERR_UNSUPPORTED,
@@ -502,6 +504,10 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
     for (int i = 0; i < d->n_tiles; ++i) {
         const ffk_tile& t = d->tiles[i];
         all_c = all_c && ((t.kind == FFK_TILE_STRIDED && t.s_d == 1) || t.kind == FFK_TILE_QK);
+    }
+    {
+        int status = FFK_OK;
+        if (ffk_linear_ws_try(d, (hipStream_t)stream, &status)) return status;
     }
     if (all_c) return ffk_linear_slab_launch(d, (hipStream_t)stream);
     switch (d->dtype) {

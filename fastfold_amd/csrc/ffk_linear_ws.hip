@@ -1,0 +1,497 @@
+// Weights-stationary variant of the fused linear layer (see ffk_fused_linear in include/ffk.h),
+// bf16, K = 128: the projections of the pair stack, where M is ~10^6 rows and the whole weight
+// matrix is a few hundred KB.
+//
+// One persistent workgroup of 8 wavefronts per CU.  The weight matrix is split into "slots" of 32
+// output rows; every wave keeps the MFMA fragments of up to three slots in registers for the whole
+// kernel, so weights are read from memory exactly once per workgroup.  Rows of A stream through a
+// double-buffered 128-row slab in LDS: global -> registers -> (LayerNorm in registers, 16 lanes
+// per row) -> LDS, the loads of slab i+1 being in flight while slab i is multiplied.  Each wave
+// multiplies every 32-row group of the slab against its own slots and finishes the resulting
+// 32x32 blocks straight from the accumulator registers - bias, activation, GLU, row mask, gate
+// and residual - and stores them without LDS staging:
+//   * tiles that are contiguous along channels (plain [row][channel] outputs, q / k / gate tiles)
+//     use the product W . A^T, so a lane owns one row and 4 x 4 consecutive channels;
+//   * tiles that are contiguous along rows (v tiles, channel-major outputs) use A . W^T, so a
+//     lane owns one channel and 4 x 4 consecutive rows.
+// Attention operand tiles are written as 32 contiguous bytes per lane, the order in which the
+// attention kernel loads them.
+#include "ffk_common.h"
+#include <stdlib.h>
+
+namespace {
+
+constexpr int WS_WAVES = 8;
+constexpr int WS_THREADS = 64 * WS_WAVES;
+constexpr int WS_BM = 128;               // rows per slab
+constexpr int WS_RG = WS_BM / 32;        // 32-row groups per slab
+constexpr int WS_NS = 3;                 // weight slots per wave
+constexpr int WS_K = 128;
+constexpr int WS_KS = WS_K / 16;         // MFMA K steps
+constexpr int WS_AP = WS_K * 2 + 16;     // LDS row pitch in bytes
+constexpr int WS_MAX_GRID = 256;         // one workgroup per CU
+
+typedef bf16_t T;
+
+struct WsPlan {
+    int wrow[WS_WAVES][WS_NS];   // first weight row of the slot
+    int tile[WS_WAVES][WS_NS];   // descriptor tile the slot belongs to, -1 = unused
+    int chan[WS_WAVES][WS_NS];   // first output channel (within the tile) of the slot's unit
+    int glu[WS_WAVES][WS_NS];    // 0 plain, 1 value half of a GLU unit (gate half in the next slot), 2 gate half
+    int rg_first[WS_WAVES], rg_step[WS_WAVES];   // row groups of a slab this wave works on
+    int row_perm;                // 1: rows of a group are read through tau (launch has channel-major tiles)
+};
+
+struct WsArgs {
+    ffk_linear_desc d;
+    WsPlan plan;
+};
+
+// tiles stored with channels contiguous (lane = row) vs rows contiguous (lane = channel)
+__host__ __device__ __forceinline__ bool ws_by_rows(const ffk_tile& t) {
+    return t.kind == FFK_TILE_QK || t.kind == FFK_TILE_ACC || (t.kind == FFK_TILE_STRIDED && t.s_d == 1);
+}
+
+__device__ __forceinline__ void unpack4(const T* p, float (&f)[4]) {
+    u32x2 raw = *reinterpret_cast<const u32x2*>(p);
+    const T* h = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = (float)h[e];
+}
+
+__device__ __forceinline__ void ws_activate(float (&x)[16], int act) {
+    if (act == FFK_ACT_RELU) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = fmaxf(x[v], 0.0f);
+    } else if (act == FFK_ACT_SIGMOID) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = sigmoid_f(x[v]);
+    }
+}
+
+// Index permutation tau(8a + 4h + b) = 16h + 4a + b.  An MFMA accumulator register v = 4a + b of
+// half-wave h holds row 8a + 4h + b of the M operand; loading M-operand row i from source row tau(i)
+// therefore leaves source rows 16h .. 16h + 15 in registers 0 .. 15: sixteen consecutive channels
+// (or rows) per lane, i.e. 32 contiguous bytes to store.
+__device__ __forceinline__ int ws_tau(int i) { return ((i >> 2) & 1) * 16 + (i >> 3) * 4 + (i & 3); }
+
+__device__ __forceinline__ void unpack8(const T* p, float* f) {
+    u32x4 raw = *reinterpret_cast<const u32x4*>(p);
+    const T* h = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
+}
+
+// ---- lane = row (n32 = its row within the group), registers = channels -----------------------
+// STRIDED tiles: weight rows were loaded through tau, registers hold channels 16*half + v.
+// ACC / QK tiles: natural weight order, registers hold channels 8a + 4*half + b.
+template <bool GLU>
+__device__ __forceinline__ void ws_store_rows(const ffk_tile& t, const f32x16& acc, const f32x16& accg, int chb, int c0,
+                                              long m0g, int M, int n32, int half) {
+    const long m = m0g + n32;
+    const bool valid = m < M;
+    const unsigned mc = (unsigned)(valid ? m : M - 1);
+    const unsigned hi = mc / (unsigned)t.inner, lo = mc - hi * (unsigned)t.inner;
+    const bool strided = t.kind == FFK_TILE_STRIDED;
+    float x[16];
+    if (t.bias) {
+        float bv[16], bg[16];
+        const T* bias = (const T*)t.bias + chb;
+        if (strided) {
+            unpack8(bias + 16 * half, bv);
+            unpack8(bias + 16 * half + 8, bv + 8);
+            if (GLU) {
+                unpack8(bias + 32 + 16 * half, bg);
+                unpack8(bias + 32 + 16 * half + 8, bg + 8);
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                float t4[4];
+                unpack4(bias + 4 * half + 8 * a, t4);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) bv[4 * a + b] = t4[b];
+                if (GLU) {
+                    unpack4(bias + 32 + 4 * half + 8 * a, t4);
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) bg[4 * a + b] = t4[b];
+                }
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = GLU ? (acc[v] + bv[v]) * sigmoid_f(accg[v] + bg[v]) : acc[v] + bv[v];
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = GLU ? acc[v] * sigmoid_f(accg[v]) : acc[v];
+    }
+    if (!GLU) ws_activate(x, t.act);
+    float scl = t.scale;
+    if (t.rowmask) scl *= (float)((const T*)t.rowmask)[(long)hi * t.m_so + (long)lo * t.m_si];
+    T y[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * scl);
+
+    T* out = (T*)t.out;
+    if (t.kind == FFK_TILE_ACC) {
+        if (valid && c0 + 32 <= t.ncols) {
+            T* p = out + (long)hi * t.s_o + (long)(c0 >> 5) * t.s_h + (long)(lo >> 5) * 1024 + ((half * 32 + (lo & 31)) << 4);
+            *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+            *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+        }
+    } else if (t.kind == FFK_TILE_QK) {
+        if (valid && c0 + 32 <= t.ncols) {
+            T* p = out + (long)hi * t.s_o + (long)(c0 >> 5) * t.s_h + (long)(lo >> 5) * 1024 + (lo & 31) * 16 + 4 * half;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)      // d = 8a + 4 half + b  ->  (d >> 4) * 512 + n * 16 + (d & 15)
+                *reinterpret_cast<u32x2*>(p + (a >> 1) * 512 + (a & 1) * 8) = *reinterpret_cast<const u32x2*>(&y[4 * a]);
+        }
+    } else {
+        const int cl = c0 + 16 * half;                   // this lane's 16 channels
+        const long off = (long)hi * t.s_o + (long)lo * t.s_i + (long)(c0 >> 5) * t.s_h + 16 * half;
+        const bool ok0 = valid && cl + 8 <= t.ncols, ok1 = valid && cl + 16 <= t.ncols;
+        if (t.gate || t.resid) {
+            // every load first (clamped, unconditional), then combine and store
+            u32x4 gv[2], rv[2];
+            const T* gate = t.gate ? (const T*)t.gate + (long)mc * t.gate_ld + cl : nullptr;
+            const T* resid = t.resid ? (const T*)t.resid + off : nullptr;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int cj = cl + 8 * j + 8 <= t.ncols ? 8 * j : (cl + 8 <= t.ncols ? 0 : -16 * half);
+                if (gate) gv[j] = *reinterpret_cast<const u32x4*>(gate + cj);
+                if (resid) rv[j] = *reinterpret_cast<const u32x4*>(resid + cj);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const T* gh = reinterpret_cast<const T*>(&gv[j]);
+                const T* rh = reinterpret_cast<const T*>(&rv[j]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float f = (float)y[8 * j + e];
+                    if (gate) f = (float)(T)(f * (float)gh[e]);
+                    if (resid) f += (float)rh[e];
+                    y[8 * j + e] = (T)f;
+                }
+            }
+        }
+        if (ok0) *reinterpret_cast<u32x4*>(out + off) = *reinterpret_cast<const u32x4*>(&y[0]);
+        if (ok1) *reinterpret_cast<u32x4*>(out + off + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+    }
+}
+
+// ---- lane = channel, registers = rows ----------------------------------------------------------
+// V tiles: natural row order (registers hold rows 8a + 4*half + b of the group).
+// STRIDED (channel-major) tiles: the A fragments were loaded through tau, registers hold rows
+// 16*half + v: sixteen consecutive rows, which never straddle `inner` (inner % 16 == 0, M % 16 == 0).
+template <bool GLU>
+__device__ __forceinline__ void ws_store_cols(const ffk_tile& t, const f32x16& acc, const f32x16& accg, int chb, int c0,
+                                              long m0g, int M, int l32, int half) {
+    const int ch = c0 + l32;
+    float bv = 0.0f, bg = 0.0f;
+    if (t.bias) {
+        bv = (float)((const T*)t.bias)[chb + l32];
+        if (GLU) bg = (float)((const T*)t.bias)[chb + 32 + l32];
+    }
+    float x[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) x[v] = GLU ? (acc[v] + bv) * sigmoid_f(accg[v] + bg) : acc[v] + bv;
+    if (!GLU) ws_activate(x, t.act);
+
+    T* out = (T*)t.out;
+    if (t.kind == FFK_TILE_V) {
+        const bool ok = m0g < M;                         // inner % 32 == 0: the group is one whole key tile
+        const unsigned mc = (unsigned)(ok ? m0g : 0);
+        const unsigned hi = mc / (unsigned)t.inner, lo = mc - hi * (unsigned)t.inner;
+        T y[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
+        if (ok && c0 + 32 <= t.ncols) {
+            T* p = out + (long)hi * t.s_o + (long)(c0 >> 5) * t.s_h + (long)(lo >> 5) * 1024 + ((half * 32 + l32) << 4);
+            *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+            *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+        }
+    } else {
+        const long mr = m0g + 16 * half;
+        const bool ok = mr < M;
+        const unsigned mc = (unsigned)(ok ? mr : 0);
+        const unsigned hi = mc / (unsigned)t.inner, lo = mc - hi * (unsigned)t.inner;
+        if (t.rowmask) {
+            const T* p = (const T*)t.rowmask + (long)hi * t.m_so + (long)lo * t.m_si;
+            float mk[16];
+            if (t.m_si == 1 && (t.m_so & 7) == 0 && (reinterpret_cast<uintptr_t>(t.rowmask) & 15) == 0) {
+                unpack8(p, mk);
+                unpack8(p + 8, mk + 8);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mk[v] = (float)p[(long)v * t.m_si];
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] *= mk[v];
+        }
+        T y[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
+        if (ok && ch < t.ncols) {
+            T* p = out + (long)hi * t.s_o + lo + (long)(ch >> 5) * t.s_h + (long)(ch & 31) * t.s_d;
+            *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+            *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs args) {
+    typedef Mma<T> MM;
+    const ffk_linear_desc& d = args.d;
+    extern __shared__ __align__(16) unsigned char smem[];          // [2][WS_BM][WS_AP]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const int M = d.M;
+    const T* A = (const T*)d.a;
+    const T* W = (const T*)d.w;
+
+    // ---- this wave's weight slots, resident in registers ----
+    int s_tile[WS_NS], s_chan[WS_NS], s_glu[WS_NS], s_chb[WS_NS];
+    bf16x8 wf[WS_NS][WS_KS];
+#pragma unroll
+    for (int s = 0; s < WS_NS; ++s) {
+        s_tile[s] = args.plan.tile[wave][s];
+        s_chan[s] = args.plan.chan[wave][s];
+        s_glu[s] = args.plan.glu[wave][s];
+        const int wr = s_tile[s] >= 0 ? args.plan.wrow[wave][s] : 0;
+        s_chb[s] = wr & 127;
+        // [row][channel] tiles take their weight rows through tau (16 consecutive channels per lane)
+        const ffk_tile& ts = d.tiles[s_tile[s] >= 0 ? s_tile[s] : 0];
+        const int wl = ts.kind == FFK_TILE_STRIDED && ts.s_d == 1 ? ws_tau(l32) : l32;
+#pragma unroll
+        for (int ks = 0; ks < WS_KS; ++ks) wf[s][ks] = MM::ld(W + (long)(wr + wl) * WS_K + ks * 16 + half * 8);
+    }
+    const int rg_first = args.plan.rg_first[wave], rg_step = args.plan.rg_step[wave];
+    // launches with channel-major tiles read the rows of a group through tau (16 consecutive rows per lane)
+    const int n32 = args.plan.row_perm ? ws_tau(l32) : l32;
+
+    // ---- slab streaming: thread -> (row tid/16 + 32 i, 8 channels starting at 8 * (tid % 16)) ----
+    const int c8 = tid & 15, r0 = tid >> 4;
+    const bool ln = d.ln_gamma != nullptr;
+    Vec16<T> gam, bet;                                   // kept packed: registers are scarce here
+    if (ln) {
+        gam = ld16((const T*)d.ln_gamma + c8 * 8);
+        bet = ld16((const T*)d.ln_beta + c8 * 8);
+    }
+    Vec16<T> pre[4];
+    auto fetch = [&](int slab) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            long m = (long)slab * WS_BM + r0 + 32 * i;
+            m = m < M ? m : M - 1;                       // clamped: rows past the end are never stored
+            const unsigned hi = (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
+            pre[i] = ld16(A + (long)hi * d.a_so + (long)lo * d.a_si + c8 * 8);
+        }
+    };
+    auto commit = [&](int buf) {
+        unsigned char* sa = smem + buf * (WS_BM * WS_AP);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            Vec16<T> x = pre[i];
+            if (ln) {
+                float f[8], s = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    f[e] = (float)x.e[e];
+                    s += f[e];
+                }
+                const float mu = group_sum(s, 16) * (1.0f / WS_K);
+                float q = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    f[e] -= mu;
+                    q += f[e] * f[e];
+                }
+                const float rs = rsqrtf(group_sum(q, 16) * (1.0f / WS_K) + d.ln_eps);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x.e[e] = (T)(f[e] * rs * (float)gam.e[e] + (float)bet.e[e]);
+            }
+            *reinterpret_cast<Vec16<T>*>(sa + (r0 + 32 * i) * WS_AP + c8 * 16) = x;
+        }
+    };
+
+    const int nslabs = (M + WS_BM - 1) / WS_BM;
+    int slab = blockIdx.x;                               // grid <= nslabs
+    fetch(slab);
+    commit(0);
+    lds_barrier();
+    int buf = 0;
+    for (; slab < nslabs; slab += gridDim.x) {
+        const int nxt = slab + (int)gridDim.x < nslabs ? slab + (int)gridDim.x : slab;
+        fetch(nxt);                                      // in flight during the products below
+        const unsigned char* sa = smem + buf * (WS_BM * WS_AP);
+        for (int rg = rg_first; rg < WS_RG; rg += rg_step) {
+            const long m0g = (long)slab * WS_BM + rg * 32;
+            if (m0g >= M) break;
+            bf16x8 af[WS_KS];
+            const unsigned char* ap = sa + (rg * 32 + n32) * WS_AP + half * 16;
+#pragma unroll
+            for (int ks = 0; ks < WS_KS; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + ks * 32);
+#pragma unroll
+            for (int s = 0; s < WS_NS; ++s) {
+                if (s_tile[s] < 0 || s_glu[s] == 2) continue;
+                const ffk_tile& t = d.tiles[s_tile[s]];
+                const bool by_rows = ws_by_rows(t);
+                const bool glu = s_glu[s] == 1;
+                const int sg = s + 1 < WS_NS ? s + 1 : s;          // gate slot of a GLU unit (constant after unrolling)
+                f32x16 acc, accg;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
+                if (by_rows) {
+#pragma unroll
+                    for (int ks = 0; ks < WS_KS; ++ks) MM::mma(acc, wf[s][ks], af[ks]);
+                    if (glu) {
+#pragma unroll
+                        for (int ks = 0; ks < WS_KS; ++ks) MM::mma(accg, wf[sg][ks], af[ks]);
+                        ws_store_rows<true>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, n32, half);
+                    } else {
+                        ws_store_rows<false>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, n32, half);
+                    }
+                } else {
+#pragma unroll
+                    for (int ks = 0; ks < WS_KS; ++ks) MM::mma(acc, af[ks], wf[s][ks]);
+                    if (glu) {
+#pragma unroll
+                        for (int ks = 0; ks < WS_KS; ++ks) MM::mma(accg, af[ks], wf[sg][ks]);
+                        ws_store_cols<true>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, l32, half);
+                    } else {
+                        ws_store_cols<false>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, l32, half);
+                    }
+                }
+            }
+        }
+        commit(buf ^ 1);
+        lds_barrier();
+        buf ^= 1;
+    }
+}
+
+bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (t.inner <= 0 || t.ncols <= 0 || !al16(t.out)) return false;
+    if (ws_by_rows(t)) {
+        if (t.kind == FFK_TILE_STRIDED) {
+            if (t.ncols % 8 != 0 || t.s_o % 8 || t.s_i % 8 || t.s_h % 8) return false;
+            if (t.resid && !al16(t.resid)) return false;
+            if (t.gate && (!al16(t.gate) || t.gate_ld % 8)) return false;
+        } else {
+            if (t.ncols % 32 != 0 || t.resid || t.gate || t.s_o % 8 || t.s_h % 8) return false;
+        }
+        return true;
+    }
+    if (t.resid || t.gate) return false;
+    if (t.kind == FFK_TILE_V) return t.inner % 32 == 0 && t.ncols % 32 == 0 && t.s_o % 8 == 0 && t.s_h % 8 == 0;
+    if (t.kind != FFK_TILE_STRIDED) return false;
+    return d.M % 16 == 0 && t.inner % 16 == 0 && t.s_i == 1 && t.s_o % 8 == 0 && t.s_h % 8 == 0 && t.s_d % 8 == 0;
+}
+
+// Distributes the 32-row weight units over the waves.  The waves form G = 8 / R groups; the R waves
+// of a group hold the same units and take every R-th row group of a slab (R as large as the units
+// allow, so that few units still use all eight waves).  Returns false if the units do not fit.
+bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
+    struct Unit { int tile, chan, wrow, slots; };
+    Unit units[FFK_MAX_TILES * 4];
+    int nu = 0;
+    for (int i = 0; i < d.n_tiles; ++i) {
+        const ffk_tile& t = d.tiles[i];
+        const int n = (t.ncols + 31) / 32;
+        for (int u = 0; u < n; ++u) {
+            Unit x;
+            x.tile = i;
+            x.chan = u * 32;
+            x.wrow = i * 128 + (t.glu ? u * 64 : u * 32);
+            x.slots = t.glu ? 2 : 1;
+            units[nu++] = x;
+        }
+    }
+    int assign[WS_WAVES][WS_NS];
+    int G = 0, R = 0;
+    for (R = WS_RG; R >= 1; R >>= 1) {
+        G = WS_WAVES / R;
+        int load[WS_WAVES] = {0};
+        for (int g = 0; g < G; ++g)
+            for (int s = 0; s < WS_NS; ++s) assign[g][s] = -1;
+        bool fits = true;
+        for (int pass = 2; pass >= 1 && fits; --pass) {            // two-slot (GLU) units first
+            for (int i = 0; i < nu && fits; ++i) {
+                if (units[i].slots != pass) continue;
+                int best = -1;
+                for (int g = 0; g < G; ++g)
+                    if (load[g] + pass <= WS_NS && (best < 0 || load[g] < load[best])) best = g;
+                if (best < 0) {
+                    fits = false;
+                    break;
+                }
+                assign[best][load[best]] = i;
+                if (pass == 2) assign[best][load[best] + 1] = -2 - i;   // gate half of unit i
+                load[best] += pass;
+            }
+        }
+        if (fits) break;
+    }
+    if (R < 1) return false;
+    for (int w = 0; w < WS_WAVES; ++w) {
+        const int g = w % G;
+        p.rg_first[w] = w / G;
+        p.rg_step[w] = R;
+        for (int s = 0; s < WS_NS; ++s) {
+            const int a = assign[g][s];
+            if (a == -1) {
+                p.tile[w][s] = -1;
+                p.wrow[w][s] = p.chan[w][s] = p.glu[w][s] = 0;
+            } else if (a >= 0) {
+                p.tile[w][s] = units[a].tile;
+                p.wrow[w][s] = units[a].wrow;
+                p.chan[w][s] = units[a].chan;
+                p.glu[w][s] = units[a].slots == 2 ? 1 : 0;
+            } else {
+                const Unit& u = units[-2 - a];
+                p.tile[w][s] = u.tile;
+                p.wrow[w][s] = u.wrow + 32;
+                p.chan[w][s] = u.chan;
+                p.glu[w][s] = 2;
+            }
+        }
+    }
+    return true;
+}
+
+}  // namespace
+
+// Launches the weights-stationary kernel if it can take this (already validated) descriptor and
+// returns 1 with the launch status in *status; returns 0 if the caller has to use another variant.
+int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
+    if (d->dtype != FFK_BF16 || d->K != WS_K || d->a_chanmajor) return 0;
+    if (getenv("FFK_NO_WS")) return 0;
+    bool chan_major = false, v_tiles = false;
+    for (int i = 0; i < d->n_tiles; ++i) {
+        const ffk_tile& t = d->tiles[i];
+        if (!ws_tile_ok(*d, t)) return 0;
+        chan_major = chan_major || (!ws_by_rows(t) && t.kind == FFK_TILE_STRIDED);
+        v_tiles = v_tiles || t.kind == FFK_TILE_V;
+    }
+    if (chan_major && v_tiles) return 0;          // they need different row orders within a group
+    WsArgs args;
+    if (!ws_make_plan(*d, args.plan)) return 0;
+    args.plan.row_perm = chan_major ? 1 : 0;
+    args.d = *d;
+    const size_t smem = 2 * (size_t)WS_BM * WS_AP;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) {
+            *status = ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
+            return 1;
+        }
+        configured = true;
+    }
+    const int nslabs = ffk_cdiv(d->M, WS_BM);
+    const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
+    linear_ws_kernel<<<grid, WS_THREADS, smem, st>>>(args);
+    *status = ffk_check_launch("ffk_fused_linear");
+    return 1;
+}

@@ -10,7 +10,7 @@ import math
 import torch
 
 from fastfold_amd import _lib
-from fastfold_amd._lib import (FFK_ACT_NONE, FFK_ACT_RELU, FFK_ACT_SIGMOID, FFK_TILE_BIAS, FFK_TILE_QK,
+from fastfold_amd._lib import (FFK_ACT_NONE, FFK_ACT_RELU, FFK_ACT_SIGMOID, FFK_TILE_ACC, FFK_TILE_BIAS, FFK_TILE_QK,
                                FFK_TILE_STRIDED, FFK_TILE_V, LOG2E, make_tile)
 
 _WS_BUDGET_DEFAULT = 6 << 30     # bytes of scratch one sub-module may hold at a time
@@ -133,27 +133,42 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     q_t = alloc((B2, H, NT, 1024), dt, dev, zero)
     k_t = alloc((B2, H, NT, 1024), dt, dev, zero)
     v_t = alloc((B2, H, NT, 1024), dt, dev, zero)
-    gate = torch.empty(M, HC, dtype=dt, device=dev)
+    # With bf16, 128 input channels and whole key tiles the projection runs on the weights-stationary
+    # kernel, which writes q, k and the gate in accumulator order straight from its registers.
+    acc_order = dt == torch.bfloat16 and C == 128 and N % 32 == 0
+    qk_kind = FFK_TILE_ACC if acc_order else FFK_TILE_QK
+    gate = torch.empty((B2, H, NT, 1024) if acc_order else (M, HC), dtype=dt, device=dev)
     tpg = HC // 128
     qscale = LOG2E / math.sqrt(32.0)
+    tkw = dict(inner=N, s_o=H * NT * 1024, s_h=NT * 1024)
     tiles = []
-    for buf, kind, scale in ((q_t, FFK_TILE_QK, qscale), (k_t, FFK_TILE_QK, 1.0), (v_t, FFK_TILE_V, 1.0)):
+    for buf, kind, scale in ((q_t, qk_kind, qscale), (k_t, qk_kind, 1.0), (v_t, FFK_TILE_V, 1.0)):
         for t in range(tpg):
-            tiles.append(make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, inner=N,
-                                   s_o=H * NT * 1024, s_h=NT * 1024, scale=scale))
+            tiles.append(make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, scale=scale, **tkw))
     for t in range(tpg):
-        tiles.append(make_tile(gate.data_ptr() + t * 128 * es, bias=gate_bias_pk.data_ptr() + t * 128 * es,
-                               inner=M, s_i=HC, act=FFK_ACT_SIGMOID))
-    if bias_in_launch:
-        tiles.append(make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H,
-                               scale=LOG2E))
+        if acc_order:
+            tiles.append(make_tile(gate.data_ptr() + t * 4 * NT * 1024 * es, kind=FFK_TILE_ACC,
+                                   bias=gate_bias_pk.data_ptr() + t * 128 * es, act=FFK_ACT_SIGMOID, **tkw))
+        else:
+            tiles.append(make_tile(gate.data_ptr() + t * 128 * es, bias=gate_bias_pk.data_ptr() + t * 128 * es,
+                                   inner=M, s_i=HC, act=FFK_ACT_SIGMOID))
     a_inner, a_so, a_si = a_map
+    bias_tile = None
+    if bias_in_launch:
+        bias_tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H,
+                              scale=LOG2E)
+    if bias_tile is not None and not acc_order:
+        tiles.append(bias_tile)
+        bias_tile = None
     _lib.fused_linear(x, w_pk, tiles, M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln)
+    if bias_tile is not None:      # the bias tile has its own pass (it needs the LDS-staged kernel)
+        _lib.fused_linear(x, w_pk, [bias_tile], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
+                          w_row_off=4 * tpg * 128)
     kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
     flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
     _lib.key_bias(kb, flags, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
     o = torch.empty(M, HC, dtype=dt, device=dev)
-    _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, flags, gate, B2=B2, H=H, Nq=N, Nk=N)
+    _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, flags, gate, B2=B2, H=H, Nq=N, Nk=N, gate_tiled=acc_order)
     del q_t, k_t, v_t, gate
     tiles = []
     for t in range((c_out + 127) // 128):

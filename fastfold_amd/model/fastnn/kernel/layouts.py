@@ -33,6 +33,21 @@ def untile_qk(t, N):
     return t.permute(0, 1, 2, 4, 3, 5).reshape(B2, H, NT * 32, 32)[:, :, :N]
 
 
+def tile_rows_acc(x):
+    """[B2, H, N, 32] -> [B2, H, NT, 2, 32, 4, 4]: FFK_TILE_ACC order, channel d = 8a + 4*half + b of
+    token n at [n//32, half, n%32, a, b] (the lane that owns row n of a 32x32 accumulator holds its
+    16 channels contiguously)."""
+    B2, H, N, D = x.shape
+    assert D == 32
+    x = _pad_to(x, 2, 32)
+    return x.view(B2, H, -1, 32, 4, 2, 4).permute(0, 1, 2, 5, 3, 4, 6).contiguous()
+
+
+def untile_rows_acc(t, N):
+    B2, H, NT = t.shape[:3]
+    return t.permute(0, 1, 2, 4, 5, 3, 6).reshape(B2, H, NT * 32, 32)[:, :, :N]
+
+
 def tile_acc(x):
     """[..., R, C32] with the row axis second to last (keys) and 32 columns ->
     [..., RT, 2, 32, 4, 4]: row = 8a + 4kg + b at [row//32, kg, col, a, b]."""

@@ -123,6 +123,11 @@ int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const 
  *   FFK_TILE_QK       q / k of attention in MFMA-operand tiles: [b2][h][n/32][d/16][n%32][d%16]
  *   FFK_TILE_V        v of attention in PV-operand tiles (see ffk_attention_fwd)
  *   FFK_TILE_BIAS     pair / triangle bias in score-accumulator tiles (see ffk_attention_fwd)
+ *   FFK_TILE_ACC      [b2][h][n/32] tiles in MFMA accumulator order: element (n, d) of a tile at
+ *                     ((d & 7) >> 2) * 512 + (n % 32) * 16 + 4 * (d >> 3) + (d & 3), i.e. the lane that
+ *                     owns row n in a 32x32 accumulator holds its 16 channels contiguously.  Valid for
+ *                     q and k (any common order of the head dim gives the same q.k) and required
+ *                     for a gate that ffk_attention_fwd reads with FFK_ATT_GATE_TILED.
  * Per-tile value: v = act(acc + bias[c]) * scale; with glu != 0 the tile's packed channels are
  * [p 0..31 | g 0..31 | p 32..63 | g 32..63] and v = (p + bias_p) * sigmoid(g + bias_g) (64
  * outputs); rowmask (0/1 per logical row, own strides) multiplies v.
@@ -130,7 +135,7 @@ int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const 
  * Replaces the F.linear + LayerNorm + elementwise chains of fastfold/model/fastnn/ops.py:
  * 79-82,143-155,305-324,393-399,404-412,659-670 and msa.py:61-72.
  */
-enum { FFK_TILE_STRIDED = 0, FFK_TILE_QK = 1, FFK_TILE_V = 2, FFK_TILE_BIAS = 3 };
+enum { FFK_TILE_STRIDED = 0, FFK_TILE_QK = 1, FFK_TILE_V = 2, FFK_TILE_BIAS = 3, FFK_TILE_ACC = 4 };
 enum { FFK_ACT_NONE = 0, FFK_ACT_RELU = 1, FFK_ACT_SIGMOID = 2 };
 #define FFK_MAX_TILES 10
 
@@ -210,21 +215,23 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  * hugely negative finite value for the padding up to a multiple of 32; build it with
  * ffk_key_bias).  Operands arrive in 32x32 operand tiles (1024 elements, see
  * ffk_fused_linear tile kinds):
- *   q_t, k_t : [B2][H][ceil(N/32)][1024]   FFK_TILE_QK order
+ *   q_t, k_t : [B2][H][ceil(N/32)][1024]   FFK_TILE_QK or FFK_TILE_ACC order (the same for both)
  *   v_t      : [B2][H][ceil(Nk/32)][1024]  FFK_TILE_V  order
  *   bias_t   : [H][ceil(Nq/32)][ceil(Nk/32)][1024]  FFK_TILE_BIAS order (keys x queries as an
  *              MFMA operand: element (k, q) at (q%32/16)*512 + (k%32)*16 + q%16), or NULL
  *   keybias  : [B2][ceil(Nk/32)*32] fp32
  *   tileflags: [B2][ceil(Nk/32)] int32 per 32-key tile: 0 all keys valid, 1 mixed, 2 all masked
- *   gate     : [B2*Nq, H*32] row-major multiplicative gate (already sigmoid-ed), or NULL
+ *   gate     : multiplicative gate (already sigmoid-ed) or NULL: [B2*Nq, H*32] row-major, or with
+ *              FFK_ATT_GATE_TILED in flags [B2][H][ceil(Nq/32)][1024] in FFK_TILE_ACC order
  *   out      : [B2*Nq, H*32] row-major
  * Replaces: the matmul / fused_softmax / matmul (+ bias_sigmod_ele) chain of
  * SelfAttention.forward (fastfold/model/fastnn/ops.py:310-322) and
  * fused_attention_core (kernel/attention_core.py:17-52, kernel/triton/attention_core.py:12-190).
  */
+enum { FFK_ATT_GATE_TILED = 1 };
 int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t,
                       const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
-                      int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int dtype, void* stream);
+                      int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int flags, int dtype, void* stream);
 
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the

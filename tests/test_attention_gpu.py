@@ -55,6 +55,11 @@ def test_attention_core(dev, dtype, tol, B2, H, N, use_bias, use_gate):
     if use_gate:
         ref = ref * _np(gate).reshape(B2, N, H * 32)
     assert _rel(_np(out).reshape(B2, N, H * 32), ref) < tol
+    if use_gate:     # the same gate handed over in accumulator-tile order gives the same bits
+        gate_t = layouts.tile_rows_acc(gate.view(B2, N, H, 32).permute(0, 2, 1, 3))
+        out2 = torch.empty_like(out)
+        _lib.attention_fwd(out2, qt, kt, vt, bt, kb, fl, gate_t, B2=B2, H=H, Nq=N, Nk=N, gate_tiled=True)
+        assert torch.equal(out, out2)
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])

@@ -222,3 +222,86 @@ def test_bad_descriptors_are_rejected(dev):
         _lib.fused_linear(a, w, [_lib.make_tile(out, inner=0, s_i=128)], M=64, K=128)      # inner
     with pytest.raises(RuntimeError):
         _lib.fused_linear(a, w, [_lib.make_tile(out, inner=64, s_i=128, s_d=2, resid=out)], M=64, K=128)
+
+
+def test_weights_stationary_many_slabs(dev):
+    """bf16, K = 128, more slabs than workgroups (persistent loop, ragged last slab): q in accumulator
+    order with a scale, k in q/k order, v, a sigmoid gate in accumulator order and a plain relu tile,
+    all from one LayerNorm-ed pass over A."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    dtype = torch.bfloat16
+    B2, N, H, K = 131, 288, 4, 128                      # M = 37728 rows = 294.75 slabs
+    C = H * 32
+    M = B2 * N
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(B2, N, K, generator=g) + 0.3).to(dev, dtype)
+    ws_ = [(torch.randn(C, K, generator=g) / K ** 0.5).to(dev, dtype) for _ in range(5)]
+    bias_g = torch.randn(C, generator=g).to(dev, dtype)
+    bias_r = torch.randn(C, generator=g).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(K, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(K, generator=g)).to(dev, dtype)
+    NT = layouts.n_tiles(N)
+    q = torch.zeros(B2, H, NT, 2, 32, 4, 4, dtype=dtype, device=dev)
+    k = torch.zeros(B2, H, NT, 2, 32, 16, dtype=dtype, device=dev)
+    v = torch.zeros(B2, H, NT, 2, 32, 4, 4, dtype=dtype, device=dev)
+    gt = torch.zeros(B2, H, NT, 2, 32, 4, 4, dtype=dtype, device=dev)
+    plain = torch.zeros(M, C, dtype=dtype, device=dev)
+    tk = dict(inner=N, s_o=H * NT * 1024, s_h=NT * 1024)
+    tiles = [_lib.make_tile(q, kind=_lib.FFK_TILE_ACC, scale=0.25, **tk),
+             _lib.make_tile(k, kind=_lib.FFK_TILE_QK, **tk),
+             _lib.make_tile(v, kind=_lib.FFK_TILE_V, **tk),
+             _lib.make_tile(gt, kind=_lib.FFK_TILE_ACC, bias=bias_g, act=_lib.FFK_ACT_SIGMOID, **tk),
+             _lib.make_tile(plain, bias=bias_r, act=_lib.FFK_ACT_RELU, inner=M, s_i=C)]
+    bias_all = torch.zeros(5 * 128, dtype=dtype, device=dev)
+    bias_all[3 * 128:4 * 128] = bias_g
+    bias_all[4 * 128:] = bias_r
+    tiles[3].bias = bias_all.data_ptr() + 3 * 128 * 2
+    tiles[4].bias = bias_all.data_ptr() + 4 * 128 * 2
+    _lib.fused_linear(x, torch.cat(ws_).contiguous(), tiles, M=M, K=K, ln=(gam, bet))
+    xn = _np(torch.from_numpy(ops_np.layer_norm(_np(x), _np(gam), _np(bet))).to(torch.bfloat16))
+    lin = [ops_np.linear(xn, _np(w)) for w in ws_]
+    heads = lambda y: y.reshape(B2, N, H, 32).transpose(0, 2, 1, 3)
+    assert _rel(_np(layouts.untile_rows_acc(q, N)), heads(lin[0] * 0.25)) < TOL[dtype]
+    assert _rel(_np(layouts.untile_qk(k, N)), heads(lin[1])) < TOL[dtype]
+    assert _rel(_np(layouts.untile_v(v, N)), heads(lin[2])) < TOL[dtype]
+    assert _rel(_np(layouts.untile_rows_acc(gt, N)), heads(_sig(lin[3] + _np(bias_g)))) < TOL[dtype]
+    assert _rel(_np(plain).reshape(B2, N, C), np.maximum(lin[4] + _np(bias_r), 0)) < TOL[dtype]
+
+
+def test_weights_stationary_matches_other_variant(dev, monkeypatch):
+    """GLU + row mask, channel-major store, both traversal orders, at a multi-slab size: the
+    weights-stationary kernel and the LDS-staged kernel must agree to bf16 rounding."""
+    from fastfold_amd import _lib
+    dtype = torch.bfloat16
+    r, C, Ch = 200, 128, 128
+    g = torch.Generator().manual_seed(5)
+    z = torch.randn(r, r, C, generator=g).to(dev, dtype)
+    wpk = (torch.randn(2 * Ch + 128, C, generator=g) / C ** 0.5).to(dev, dtype)
+    bpk = torch.randn(2 * Ch + 128, generator=g).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    mask = (torch.rand(r, r, generator=g) > 0.2).to(dev, dtype)
+    outs = []
+    for no_ws in (False, True):
+        if no_ws:
+            monkeypatch.setenv("FFK_NO_WS", "1")
+        res = []
+        for transposed in (False, True):
+            out = torch.zeros(Ch, r, r, dtype=dtype, device=dev)
+            gate = torch.zeros(r * r, C, dtype=dtype, device=dev)
+            tiles = []
+            for t in range(Ch // 64):
+                tiles.append(_lib.make_tile(out.data_ptr() + t * 64 * r * r * 2, bias=bpk.data_ptr() + t * 128 * 2,
+                                            glu=1, ncols=64, inner=r, s_o=r, s_i=1, s_h=32 * r * r, s_d=r * r,
+                                            rowmask=mask, m_so=(1 if transposed else r), m_si=(r if transposed else 1)))
+            kw = dict(inner=r, s_o=C, s_i=r * C) if transposed else dict(inner=r * r, s_i=C)
+            tiles.append(_lib.make_tile(gate, bias=bpk.data_ptr() + 2 * 128 * 2, act=_lib.FFK_ACT_SIGMOID, **kw))
+            akw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else {}
+            _lib.fused_linear(z, wpk, tiles, M=r * r, K=C, ln=(gam, bet), **akw)
+            res += [out, gate]
+        outs.append(res)
+    monkeypatch.delenv("FFK_NO_WS")
+    for a, b in zip(*outs):
+        assert float(a.float().abs().max()) > 0.1
+        assert _rel(_np(a), _np(b)) < 1e-2
