@@ -40,11 +40,28 @@ struct WsPlan {
     int glu[WS_WAVES][WS_NS];    // 0 plain, 1 value half of a GLU unit (gate half in the next slot), 2 gate half
     int rg_first[WS_WAVES], rg_step[WS_WAVES];   // row groups of a slab this wave works on
     int row_perm;                // 1: rows of a group are read through tau (launch has channel-major tiles)
+    int mask_tile;               // first tile with a row mask (all masked tiles share its mask), -1 = none
+    int max_slots;               // largest number of slots any wave holds
 };
 
 struct WsArgs {
     ffk_linear_desc d;
     WsPlan plan;
+};
+
+// What the epilogue of one slot needs, copied out of the tile descriptor once per kernel so that it
+// lives in scalar registers (reading descriptor fields inside the loops costs a scalar load plus a
+// full wait each time).  Channel offsets of the slot's unit are folded into the pointers.
+struct WsSlot {
+    T* out;
+    const T* resid;
+    const T* gate;
+    long s_o, s_i, s_d, gate_ld;
+    unsigned inner;
+    int ncols_left;          // valid channels from the unit's first channel on
+    int kind, act;
+    float scale;
+    bool masked;
 };
 
 // tiles stored with channels contiguous (lane = row) vs rows contiguous (lane = channel)
@@ -85,78 +102,56 @@ __device__ __forceinline__ void unpack8(const T* p, float* f) {
 // ---- lane = row (n32 = its row within the group), registers = channels -----------------------
 // STRIDED tiles: weight rows were loaded through tau, registers hold channels 16*half + v.
 // ACC / QK tiles: natural weight order, registers hold channels 8a + 4*half + b.
+// sb: this slot's 32 (GLU: 64) bias values in LDS (fp32); rmask: the row's mask value.
 template <bool GLU>
-__device__ __forceinline__ void ws_store_rows(const ffk_tile& t, const f32x16& acc, const f32x16& accg, int chb, int c0,
-                                              long m0g, int M, int n32, int half) {
-    const long m = m0g + n32;
-    const bool valid = m < M;
-    const unsigned mc = (unsigned)(valid ? m : M - 1);
-    const unsigned hi = mc / (unsigned)t.inner, lo = mc - hi * (unsigned)t.inner;
+__device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+                                              bool valid, unsigned mc, unsigned hi, unsigned lo, float rmask, int half) {
     const bool strided = t.kind == FFK_TILE_STRIDED;
     float x[16];
-    if (t.bias) {
-        float bv[16], bg[16];
-        const T* bias = (const T*)t.bias + chb;
-        if (strided) {
-            unpack8(bias + 16 * half, bv);
-            unpack8(bias + 16 * half + 8, bv + 8);
-            if (GLU) {
-                unpack8(bias + 32 + 16 * half, bg);
-                unpack8(bias + 32 + 16 * half + 8, bg + 8);
-            }
-        } else {
+    {
+        f32x4 bv[4], bg[4];
 #pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                float t4[4];
-                unpack4(bias + 4 * half + 8 * a, t4);
-#pragma unroll
-                for (int b = 0; b < 4; ++b) bv[4 * a + b] = t4[b];
-                if (GLU) {
-                    unpack4(bias + 32 + 4 * half + 8 * a, t4);
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) bg[4 * a + b] = t4[b];
-                }
-            }
+        for (int a = 0; a < 4; ++a) {
+            const int o = strided ? 16 * half + 4 * a : 4 * half + 8 * a;
+            bv[a] = *reinterpret_cast<const f32x4*>(sb + o);
+            if (GLU) bg[a] = *reinterpret_cast<const f32x4*>(sb + 32 + o);
         }
 #pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = GLU ? (acc[v] + bv[v]) * sigmoid_f(accg[v] + bg[v]) : acc[v] + bv[v];
-    } else {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = GLU ? acc[v] * sigmoid_f(accg[v]) : acc[v];
+        for (int v = 0; v < 16; ++v)
+            x[v] = GLU ? (acc[v] + bv[v >> 2][v & 3]) * sigmoid_f(accg[v] + bg[v >> 2][v & 3]) : acc[v] + bv[v >> 2][v & 3];
     }
     if (!GLU) ws_activate(x, t.act);
-    float scl = t.scale;
-    if (t.rowmask) scl *= (float)((const T*)t.rowmask)[(long)hi * t.m_so + (long)lo * t.m_si];
+    const float scl = t.scale * rmask;
     T y[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * scl);
 
-    T* out = (T*)t.out;
+    T* out = t.out;
     if (t.kind == FFK_TILE_ACC) {
-        if (valid && c0 + 32 <= t.ncols) {
-            T* p = out + (long)hi * t.s_o + (long)(c0 >> 5) * t.s_h + (long)(lo >> 5) * 1024 + ((half * 32 + (lo & 31)) << 4);
+        if (valid && t.ncols_left >= 32) {
+            T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + ((half * 32 + (lo & 31)) << 4);
             *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
             *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
     } else if (t.kind == FFK_TILE_QK) {
-        if (valid && c0 + 32 <= t.ncols) {
-            T* p = out + (long)hi * t.s_o + (long)(c0 >> 5) * t.s_h + (long)(lo >> 5) * 1024 + (lo & 31) * 16 + 4 * half;
+        if (valid && t.ncols_left >= 32) {
+            T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + (lo & 31) * 16 + 4 * half;
 #pragma unroll
             for (int a = 0; a < 4; ++a)      // d = 8a + 4 half + b  ->  (d >> 4) * 512 + n * 16 + (d & 15)
                 *reinterpret_cast<u32x2*>(p + (a >> 1) * 512 + (a & 1) * 8) = *reinterpret_cast<const u32x2*>(&y[4 * a]);
         }
     } else {
-        const int cl = c0 + 16 * half;                   // this lane's 16 channels
-        const long off = (long)hi * t.s_o + (long)lo * t.s_i + (long)(c0 >> 5) * t.s_h + 16 * half;
-        const bool ok0 = valid && cl + 8 <= t.ncols, ok1 = valid && cl + 16 <= t.ncols;
+        const int cl = 16 * half;                        // this lane's 16 channels, relative to the unit
+        const long off = (long)hi * t.s_o + (long)lo * t.s_i + cl;
+        const bool ok0 = valid && cl + 8 <= t.ncols_left, ok1 = valid && cl + 16 <= t.ncols_left;
         if (t.gate || t.resid) {
             // every load first (clamped, unconditional), then combine and store
             u32x4 gv[2], rv[2];
-            const T* gate = t.gate ? (const T*)t.gate + (long)mc * t.gate_ld + cl : nullptr;
-            const T* resid = t.resid ? (const T*)t.resid + off : nullptr;
+            const T* gate = t.gate ? t.gate + (long)mc * t.gate_ld + cl : nullptr;
+            const T* resid = t.resid ? t.resid + off : nullptr;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int cj = cl + 8 * j + 8 <= t.ncols ? 8 * j : (cl + 8 <= t.ncols ? 0 : -16 * half);
+                const int cj = cl + 8 * j + 8 <= t.ncols_left ? 8 * j : (cl + 8 <= t.ncols_left ? 0 : -cl);
                 if (gate) gv[j] = *reinterpret_cast<const u32x4*>(gate + cj);
                 if (resid) rv[j] = *reinterpret_cast<const u32x4*>(resid + cj);
             }
@@ -182,66 +177,58 @@ __device__ __forceinline__ void ws_store_rows(const ffk_tile& t, const f32x16& a
 // V tiles: natural row order (registers hold rows 8a + 4*half + b of the group).
 // STRIDED (channel-major) tiles: the A fragments were loaded through tau, registers hold rows
 // 16*half + v: sixteen consecutive rows, which never straddle `inner` (inner % 16 == 0, M % 16 == 0).
+// sm: mask values (fp32, LDS) of the group's 32 rows, or nullptr.
 template <bool GLU>
-__device__ __forceinline__ void ws_store_cols(const ffk_tile& t, const f32x16& acc, const f32x16& accg, int chb, int c0,
-                                              long m0g, int M, int l32, int half) {
-    const int ch = c0 + l32;
-    float bv = 0.0f, bg = 0.0f;
-    if (t.bias) {
-        bv = (float)((const T*)t.bias)[chb + l32];
-        if (GLU) bg = (float)((const T*)t.bias)[chb + 32 + l32];
-    }
+__device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+                                              const float* sm, long m0g, int M, int l32, int half) {
+    const float bv = sb[l32], bg = GLU ? sb[32 + l32] : 0.0f;
     float x[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) x[v] = GLU ? (acc[v] + bv) * sigmoid_f(accg[v] + bg) : acc[v] + bv;
     if (!GLU) ws_activate(x, t.act);
 
-    T* out = (T*)t.out;
-    if (t.kind == FFK_TILE_V) {
-        const bool ok = m0g < M;                         // inner % 32 == 0: the group is one whole key tile
-        const unsigned mc = (unsigned)(ok ? m0g : 0);
-        const unsigned hi = mc / (unsigned)t.inner, lo = mc - hi * (unsigned)t.inner;
-        T y[16];
+    T* out = t.out;
+    const bool vt = t.kind == FFK_TILE_V;
+    const long mr = vt ? m0g : m0g + 16 * half;          // V: the group is one whole key tile (inner % 32 == 0)
+    const bool ok = mr < M;
+    const unsigned mc = (unsigned)(ok ? mr : 0);
+    unsigned hi = 0, lo = mc;
+    if (t.inner < (unsigned)M) {
+        hi = mc / t.inner;
+        lo = mc - hi * t.inner;
+    }
+    if (sm && !vt) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
-        if (ok && c0 + 32 <= t.ncols) {
-            T* p = out + (long)hi * t.s_o + (long)(c0 >> 5) * t.s_h + (long)(lo >> 5) * 1024 + ((half * 32 + l32) << 4);
+        for (int a = 0; a < 4; ++a) {
+            const f32x4 mk = *reinterpret_cast<const f32x4*>(sm + 16 * half + 4 * a);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) x[4 * a + b] *= mk[b];
+        }
+    }
+    T y[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
+    if (vt) {
+        if (ok && t.ncols_left >= 32) {
+            T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + ((half * 32 + l32) << 4);
             *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
             *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
-    } else {
-        const long mr = m0g + 16 * half;
-        const bool ok = mr < M;
-        const unsigned mc = (unsigned)(ok ? mr : 0);
-        const unsigned hi = mc / (unsigned)t.inner, lo = mc - hi * (unsigned)t.inner;
-        if (t.rowmask) {
-            const T* p = (const T*)t.rowmask + (long)hi * t.m_so + (long)lo * t.m_si;
-            float mk[16];
-            if (t.m_si == 1 && (t.m_so & 7) == 0 && (reinterpret_cast<uintptr_t>(t.rowmask) & 15) == 0) {
-                unpack8(p, mk);
-                unpack8(p + 8, mk + 8);
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) mk[v] = (float)p[(long)v * t.m_si];
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) x[v] *= mk[v];
-        }
-        T y[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
-        if (ok && ch < t.ncols) {
-            T* p = out + (long)hi * t.s_o + lo + (long)(ch >> 5) * t.s_h + (long)(ch & 31) * t.s_d;
-            *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
-            *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
-        }
+    } else if (ok && l32 < t.ncols_left) {
+        T* p = out + (long)hi * t.s_o + lo + (long)l32 * t.s_d;
+        *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+        *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
     }
 }
 
+template <int NS>
 __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs args) {
     typedef Mma<T> MM;
     const ffk_linear_desc& d = args.d;
-    extern __shared__ __align__(16) unsigned char smem[];          // [2][WS_BM][WS_AP]
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char* s_a = smem;                                                 // [2][WS_BM][WS_AP]
+    float* s_mask = reinterpret_cast<float*>(smem + 2 * WS_BM * WS_AP);        // [2][WS_BM]
+    float* s_bias = s_mask + 2 * WS_BM;                                        // [n_tiles][128]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
@@ -249,21 +236,45 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const T* A = (const T*)d.a;
     const T* W = (const T*)d.w;
 
+    // ---- bias table: no global loads in the epilogues ----
+    for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) {
+        const T* bp = (const T*)d.tiles[i >> 7].bias;
+        s_bias[i] = bp ? (float)bp[i & 127] : 0.0f;
+    }
+
     // ---- this wave's weight slots, resident in registers ----
-    int s_tile[WS_NS], s_chan[WS_NS], s_glu[WS_NS], s_chb[WS_NS];
-    bf16x8 wf[WS_NS][WS_KS];
+    int s_tile[NS], s_chan[NS], s_glu[NS], s_wrow[NS];
+    WsSlot sp[NS];
+    bool by_rows[NS];
+    bf16x8 wf[NS][WS_KS];
 #pragma unroll
-    for (int s = 0; s < WS_NS; ++s) {
+    for (int s = 0; s < NS; ++s) {
         s_tile[s] = args.plan.tile[wave][s];
         s_chan[s] = args.plan.chan[wave][s];
         s_glu[s] = args.plan.glu[wave][s];
-        const int wr = s_tile[s] >= 0 ? args.plan.wrow[wave][s] : 0;
-        s_chb[s] = wr & 127;
+        s_wrow[s] = s_tile[s] >= 0 ? args.plan.wrow[wave][s] : 0;
         // [row][channel] tiles take their weight rows through tau (16 consecutive channels per lane)
         const ffk_tile& ts = d.tiles[s_tile[s] >= 0 ? s_tile[s] : 0];
         const int wl = ts.kind == FFK_TILE_STRIDED && ts.s_d == 1 ? ws_tau(l32) : l32;
+        {
+            const long coff = (long)(s_chan[s] >> 5) * ts.s_h;
+            sp[s].out = (T*)ts.out + coff;
+            sp[s].resid = ts.resid ? (const T*)ts.resid + coff : nullptr;
+            sp[s].gate = ts.gate ? (const T*)ts.gate + s_chan[s] : nullptr;
+            sp[s].s_o = ts.s_o;
+            sp[s].s_i = ts.s_i;
+            sp[s].s_d = ts.s_d;
+            sp[s].gate_ld = ts.gate_ld;
+            sp[s].inner = (unsigned)ts.inner;
+            sp[s].ncols_left = ts.ncols - s_chan[s];
+            sp[s].kind = ts.kind;
+            sp[s].act = ts.act;
+            sp[s].scale = ts.scale;
+            sp[s].masked = ts.rowmask != nullptr;
+            by_rows[s] = ws_by_rows(ts);
+        }
 #pragma unroll
-        for (int ks = 0; ks < WS_KS; ++ks) wf[s][ks] = MM::ld(W + (long)(wr + wl) * WS_K + ks * 16 + half * 8);
+        for (int ks = 0; ks < WS_KS; ++ks) wf[s][ks] = MM::ld(W + (long)(s_wrow[s] + wl) * WS_K + ks * 16 + half * 8);
     }
     const int rg_first = args.plan.rg_first[wave], rg_step = args.plan.rg_step[wave];
     // launches with channel-major tiles read the rows of a group through tau (16 consecutive rows per lane)
@@ -277,7 +288,13 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         gam = ld16((const T*)d.ln_gamma + c8 * 8);
         bet = ld16((const T*)d.ln_beta + c8 * 8);
     }
+    // row mask of the launch (all masked tiles share it): fetched with the slab, kept in LDS as fp32
+    const int mt = args.plan.mask_tile;
+    const T* rm = mt >= 0 ? (const T*)d.tiles[mt].rowmask : nullptr;
+    const unsigned m_inner = mt >= 0 ? (unsigned)d.tiles[mt].inner : 1u;
+    const long m_so = mt >= 0 ? d.tiles[mt].m_so : 0, m_si = mt >= 0 ? d.tiles[mt].m_si : 0;
     Vec16<T> pre[4];
+    T pm[4];
     auto fetch = [&](int slab) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -285,10 +302,14 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             m = m < M ? m : M - 1;                       // clamped: rows past the end are never stored
             const unsigned hi = (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
             pre[i] = ld16(A + (long)hi * d.a_so + (long)lo * d.a_si + c8 * 8);
+            if (rm) {
+                const unsigned mh = (unsigned)m / m_inner, ml = (unsigned)m - mh * m_inner;
+                pm[i] = rm[(long)mh * m_so + (long)ml * m_si];
+            }
         }
     };
     auto commit = [&](int buf) {
-        unsigned char* sa = smem + buf * (WS_BM * WS_AP);
+        unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             Vec16<T> x = pre[i];
@@ -311,6 +332,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                 for (int e = 0; e < 8; ++e) x.e[e] = (T)(f[e] * rs * (float)gam.e[e] + (float)bet.e[e]);
             }
             *reinterpret_cast<Vec16<T>*>(sa + (r0 + 32 * i) * WS_AP + c8 * 16) = x;
+            if (rm && c8 == 0) s_mask[buf * WS_BM + r0 + 32 * i] = (float)pm[i];
         }
     };
 
@@ -323,44 +345,66 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     for (; slab < nslabs; slab += gridDim.x) {
         const int nxt = slab + (int)gridDim.x < nslabs ? slab + (int)gridDim.x : slab;
         fetch(nxt);                                      // in flight during the products below
-        const unsigned char* sa = smem + buf * (WS_BM * WS_AP);
+        const unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
         for (int rg = rg_first; rg < WS_RG; rg += rg_step) {
             const long m0g = (long)slab * WS_BM + rg * 32;
             if (m0g >= M) break;
-            bf16x8 af[WS_KS];
             const unsigned char* ap = sa + (rg * 32 + n32) * WS_AP + half * 16;
+            // position of this lane's row for the [row][channel] tiles; the division is redone only
+            // when a slot's tile has another `inner`
+            const long mrow = m0g + n32;
+            const bool valid = mrow < M;
+            const unsigned mc = (unsigned)(valid ? mrow : M - 1);
+            unsigned c_inner = 0, c_hi = 0, c_lo = mc;
+            const float* smk = s_mask + buf * WS_BM + rg * 32;
 #pragma unroll
-            for (int ks = 0; ks < WS_KS; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + ks * 32);
-#pragma unroll
-            for (int s = 0; s < WS_NS; ++s) {
+            for (int s = 0; s < NS; ++s) {
                 if (s_tile[s] < 0 || s_glu[s] == 2) continue;
-                const ffk_tile& t = d.tiles[s_tile[s]];
-                const bool by_rows = ws_by_rows(t);
+                const WsSlot& t = sp[s];
                 const bool glu = s_glu[s] == 1;
-                const int sg = s + 1 < WS_NS ? s + 1 : s;          // gate slot of a GLU unit (constant after unrolling)
+                const int sg = s + 1 < NS ? s + 1 : s;             // gate slot of a GLU unit (constant after unrolling)
+                const float* sb = s_bias + s_wrow[s];
+                // The A fragments are re-read from LDS for every slot: keeping them across the epilogue of
+                // the previous slot costs 32 registers, and a single spilled register puts a scratch
+                // reload with a full vector-memory wait into every epilogue.
+                bf16x8 af[WS_KS];
+                int reread = 0;
+                asm volatile("" : "+v"(reread));                   // opaque zero: keeps the compiler from reusing the loads
+#pragma unroll
+                for (int ks = 0; ks < WS_KS; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + ks * 32);
                 f32x16 acc, accg;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
-                if (by_rows) {
+                if (by_rows[s]) {
 #pragma unroll
                     for (int ks = 0; ks < WS_KS; ++ks) MM::mma(acc, wf[s][ks], af[ks]);
                     if (glu) {
 #pragma unroll
                         for (int ks = 0; ks < WS_KS; ++ks) MM::mma(accg, wf[sg][ks], af[ks]);
-                        ws_store_rows<true>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, n32, half);
-                    } else {
-                        ws_store_rows<false>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, n32, half);
                     }
+                    if (t.inner != c_inner) {
+                        c_inner = t.inner;
+                        if (c_inner < (unsigned)M) {
+                            c_hi = mc / c_inner;
+                            c_lo = mc - c_hi * c_inner;
+                        } else {
+                            c_hi = 0;
+                            c_lo = mc;
+                        }
+                    }
+                    const float rmask = t.masked ? smk[n32] : 1.0f;
+                    if (glu) ws_store_rows<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                    else ws_store_rows<false>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                 } else {
 #pragma unroll
                     for (int ks = 0; ks < WS_KS; ++ks) MM::mma(acc, af[ks], wf[s][ks]);
                     if (glu) {
 #pragma unroll
                         for (int ks = 0; ks < WS_KS; ++ks) MM::mma(accg, af[ks], wf[sg][ks]);
-                        ws_store_cols<true>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, l32, half);
-                    } else {
-                        ws_store_cols<false>(t, acc, accg, s_chb[s], s_chan[s], m0g, M, l32, half);
                     }
+                    const float* sm = t.masked ? smk : nullptr;
+                    if (glu) ws_store_cols<true>(t, acc, accg, sb, sm, m0g, M, l32, half);
+                    else ws_store_cols<false>(t, acc, accg, sb, sm, m0g, M, l32, half);
                 }
             }
         }
@@ -370,6 +414,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     }
 }
 
+// tiles stored with channels contiguous (lane = row) vs rows contiguous (lane = channel): host side
 bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (t.inner <= 0 || t.ncols <= 0 || !al16(t.out)) return false;
@@ -434,6 +479,12 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
         if (fits) break;
     }
     if (R < 1) return false;
+    p.max_slots = 0;
+    for (int g = 0; g < G; ++g) {
+        int n = 0;
+        for (int sl = 0; sl < WS_NS; ++sl) n += assign[g][sl] != -1;
+        p.max_slots = n > p.max_slots ? n : p.max_slots;
+    }
     for (int w = 0; w < WS_WAVES; ++w) {
         const int g = w % G;
         p.rg_first[w] = w / G;
@@ -460,6 +511,22 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
     return true;
 }
 
+template <int NS>
+int ws_launch(const WsArgs& args, hipStream_t st) {
+    const size_t smem = 2 * (size_t)WS_BM * WS_AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess)
+            return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
+        configured = true;
+    }
+    const int nslabs = ffk_cdiv(args.d.M, WS_BM);
+    const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
+    linear_ws_kernel<NS><<<grid, WS_THREADS, smem, st>>>(args);
+    return ffk_check_launch("ffk_fused_linear");
+}
+
 }  // namespace
 
 // Launches the weights-stationary kernel if it can take this (already validated) descriptor and
@@ -468,30 +535,27 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->dtype != FFK_BF16 || d->K != WS_K || d->a_chanmajor) return 0;
     if (getenv("FFK_NO_WS")) return 0;
     bool chan_major = false, v_tiles = false;
+    int mask_tile = -1;
     for (int i = 0; i < d->n_tiles; ++i) {
         const ffk_tile& t = d->tiles[i];
         if (!ws_tile_ok(*d, t)) return 0;
         chan_major = chan_major || (!ws_by_rows(t) && t.kind == FFK_TILE_STRIDED);
         v_tiles = v_tiles || t.kind == FFK_TILE_V;
+        if (t.rowmask) {
+            if (mask_tile < 0) {
+                mask_tile = i;
+            } else {
+                const ffk_tile& f = d->tiles[mask_tile];     // one mask per launch
+                if (t.rowmask != f.rowmask || t.inner != f.inner || t.m_so != f.m_so || t.m_si != f.m_si) return 0;
+            }
+        }
     }
     if (chan_major && v_tiles) return 0;          // they need different row orders within a group
     WsArgs args;
     if (!ws_make_plan(*d, args.plan)) return 0;
     args.plan.row_perm = chan_major ? 1 : 0;
+    args.plan.mask_tile = mask_tile;
     args.d = *d;
-    const size_t smem = 2 * (size_t)WS_BM * WS_AP;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) {
-            *status = ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
-            return 1;
-        }
-        configured = true;
-    }
-    const int nslabs = ffk_cdiv(d->M, WS_BM);
-    const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
-    linear_ws_kernel<<<grid, WS_THREADS, smem, st>>>(args);
-    *status = ffk_check_launch("ffk_fused_linear");
+    *status = args.plan.max_slots <= 2 ? ws_launch<2>(args, st) : ws_launch<3>(args, st);
     return 1;
 }
