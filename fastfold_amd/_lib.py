@@ -239,6 +239,14 @@ def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H
          B2, H, Nq, Nk, FFK_ATT_GATE_TILED if gate_tiled else 0, dtype_tag(q_t.dtype), stream_ptr())
 
 
+SIGNATURES["ffk_pair_bias"] = [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _F, _F, _I, _P]
+
+
+def pair_bias(bias_t, z, gamma, beta, w, scratch, *, N, C, H, a_inner, a_so, a_si, scale, eps=1e-5):
+    call("ffk_pair_bias", ptr(bias_t), ptr(z), ptr(gamma), ptr(beta), ptr(w), ptr(scratch), N, C, H, a_inner, a_so, a_si,
+         scale, eps, dtype_tag(z.dtype), stream_ptr())
+
+
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):
     call("ffk_key_bias", ptr(keybias), ptr(tileflags), ptr(mask), B, N, mask_sb, mask_sn,
          dtype_tag(mask.dtype) if mask is not None else FFK_F32, stream_ptr())

@@ -161,9 +161,10 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         tiles.append(bias_tile)
         bias_tile = None
     _lib.fused_linear(x, w_pk, tiles, M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln)
-    if bias_tile is not None:      # the bias tile has its own pass (it needs the LDS-staged kernel)
-        _lib.fused_linear(x, w_pk, [bias_tile], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
-                          w_row_off=4 * tpg * 128)
+    if bias_tile is not None:      # the skinny bias projection has its own pass over x
+        scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=dev)
+        _lib.pair_bias(bias_t, x, ln[0], ln[1], w_pk[4 * tpg * 128:], scratch, N=N, C=C, H=H, a_inner=a_inner,
+                       a_so=a_so, a_si=a_si, scale=LOG2E)
     kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
     flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
     _lib.key_bias(kb, flags, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
@@ -184,6 +185,11 @@ def pair_bias(z, *, r, C, H, ln, wb_pk):
     """bias_t[h][q/32][k/32][tile] = log2e * (LN(z)[q, k, :] . Wb[h, :]) in score-accumulator tiles."""
     NT = (r + 31) // 32
     bias_t = alloc((H, NT, NT, 1024), z.dtype, z.device, zero=(r % 32) != 0)
+    if z.dtype == torch.bfloat16 and C == 128 and H <= 8:
+        scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=z.device)
+        _lib.pair_bias(bias_t, z, ln[0], ln[1], wb_pk, scratch, N=r, C=C, H=H, a_inner=r * r, a_so=0, a_si=C,
+                       scale=LOG2E)
+        return bias_t
     tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=r, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H, scale=LOG2E)
     _lib.fused_linear(z, wb_pk, [tile], M=r * r, K=C, ln=ln)
     return bias_t

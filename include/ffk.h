@@ -233,6 +233,19 @@ int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v
                       const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
                       int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int flags, int dtype, void* stream);
 
+/* Pair bias of a biased attention, straight into the operand tiles ffk_attention_fwd reads:
+ *     bias_t[h][q/32][k/32][tile(k, q)] = scale * ( LayerNorm(z[q, k, :]; gamma, beta, eps) . w[h, :] )
+ * z holds N*N rows of C channels; logical row m = q*N + k lives at (m / a_inner) * a_so + (m % a_inner) * a_si
+ * (elements), which also expresses the transposed traversal of the ending-node attention.
+ * w is [H][C], H <= 8; bias_t is [H][ceil(N/32)][ceil(N/32)][1024] in FFK_TILE_BIAS order and must be
+ * zero-filled by the caller when N is not a multiple of 32; scratch is caller-owned device memory of
+ * at least (H*C + 2*H) floats.  bf16, C = 128.
+ * Replaces: F.linear(LayerNorm(Z), linear_b_weights) and its permute / unsqueeze
+ * (fastfold/model/fastnn/msa.py:61-66, ops.py:659-664,890-896). */
+int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w,
+                  float* scratch, int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so,
+                  int64_t a_si, float scale, float eps, int dtype, void* stream);
+
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the
  * given dtype, or NULL (all keys valid).  tileflags[b, k/32] classifies each 32-key tile (see

@@ -305,3 +305,30 @@ def test_weights_stationary_matches_other_variant(dev, monkeypatch):
     for a, b in zip(*outs):
         assert float(a.float().abs().max()) > 0.1
         assert _rel(_np(a), _np(b)) < 1e-2
+
+
+@pytest.mark.parametrize("r,H", [(45, 4), (64, 8), (96, 4)])
+def test_pair_bias_kernel(dev, r, H):
+    """ffk_pair_bias (bf16): LayerNorm + H-row projection written as attention bias tiles, in both
+    traversal orders, against float64 numpy."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    dtype, C = torch.bfloat16, 128
+    g = torch.Generator().manual_seed(r + H)
+    z = (torch.randn(r, r, C, generator=g) * 1.5 + 0.4).to(dev, dtype)
+    wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    T = layouts.n_tiles(r)
+    scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=dev)
+    for transposed in (False, True):
+        bt = torch.zeros(H, T, T, 2, 32, 16, dtype=dtype, device=dev)
+        kw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else dict(a_inner=r * r, a_so=0, a_si=C)
+        _lib.pair_bias(bt, z, gam, bet, wb, scratch, N=r, C=C, H=H, scale=_lib.LOG2E, **kw)
+        zz = _np(z).transpose(1, 0, 2) if transposed else _np(z)
+        x = ops_np.layer_norm(zz, _np(gam), _np(bet))
+        ref = (ops_np.linear(x, _np(wb)) * _lib.LOG2E).transpose(2, 0, 1)       # [h, q, k]
+        assert _rel(_np(layouts.untile_bias(bt, r, r)), ref) < TOL[dtype]
+        # padding of ragged tiles is left untouched (zero)
+        full = _np(layouts.untile_bias(bt, T * 32, T * 32))
+        assert np.abs(full[:, r:, :]).max(initial=0.0) == 0.0 and np.abs(full[:, :, r:]).max(initial=0.0) == 0.0
