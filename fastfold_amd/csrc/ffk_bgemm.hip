@@ -264,6 +264,10 @@ extern "C" int ffk_bgemm_nt(const ffk_bgemm_desc* d, void* stream) {
                     d->a_bs % vec == 0 && d->b_bs % vec == 0,
                 FFK_ERR_ALIGN, "ffk_bgemm_nt: operand rows must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
+    {
+        int status = FFK_OK;
+        if (ffk_bgemm_big_try(d, st, &status)) return status;
+    }
     if (d->dtype == FFK_BF16) {
         return d->out_f32 ? launch_bgemm<bf16_t, float>(*d, st) : launch_bgemm<bf16_t, bf16_t>(*d, st);
     } else if (d->dtype == FFK_F32) {

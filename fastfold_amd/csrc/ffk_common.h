@@ -21,6 +21,7 @@ int ffk_fail(int code, const char* fmt, ...);
     } while (0)
 
 int ffk_linear_slab_launch(const ffk_linear_desc* d, hipStream_t st);   // ffk_linear_slab.hip
+int ffk_bgemm_big_try(const ffk_bgemm_desc* d, hipStream_t st, int* status);    // ffk_bgemm_big.hip
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status);   // ffk_linear_ws.hip
 
 static inline bool ffk_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
