@@ -1,6 +1,6 @@
 // Weights-stationary variant of the fused linear layer (see ffk_fused_linear in include/ffk.h),
-// bf16, K = 128: the projections of the pair stack, where M is ~10^6 rows and the whole weight
-// matrix is a few hundred KB.
+// bf16, K = 128 or 256: the projections of the pair and MSA stacks, where M is 10^5 .. 10^6 rows and
+// the whole weight matrix is a few hundred KB.
 //
 // One persistent workgroup of 8 wavefronts per CU.  The weight matrix is split into "slots" of 32
 // output rows; every wave keeps the MFMA fragments of up to three slots in registers for the whole
@@ -23,13 +23,17 @@ namespace {
 
 constexpr int WS_WAVES = 8;
 constexpr int WS_THREADS = 64 * WS_WAVES;
-constexpr int WS_BM = 128;               // rows per slab
-constexpr int WS_RG = WS_BM / 32;        // 32-row groups per slab
-constexpr int WS_NS = 3;                 // weight slots per wave
-constexpr int WS_K = 128;
-constexpr int WS_KS = WS_K / 16;         // MFMA K steps
-constexpr int WS_AP = WS_K * 2 + 16;     // LDS row pitch in bytes
+constexpr int WS_NS = 3;                 // weight slots per wave (two with K = 256, where a slot costs 64 registers)
 constexpr int WS_MAX_GRID = 256;         // one workgroup per CU
+// Per-K geometry: a slab is as many rows as 512 threads fetch with four 16-byte loads each.
+template <int K> struct WsGeo {
+    static constexpr int KS = K / 16;                // MFMA K steps
+    static constexpr int AP = K * 2 + 16;            // LDS row pitch in bytes
+    static constexpr int LPR = K / 8;                // lanes (16-byte vectors) per row
+    static constexpr int RPP = WS_THREADS / LPR;     // rows fetched per pass
+    static constexpr int BM = 4 * RPP;               // rows per slab: 128 (K = 128) or 64 (K = 256)
+    static constexpr int RG = BM / 32;               // 32-row groups per slab
+};
 
 typedef bf16_t T;
 
@@ -221,9 +225,13 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
     }
 }
 
-template <int NS>
+template <int NS, int WS_K>
 __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs args) {
     typedef Mma<T> MM;
+    typedef WsGeo<WS_K> G;
+    constexpr int WS_KS = G::KS, WS_AP = G::AP, WS_BM = G::BM, WS_RG = G::RG, LPR = G::LPR, RPP = G::RPP;
+    constexpr bool ALLOW_GLU = NS >= 2 && WS_K == 128;
+    constexpr int AFC = WS_K == 128 ? 8 : 4;               // A fragments held at a time (register budget)
     const ffk_linear_desc& d = args.d;
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* s_a = smem;                                                 // [2][WS_BM][WS_AP]
@@ -280,8 +288,8 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     // launches with channel-major tiles read the rows of a group through tau (16 consecutive rows per lane)
     const int n32 = args.plan.row_perm ? ws_tau(l32) : l32;
 
-    // ---- slab streaming: thread -> (row tid/16 + 32 i, 8 channels starting at 8 * (tid % 16)) ----
-    const int c8 = tid & 15, r0 = tid >> 4;
+    // ---- slab streaming: thread -> (row tid / LPR + RPP * i, 8 channels starting at 8 * (tid % LPR)) ----
+    const int c8 = tid % LPR, r0 = tid / LPR;
     const bool ln = d.ln_gamma != nullptr;
     Vec16<T> gam, bet;                                   // kept packed: registers are scarce here
     if (ln) {
@@ -298,7 +306,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     auto fetch = [&](int slab) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            long m = (long)slab * WS_BM + r0 + 32 * i;
+            long m = (long)slab * WS_BM + r0 + RPP * i;
             m = m < M ? m : M - 1;                       // clamped: rows past the end are never stored
             const unsigned hi = (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
             pre[i] = ld16(A + (long)hi * d.a_so + (long)lo * d.a_si + c8 * 8);
@@ -320,19 +328,19 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                     f[e] = (float)x.e[e];
                     s += f[e];
                 }
-                const float mu = group_sum(s, 16) * (1.0f / WS_K);
+                const float mu = group_sum(s, LPR) * (1.0f / WS_K);
                 float q = 0.0f;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     f[e] -= mu;
                     q += f[e] * f[e];
                 }
-                const float rs = rsqrtf(group_sum(q, 16) * (1.0f / WS_K) + d.ln_eps);
+                const float rs = rsqrtf(group_sum(q, LPR) * (1.0f / WS_K) + d.ln_eps);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) x.e[e] = (T)(f[e] * rs * (float)gam.e[e] + (float)bet.e[e]);
             }
-            *reinterpret_cast<Vec16<T>*>(sa + (r0 + 32 * i) * WS_AP + c8 * 16) = x;
-            if (rm && c8 == 0) s_mask[buf * WS_BM + r0 + 32 * i] = (float)pm[i];
+            *reinterpret_cast<Vec16<T>*>(sa + (r0 + RPP * i) * WS_AP + c8 * 16) = x;
+            if (rm && c8 == 0) s_mask[buf * WS_BM + r0 + RPP * i] = (float)pm[i];
         }
     };
 
@@ -367,21 +375,34 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                 // The A fragments are re-read from LDS for every slot: keeping them across the epilogue of
                 // the previous slot costs 32 registers, and a single spilled register puts a scratch
                 // reload with a full vector-memory wait into every epilogue.
-                bf16x8 af[WS_KS];
                 int reread = 0;
                 asm volatile("" : "+v"(reread));                   // opaque zero: keeps the compiler from reusing the loads
-#pragma unroll
-                for (int ks = 0; ks < WS_KS; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + ks * 32);
                 f32x16 acc, accg;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
-                if (by_rows[s]) {
+                const bool rows = by_rows[s];
 #pragma unroll
-                    for (int ks = 0; ks < WS_KS; ++ks) MM::mma(acc, wf[s][ks], af[ks]);
-                    if (glu) {
+                for (int k0 = 0; k0 < WS_KS; k0 += AFC) {          // AFC K steps of A in registers at a time
+                    bf16x8 af[AFC];
 #pragma unroll
-                        for (int ks = 0; ks < WS_KS; ++ks) MM::mma(accg, wf[sg][ks], af[ks]);
+                    for (int ks = 0; ks < AFC; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + (k0 + ks) * 32);
+                    if (rows) {
+#pragma unroll
+                        for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, wf[s][k0 + ks], af[ks]);
+                        if (ALLOW_GLU && glu) {
+#pragma unroll
+                            for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, af[ks], wf[s][k0 + ks]);
+                        if (ALLOW_GLU && glu) {
+#pragma unroll
+                            for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, af[ks], wf[sg][k0 + ks]);
+                        }
                     }
+                }
+                if (rows) {
                     if (t.inner != c_inner) {
                         c_inner = t.inner;
                         if (c_inner < (unsigned)M) {
@@ -393,17 +414,11 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                         }
                     }
                     const float rmask = t.masked ? smk[n32] : 1.0f;
-                    if (glu) ws_store_rows<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                    if (ALLOW_GLU && glu) ws_store_rows<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                     else ws_store_rows<false>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                 } else {
-#pragma unroll
-                    for (int ks = 0; ks < WS_KS; ++ks) MM::mma(acc, af[ks], wf[s][ks]);
-                    if (glu) {
-#pragma unroll
-                        for (int ks = 0; ks < WS_KS; ++ks) MM::mma(accg, af[ks], wf[sg][ks]);
-                    }
                     const float* sm = t.masked ? smk : nullptr;
-                    if (glu) ws_store_cols<true>(t, acc, accg, sb, sm, m0g, M, l32, half);
+                    if (ALLOW_GLU && glu) ws_store_cols<true>(t, acc, accg, sb, sm, m0g, M, l32, half);
                     else ws_store_cols<false>(t, acc, accg, sb, sm, m0g, M, l32, half);
                 }
             }
@@ -437,7 +452,7 @@ bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
 // Distributes the 32-row weight units over the waves.  The waves form G = 8 / R groups; the R waves
 // of a group hold the same units and take every R-th row group of a slab (R as large as the units
 // allow, so that few units still use all eight waves).  Returns false if the units do not fit.
-bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
+bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p, int rg_per_slab, int max_ns) {
     struct Unit { int tile, chan, wrow, slots; };
     Unit units[FFK_MAX_TILES * 4];
     int nu = 0;
@@ -455,7 +470,7 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
     }
     int assign[WS_WAVES][WS_NS];
     int G = 0, R = 0;
-    for (R = WS_RG; R >= 1; R >>= 1) {
+    for (R = rg_per_slab; R >= 1; R >>= 1) {
         G = WS_WAVES / R;
         int load[WS_WAVES] = {0};
         for (int g = 0; g < G; ++g)
@@ -466,7 +481,7 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
                 if (units[i].slots != pass) continue;
                 int best = -1;
                 for (int g = 0; g < G; ++g)
-                    if (load[g] + pass <= WS_NS && (best < 0 || load[g] < load[best])) best = g;
+                    if (load[g] + pass <= max_ns && (best < 0 || load[g] < load[best])) best = g;
                 if (best < 0) {
                     fits = false;
                     break;
@@ -511,19 +526,20 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p) {
     return true;
 }
 
-template <int NS>
+template <int NS, int K>
 int ws_launch(const WsArgs& args, hipStream_t st) {
-    const size_t smem = 2 * (size_t)WS_BM * WS_AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float);
+    constexpr int WS_BM = WsGeo<K>::BM;
+    const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess)
             return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
         configured = true;
     }
     const int nslabs = ffk_cdiv(args.d.M, WS_BM);
     const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
-    linear_ws_kernel<NS><<<grid, WS_THREADS, smem, st>>>(args);
+    linear_ws_kernel<NS, K><<<grid, WS_THREADS, smem, st>>>(args);
     return ffk_check_launch("ffk_fused_linear");
 }
 
@@ -532,7 +548,8 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
 // Launches the weights-stationary kernel if it can take this (already validated) descriptor and
 // returns 1 with the launch status in *status; returns 0 if the caller has to use another variant.
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
-    if (d->dtype != FFK_BF16 || d->K != WS_K || d->a_chanmajor) return 0;
+    if (d->dtype != FFK_BF16 || (d->K != 128 && d->K != 256) || d->a_chanmajor) return 0;
+    const bool k256 = d->K == 256;
     if (getenv("FFK_NO_WS")) return 0;
     bool chan_major = false, v_tiles = false;
     int mask_tile = -1;
@@ -552,10 +569,15 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     }
     if (chan_major && v_tiles) return 0;          // they need different row orders within a group
     WsArgs args;
-    if (!ws_make_plan(*d, args.plan)) return 0;
+    if (!ws_make_plan(*d, args.plan, k256 ? WsGeo<256>::RG : WsGeo<128>::RG, k256 ? 2 : WS_NS)) return 0;
+    if (k256) {
+        for (int i = 0; i < d->n_tiles; ++i)
+            if (d->tiles[i].glu) return 0;                   // GLU units are only built for K = 128
+    }
     args.plan.row_perm = chan_major ? 1 : 0;
     args.plan.mask_tile = mask_tile;
     args.d = *d;
-    *status = args.plan.max_slots <= 2 ? ws_launch<2>(args, st) : ws_launch<3>(args, st);
+    if (k256) *status = ws_launch<2, 256>(args, st);
+    else *status = args.plan.max_slots <= 2 ? ws_launch<2, 128>(args, st) : ws_launch<3, 128>(args, st);
     return 1;
 }

@@ -101,10 +101,11 @@ def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
     nt = hidden // 128
     for r0 in range(0, M, rows):
         n = min(rows, M - r0)
-        for t0 in range(0, nt, _lib.FFK_MAX_TILES):
+        per = 4 if (dt == torch.bfloat16 and C == 256) else _lib.FFK_MAX_TILES
+        for t0 in range(0, nt, per):
             tiles = [make_tile(hid.data_ptr() + t * 128 * es, bias=b1_pk.data_ptr() + t * 128 * es, inner=n,
                                s_i=hidden, act=FFK_ACT_RELU)
-                     for t in range(t0, min(nt, t0 + _lib.FFK_MAX_TILES))]
+                     for t in range(t0, min(nt, t0 + per))]
             _lib.fused_linear(x, w1_pk, tiles, M=n, K=C, ln=ln, a_off=r0 * C, w_row_off=t0 * 128)
         _lib.bgemm_nt(hid, w2, out.data_ptr() + r0 * C * es, M=n, N=C, K=hidden, lda=hidden, ldb=hidden, bias=b2,
                       resid=x.data_ptr() + r0 * C * es, dtype=dt)
@@ -135,7 +136,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     v_t = alloc((B2, H, NT, 1024), dt, dev, zero)
     # With bf16, 128 input channels and whole key tiles the projection runs on the weights-stationary
     # kernel, which writes q, k and the gate in accumulator order straight from its registers.
-    acc_order = dt == torch.bfloat16 and C == 128 and N % 32 == 0
+    acc_order = dt == torch.bfloat16 and C in (128, 256) and N % 32 == 0
     qk_kind = FFK_TILE_ACC if acc_order else FFK_TILE_QK
     gate = torch.empty((B2, H, NT, 1024) if acc_order else (M, HC), dtype=dt, device=dev)
     tpg = HC // 128
@@ -160,7 +161,11 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     if bias_tile is not None and not acc_order:
         tiles.append(bias_tile)
         bias_tile = None
-    _lib.fused_linear(x, w_pk, tiles, M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln)
+    # the weights-stationary kernel holds at most 16 (K = 256) or 24 (K = 128) 32-channel units per launch
+    per = 4 if (acc_order and C == 256) else len(tiles)
+    for t0 in range(0, len(tiles), per):
+        _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
+                          w_row_off=t0 * 128)
     if bias_tile is not None:      # the skinny bias projection has its own pass over x
         scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=dev)
         _lib.pair_bias(bias_t, x, ln[0], ln[1], w_pk[4 * tpg * 128:], scratch, N=N, C=C, H=H, a_inner=a_inner,
