@@ -225,7 +225,7 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
     }
 }
 
-template <int NS, int WS_K>
+template <int NS, int WS_K, bool CM>
 __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs args) {
     typedef Mma<T> MM;
     typedef WsGeo<WS_K> G;
@@ -292,9 +292,17 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const int c8 = tid % LPR, r0 = tid / LPR;
     const bool ln = d.ln_gamma != nullptr;
     Vec16<T> gam, bet;                                   // kept packed: registers are scarce here
-    if (ln) {
+    float cm_g[4], cm_b[4];                              // channel-major A: gamma / beta of this lane's four channels
+    if (ln && !CM) {
         gam = ld16((const T*)d.ln_gamma + c8 * 8);
         bet = ld16((const T*)d.ln_beta + c8 * 8);
+    }
+    if (ln && CM) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            cm_g[i] = (float)((const T*)d.ln_gamma)[(lane & 31) + 32 * i];
+            cm_b[i] = (float)((const T*)d.ln_beta)[(lane & 31) + 32 * i];
+        }
     }
     // row mask of the launch (all masked tiles share it): fetched with the slab, kept in LDS as fp32
     const int mt = args.plan.mask_tile;
@@ -303,7 +311,21 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const long m_so = mt >= 0 ? d.tiles[mt].m_so : 0, m_si = mt >= 0 ? d.tiles[mt].m_si : 0;
     Vec16<T> pre[4];
     T pm[4];
+    // Channel-major A (element (m, k) at a + k * a_cs + rowoffset(m), K = 128): a thread fetches eight
+    // consecutive rows of channel k = lane % 32 + 32 i; the two half-waves of wave w own the row groups
+    // 2w and 2w + 1 of the slab, so the LayerNorm reduction over k stays inside 32 lanes.  The slab is
+    // transposed on its way into LDS (2-byte stores, consecutive lanes -> consecutive k of one row).
+    const int cm_k = lane & 31, cm_mg = 2 * wave + (lane >> 5);
     auto fetch = [&](int slab) {
+        if (CM) {
+            long m = (long)slab * WS_BM + cm_mg * 8;
+            m = m < M ? m : M - 8;                       // M % 8 == 0; clamped groups are never stored
+            const unsigned hi = (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
+            const T* base = A + (long)hi * d.a_so + lo;  // a_si == 1
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pre[i] = ld16(base + (long)(cm_k + 32 * i) * d.a_cs);
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             long m = (long)slab * WS_BM + r0 + RPP * i;
@@ -318,6 +340,34 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     };
     auto commit = [&](int buf) {
         unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
+        if (CM) {
+            float f[4][8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[i][j] = (float)pre[i].e[j];
+            if (ln) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float mu = group_sum((f[0][j] + f[1][j]) + (f[2][j] + f[3][j]), 32) * (1.0f / WS_K);
+                    float q = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        f[i][j] -= mu;
+                        q += f[i][j] * f[i][j];
+                    }
+                    const float rs = rsqrtf(group_sum(q, 32) * (1.0f / WS_K) + d.ln_eps);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) f[i][j] = f[i][j] * rs * cm_g[i] + cm_b[i];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    *reinterpret_cast<T*>(sa + (cm_mg * 8 + j) * WS_AP + (cm_k + 32 * i) * 2) = (T)f[i][j];
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             Vec16<T> x = pre[i];
@@ -526,20 +576,20 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p, int rg_per_slab, int max_
     return true;
 }
 
-template <int NS, int K>
+template <int NS, int K, bool CM>
 int ws_launch(const WsArgs& args, hipStream_t st) {
     constexpr int WS_BM = WsGeo<K>::BM;
     const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K, CM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess)
             return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
         configured = true;
     }
     const int nslabs = ffk_cdiv(args.d.M, WS_BM);
     const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
-    linear_ws_kernel<NS, K><<<grid, WS_THREADS, smem, st>>>(args);
+    linear_ws_kernel<NS, K, CM><<<grid, WS_THREADS, smem, st>>>(args);
     return ffk_check_launch("ffk_fused_linear");
 }
 
@@ -548,7 +598,8 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
 // Launches the weights-stationary kernel if it can take this (already validated) descriptor and
 // returns 1 with the launch status in *status; returns 0 if the caller has to use another variant.
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
-    if (d->dtype != FFK_BF16 || (d->K != 128 && d->K != 256) || d->a_chanmajor) return 0;
+    if (d->dtype != FFK_BF16 || (d->K != 128 && d->K != 256)) return 0;
+    if (d->a_chanmajor && (d->K != 128 || d->a_si != 1 || d->a_inner % 8 || d->a_so % 8 || d->a_cs % 8 || d->M % 8)) return 0;
     const bool k256 = d->K == 256;
     if (getenv("FFK_NO_WS")) return 0;
     bool chan_major = false, v_tiles = false;
@@ -577,7 +628,13 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     args.plan.row_perm = chan_major ? 1 : 0;
     args.plan.mask_tile = mask_tile;
     args.d = *d;
-    if (k256) *status = ws_launch<2, 256>(args, st);
-    else *status = args.plan.max_slots <= 2 ? ws_launch<2, 128>(args, st) : ws_launch<3, 128>(args, st);
+    if (d->a_chanmajor) {
+        if (args.plan.max_slots > 2 || mask_tile >= 0) return 0;
+        *status = ws_launch<2, 128, true>(args, st);
+    } else if (k256) {
+        *status = ws_launch<2, 256, false>(args, st);
+    } else {
+        *status = args.plan.max_slots <= 2 ? ws_launch<2, 128, false>(args, st) : ws_launch<3, 128, false>(args, st);
+    }
     return 1;
 }

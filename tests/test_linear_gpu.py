@@ -184,7 +184,7 @@ def test_bias_tiles(dev, dtype, r, H):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("r", [40, 27])
+@pytest.mark.parametrize("r", [40, 27, 104])
 def test_channel_major_a_with_layernorm(dev, dtype, r):
     """Triangle-multiplication output stage: A[(i,j), c] = P[c][i][jpad]."""
     from fastfold_amd import _lib
