@@ -50,53 +50,69 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
     const int l32 = lane & 31, half = lane >> 5;
     const int M = d.M, N = d.N, K = d.K;
 
-    // workgroup -> tile (batched launches: every XCD takes a contiguous eighth of the tile order)
     const unsigned tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    unsigned item = blockIdx.x;
-    if (d.batch >= 8) {
-        const unsigned total = tiles_m * tiles_n * (unsigned)d.batch, per_xcd = (total + 7) >> 3;
-        item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-        if (item >= total) return;
-    }
-    const long m0 = (long)(item % tiles_m) * BM, n0 = (long)((item / tiles_m) % tiles_n) * BN;
-    const int bz = (item / tiles_m) / tiles_n;
-    const T* A = (const T*)d.a + (long)bz * d.a_bs;
-    const T* B = (const T*)d.b + (long)bz * d.b_bs;
+    const unsigned total = tiles_m * tiles_n * (unsigned)d.batch;
+    const int kchunks = K / BG_BK;
 
-    // ---- loader set-up ----
+    // Persistent workgroups.  Tile t of this workgroup: batched launches give every XCD a contiguous
+    // eighth of the (batch, n-tile, m-tile) order (consecutive workgroup ids go to the eight XCDs in turn,
+    // each with its own L2), so that all tiles of a batch run behind one L2; otherwise tiles are dealt
+    // round-robin.  Returns false past the end.
+    auto tile_at = [&](unsigned t, unsigned& item) {
+        if (d.batch >= 8) {
+            const unsigned per_xcd = (total + 7) >> 3, xcd = blockIdx.x & 7;
+            const unsigned j = (blockIdx.x >> 3) + (gridDim.x >> 3) * t;
+            item = xcd * per_xcd + j;
+            return j < per_xcd && item < total;
+        }
+        item = blockIdx.x + gridDim.x * t;
+        return item < total;
+    };
+
+    // ---- loader ----
     // Load i of a thread fills LDS position (row i*128 + wave*16 + lane/4, column lane%4) of a slot.
     // Rows 0..255 are A rows, the rest B rows.  Rows are unpadded, so to keep the fragment reads free of
     // bank conflicts position (row, c) holds global column  c ^ ((row >> 2) & 3)  of the chunk.
+    // The chunk stream runs on across tiles: while the last chunks of one tile are multiplied and its
+    // results stored, the first chunks of the next tile are already arriving.
     const T* src[NLD];
+    unsigned f_t = 0;          // tile (of this workgroup) being fetched
+    int f_kc = 0;              // next chunk of it
+    unsigned g_fetch = 0;      // running chunk count -> ring slot
+    auto fetch_setup = [&](unsigned item) {
+        const long fm0 = (long)(item % tiles_m) * BM, fn0 = (long)((item / tiles_m) % tiles_n) * BN;
+        const int fbz = (item / tiles_m) / tiles_n;
+        const T* A = (const T*)d.a + (long)fbz * d.a_bs;
+        const T* B = (const T*)d.b + (long)fbz * d.b_bs;
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-        const int row = i * 128 + wave * 16 + (lane >> 2);
-        const int g = (lane & 3) ^ ((row >> 2) & 3);
-        if (i < BM / 128) {
-            long m = m0 + row;
-            m = m < M ? m : M - 1;                           // clamped once; such rows are never stored
-            src[i] = A + m * d.lda + g * 8;
-        } else {
-            long n = n0 + row - BM;
-            n = n < N ? n : N - 1;
-            src[i] = B + n * d.ldb + g * 8;
+        for (int i = 0; i < NLD; ++i) {
+            const int row = i * 128 + wave * 16 + (lane >> 2);
+            const int g = (lane & 3) ^ ((row >> 2) & 3);
+            if (i < BM / 128) {
+                long m = fm0 + row;
+                m = m < M ? m : M - 1;                       // clamped once; such rows are never stored
+                src[i] = A + m * d.lda + g * 8;
+            } else {
+                long n = fn0 + row - BM;
+                n = n < N ? n : N - 1;
+                src[i] = B + n * d.ldb + g * 8;
+            }
         }
-    }
-    const int kchunks = K / BG_BK;
-    auto fetch = [&](int kc) {
-        const int kk = (kc < kchunks ? kc : kchunks - 1) * BG_BK;   // past the end: harmless re-read into a free slot
-        unsigned char* slot = smem + (kc & (BG_SLOTS - 1)) * SLOT + wave * 1024;
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) bg_load_lds(src[i] + kk, slot + i * 8192);
     };
-
-    f32x16 acc[NI][2];   // [ni][mi]
+    auto fetch_next = [&]() {
+        unsigned char* slot = smem + (g_fetch & (BG_SLOTS - 1)) * SLOT + wave * 1024;
 #pragma unroll
-    for (int a = 0; a < NI; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+        for (int i = 0; i < NLD; ++i) bg_load_lds(src[i] + f_kc * BG_BK, slot + i * 8192);
+        ++g_fetch;
+        if (++f_kc == kchunks) {                             // on to the next tile; past the last one the
+            unsigned item;                                   // same chunks are re-read into free slots (harmless)
+            f_kc = 0;
+            if (tile_at(f_t + 1, item)) {
+                ++f_t;
+                fetch_setup(item);
+            }
+        }
+    };
 
     // fragment addresses: A rows in natural order, B rows through tau; column (2 ks + half) un-swizzled
     const int ra = wm * 64 + l32, rb = BM + wn * WTN + bg_tau(l32);
@@ -107,30 +123,54 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
         fb_off[ks] = rb * 64 + (((2 * ks + half) ^ ((rb >> 2) & 3)) << 4);
     }
 
-    fetch(0);
-    fetch(1);
-    fetch(2);
-    for (int kc = 0; kc < kchunks; ++kc) {
-        // chunk kc has landed once at most the loads of the two younger chunks are outstanding
-        if (NLD == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-        __builtin_amdgcn_s_barrier();                        // ... for every wave; slot (kc - 1) % 4 is free again
-        fetch(kc + 3);
-        const unsigned char* s = smem + (kc & (BG_SLOTS - 1)) * SLOT;
+    unsigned item;
+    if (!tile_at(0, item)) return;                           // whole workgroup leaves together
+    fetch_setup(item);
+    fetch_next();
+    fetch_next();
+    fetch_next();
+    unsigned g_use = 0;
+    bool relaxed = false;      // previous tile was full: its stores are counted exactly
+    for (unsigned t = 0; tile_at(t, item); ++t) {
+        const long m0 = (long)(item % tiles_m) * BM, n0 = (long)((item / tiles_m) % tiles_n) * BN;
+        const int bz = (item / tiles_m) / tiles_n;
+        f32x16 acc[NI][2];   // [ni][mi]
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            bf16x8 fa[2], fb[NI];
+        for (int a = 0; a < NI; ++a)
 #pragma unroll
-            for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(s + fa_off[ks] + i * 32 * 64);
+            for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int i = 0; i < NI; ++i) fb[i] = *reinterpret_cast<const bf16x8*>(s + fb_off[ks] + i * 32 * 64);
+                for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+
+        for (int kc = 0; kc < kchunks; ++kc, ++g_use) {
+            // the chunk in use has landed once at most the loads of the two younger chunks are outstanding
+            // (stores of the previous tile's results are younger still)
+            // Right after a tile whose every store was issued (a full tile: no lane predicate can have
+            // skipped one), those 4 * NI stores are known to be younger than the chunks still awaited
+            // and need not be waited for.
+            if (relaxed && kc < 3) {
+                if (NLD == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+            } else {
+                if (NLD == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();                    // ... for every wave; the slot used last step is free again
+            fetch_next();
+            const unsigned char* s = smem + (g_use & (BG_SLOTS - 1)) * SLOT;
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni)
+            for (int ks = 0; ks < 2; ++ks) {
+                bf16x8 fa[2], fb[NI];
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
+                for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(s + fa_off[ks] + i * 32 * 64);
+#pragma unroll
+                for (int i = 0; i < NI; ++i) fb[i] = *reinterpret_cast<const bf16x8*>(s + fb_off[ks] + i * 32 * 64);
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
+            }
         }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the re-reads past the end
 
     // ---- epilogue from registers: lane = row, registers = 16 consecutive columns ----
     T* out = (T*)d.out + (long)bz * d.o_bs;
@@ -180,6 +220,9 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             if (ok1) *reinterpret_cast<u32x4*>(out + o + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
     }
+        relaxed = m0 + BM <= M && n0 + BN <= N;
+    }   // tiles
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the re-reads past the end
 }
 
 template <int WTN>
@@ -194,7 +237,7 @@ int bg_launch(const ffk_bgemm_desc& d, hipStream_t st) {
     }
     const long tiles = (long)ffk_cdiv(d.M, BM) * ffk_cdiv(d.N, BN) * d.batch;
     if (tiles >= (1L << 31) - 8) return ffk_fail(FFK_ERR_SHAPE, "ffk_bgemm_nt: %ld output tiles exceed the grid limit", tiles);
-    const unsigned grid = (unsigned)(d.batch >= 8 ? 8 * ffk_cdiv(tiles, 8) : tiles);
+    const unsigned grid = (unsigned)(tiles < 256 ? 8 * ffk_cdiv(tiles, 8) : 256);   // persistent: one workgroup per CU
     bgemm_big_kernel<WTN><<<grid, BG_THREADS, smem, st>>>(d);
     return ffk_check_launch("ffk_bgemm_nt");
 }
