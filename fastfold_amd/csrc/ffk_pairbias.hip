@@ -2,13 +2,17 @@
 //     bias_t[h][q/32][k/32][tile(k, q)] = scale * ( LayerNorm(z[q, k, :]) . w[h, :] )
 // written directly in the keys x queries operand tiles the attention kernel consumes.
 //
-// The op is a skinny projection (C = 128 channels -> H <= 8 heads), far too thin for the matrix
-// pipe and purely HBM-bound (one read of z).  One workgroup owns a 32 x 32 block of (q, k) and walks
-// it in four 16 x 16 quarter blocks: the 256 rows of a quarter are fetched with 16 lanes per row
-// (coalesced 256-byte rows, 16 loads in flight per thread) into LDS, then every thread finishes one
-// whole row on its own - statistics, normalisation folded into the dot products - so there is no
-// cross-lane reduction at all.  Thread t of a quarter owns the row whose tile offset is t, which
-// makes the 2-byte stores of a wave contiguous.
+// The op is a skinny projection (C = 128 channels -> H <= 8 heads) and purely HBM-bound (one read of
+// z).  One workgroup owns a 32 x 32 block of (q, k) and walks it in four 16 x 16 quarter blocks: the
+// 256 rows of a quarter are fetched with 16 lanes per row (coalesced 256-byte rows, 16 loads in
+// flight per thread, the next quarter's loads issued before this one is finished) into LDS.  The
+// LayerNorm is folded into the projection,
+//     LN(x) . w = rstd * ( x . (w * gamma)  -  mean * sum(w * gamma) ) + w . beta,
+// so the raw bf16 rows are the MFMA operand: each wave multiplies two 32-row groups against a
+// 32-row weight operand held in registers whose rows 0 .. H-1 are w * gamma and rows 8 and 12 all
+// ones (they deliver sum(x) to both half-waves); sum(x^2) comes from the loader lanes.  Lane l of a
+// group owns row l, whose tile offset is its index in the quarter, so the 2-byte stores of a wave
+// are contiguous.
 #include "ffk_common.h"
 
 namespace {
@@ -18,27 +22,41 @@ constexpr int PB_MAXH = 8;
 
 template <int C>
 __global__ __launch_bounds__(PB_THREADS) void pair_bias_kernel(bf16_t* __restrict__ bias_t, const bf16_t* __restrict__ z,
-                                                              const float* __restrict__ wg,   // [H][C] w * gamma
-                                                              const float* __restrict__ c01,  // [H][2]: sum(w*gamma), w . beta
+                                                              const bf16_t* __restrict__ wop,  // [32][C] MFMA weight operand
+                                                              const float* __restrict__ c01,   // [H][2]: sum(w*gamma), w . beta
                                                               int N, int H, int a_inner, long a_so, long a_si,
                                                               float scale, float eps) {
     typedef bf16_t T;
+    typedef Mma<T> MM;
     constexpr int VPR = C / 8;                       // 16-byte vectors per row
     constexpr int PITCH = C * 2 + 16;                // LDS row pitch (bytes)
     constexpr int NLD = 256 * VPR / PB_THREADS;      // loads per thread per quarter
+    constexpr int KS = C / 16;
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* s_rows = smem;                                         // [256][PITCH]
-    float* s_w = reinterpret_cast<float*>(smem + 256 * PITCH);            // [H][C]
+    float* s_sq = reinterpret_cast<float*>(smem + 256 * PITCH);           // [256] sum of squares per row
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
     const int QT = (N + 31) >> 5;
     const int qt = blockIdx.y, kt = blockIdx.x;
-    for (int i = tid; i < H * C; i += PB_THREADS) s_w[i] = wg[i];
+
+    bf16x8 wf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) wf[ks] = MM::ld(wop + l32 * C + ks * 16 + half * 8);
+    // per-lane constants of its four heads h = 4 * half + b
+    float c_sum[4], c_beta[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const int h = 4 * half + b;
+        c_sum[b] = h < H ? c01[2 * h] : 0.0f;
+        c_beta[b] = h < H ? c01[2 * h + 1] : 0.0f;
+    }
 
     const int c8 = tid % VPR, rl = tid / VPR;        // loader role: vector c8 of rows rl, rl + 256/VPR...
-    for (int quarter = 0; quarter < 4; ++quarter) {
-        // rows of this quarter: tile offsets 256*quarter .. +255; offset o <-> q32 = (o/512)*16 + o%16, k32 = (o/16)%32
-        Vec16<T> buf[NLD];
+    // rows of a quarter: tile offsets 256*quarter .. +255; offset o <-> q32 = (o/512)*16 + o%16, k32 = (o/16)%32
+    Vec16<T> buf[NLD];
+    auto fetch = [&](int quarter) {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int o = quarter * 256 + rl + i * (PB_THREADS / VPR);
@@ -49,70 +67,74 @@ __global__ __launch_bounds__(PB_THREADS) void pair_bias_kernel(bf16_t* __restric
             const unsigned hi = m / (unsigned)a_inner, lo = m - hi * (unsigned)a_inner;
             buf[i] = ld16(z + (long)hi * a_so + (long)lo * a_si + c8 * 8);
         }
+    };
+    fetch(0);
+    for (int quarter = 0; quarter < 4; ++quarter) {
         __syncthreads();                             // previous quarter's rows are consumed
 #pragma unroll
-        for (int i = 0; i < NLD; ++i)
-            *reinterpret_cast<Vec16<T>*>(s_rows + (rl + i * (PB_THREADS / VPR)) * PITCH + c8 * 16) = buf[i];
-        __syncthreads();
-
-        // thread tid finishes row tid: pass 1 mean, pass 2 centred second moment and dot products
-        const unsigned char* row = s_rows + tid * PITCH;
-        float s = 0.0f;
-#pragma unroll
-        for (int v = 0; v < VPR; ++v) {
-            const Vec16<T> x = *reinterpret_cast<const Vec16<T>*>(row + v * 16);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s += (float)x.e[e];
-        }
-        const float mu = s * (1.0f / C);
-        float var = 0.0f, dot[PB_MAXH];
-#pragma unroll
-        for (int h = 0; h < PB_MAXH; ++h) dot[h] = 0.0f;
-#pragma unroll
-        for (int v = 0; v < VPR; ++v) {
-            const Vec16<T> x = *reinterpret_cast<const Vec16<T>*>(row + v * 16);
-            float f[8];
+        for (int i = 0; i < NLD; ++i) {
+            const int r = rl + i * (PB_THREADS / VPR);
+            *reinterpret_cast<Vec16<T>*>(s_rows + r * PITCH + c8 * 16) = buf[i];
+            float q2 = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                f[e] = (float)x.e[e] - mu;
-                var += f[e] * f[e];
+                const float f = (float)buf[i].e[e];
+                q2 += f * f;
             }
+            q2 = group_sum(q2, VPR);
+            if (c8 == 0) s_sq[r] = q2;
+        }
+        __syncthreads();
+        if (quarter < 3) fetch(quarter + 1);         // in flight while this quarter is finished below
+
 #pragma unroll
-            for (int h = 0; h < PB_MAXH; ++h) {
-                if (h < H) {                          // uniform
-                    const f32x4 w0 = *reinterpret_cast<const f32x4*>(s_w + h * C + v * 8);
-                    const f32x4 w1 = *reinterpret_cast<const f32x4*>(s_w + h * C + v * 8 + 4);
+        for (int g = 0; g < 2; ++g) {
+            const int row = (wave * 2 + g) * 32 + l32;
+            const unsigned char* ap = s_rows + row * PITCH + half * 16;
+            f32x16 acc;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) dot[h] += f[e] * w0[e] + f[4 + e] * w1[e];
+            for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) MM::mma(acc, wf[ks], *reinterpret_cast<const bf16x8*>(ap + ks * 32));
+            // registers 0..3: heads 4*half + b; register 4: sum(x) (ones rows 8 / 12 of the weight operand)
+            const float mu = acc[4] * (1.0f / C);
+            const float var = fmaxf(s_sq[row] * (1.0f / C) - mu * mu, 0.0f);
+            const float rs = rsqrtf(var + eps);
+            const int o = quarter * 256 + row;
+            const int q = qt * 32 + (o >> 9) * 16 + (o & 15), k = kt * 32 + ((o >> 4) & 31);
+            if (q < N && k < N) {
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const int h = 4 * half + b;
+                    if (h < H)
+                        bias_t[(((long)h * QT + qt) * QT + kt) * 1024 + o] = (T)(scale * (rs * (acc[b] - mu * c_sum[b]) + c_beta[b]));
                 }
             }
-        }
-        const float rs = rsqrtf(var * (1.0f / C) + eps);
-        const int o = quarter * 256 + tid;
-        const int q = qt * 32 + (o >> 9) * 16 + (o & 15), k = kt * 32 + ((o >> 4) & 31);
-        if (q < N && k < N) {
-#pragma unroll
-            for (int h = 0; h < PB_MAXH; ++h)
-                if (h < H) bias_t[(((long)h * QT + qt) * QT + kt) * 1024 + o] = (T)(scale * (rs * dot[h] + c01[2 * h + 1]));
         }
     }
 }
 
-// wg[h][c] = w[h][c] * gamma[c];  c01[h] = (unused, sum wg), w[h] . beta  - tiny, one block
-__global__ void pair_bias_prep_kernel(float* wg, float* c01, const bf16_t* w, const bf16_t* gamma, const bf16_t* beta, int H,
+// Builds the MFMA weight operand wop[32][C] (rows 0..H-1: w * gamma rounded to bf16, rows 8 and 12: ones,
+// others zero) and c01[h] = { sum_c wop[h][c], w[h] . beta }.  One block per operand row.
+__global__ void pair_bias_prep_kernel(bf16_t* wop, float* c01, const bf16_t* w, const bf16_t* gamma, const bf16_t* beta, int H,
                                       int C) {
     const int h = blockIdx.x;
     float s0 = 0.0f, s1 = 0.0f;
     for (int c = threadIdx.x; c < C; c += blockDim.x) {
-        const float wv = (float)w[h * C + c];
-        const float g = wv * (float)gamma[c];
-        wg[h * C + c] = g;
-        s0 += g;
-        s1 += wv * (float)beta[c];
+        bf16_t v = (bf16_t)0.0f;
+        if (h < H) {
+            const float wv = (float)w[h * C + c];
+            v = (bf16_t)(wv * (float)gamma[c]);
+            s0 += (float)v;                           // the sum of what the MFMA really multiplies by
+            s1 += wv * (float)beta[c];
+        } else if (h == 8 || h == 12) {
+            v = (bf16_t)1.0f;
+        }
+        wop[h * C + c] = v;
     }
     s0 = group_sum(s0, 64);
     s1 = group_sum(s1, 64);
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0 && h < H) {
         c01[2 * h] = s0;
         c01[2 * h + 1] = s1;
     }
@@ -131,22 +153,22 @@ extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, con
     FFK_REQUIRE(ffk_aligned16(z) && ffk_aligned16(scratch) && a_so % 8 == 0 && a_si % 8 == 0, FFK_ERR_ALIGN,
                 "ffk_pair_bias: rows of z must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    float* wg = scratch;                 // [H][C]
-    float* c01 = scratch + H * C;        // [H][2]
-    pair_bias_prep_kernel<<<(unsigned)H, 64, 0, st>>>(wg, c01, (const bf16_t*)w, (const bf16_t*)gamma, (const bf16_t*)beta,
-                                                      (int)H, (int)C);
+    bf16_t* wop = reinterpret_cast<bf16_t*>(scratch);     // [32][C] bf16 = 16 * C floats
+    float* c01 = scratch + 16 * C;                       // [H][2]
+    pair_bias_prep_kernel<<<32, 64, 0, st>>>(wop, c01, (const bf16_t*)w, (const bf16_t*)gamma, (const bf16_t*)beta,
+                                             (int)H, (int)C);
     int rc = ffk_check_launch("ffk_pair_bias");
     if (rc != FFK_OK) return rc;
-    const size_t smem = 256 * (128 * 2 + 16) + (size_t)H * C * sizeof(float);
+    const size_t smem = 256 * (128 * 2 + 16) + 256 * sizeof(float);
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)pair_bias_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)(256 * (128 * 2 + 16) + PB_MAXH * 128 * sizeof(float)));
+                                           (int)smem);
         if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_pair_bias: cannot reserve LDS: %s", hipGetErrorString(e));
         configured = true;
     }
     const unsigned T = (unsigned)((N + 31) / 32);
-    pair_bias_kernel<128><<<dim3(T, T), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wg, c01, (int)N, (int)H,
+    pair_bias_kernel<128><<<dim3(T, T), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wop, c01, (int)N, (int)H,
                                                                 (int)a_inner, a_so, a_si, scale, eps);
     return ffk_check_launch("ffk_pair_bias");
 }

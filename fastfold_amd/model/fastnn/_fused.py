@@ -167,7 +167,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
                           w_row_off=t0 * 128)
     if bias_tile is not None:      # the skinny bias projection has its own pass over x
-        scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=dev)
+        scratch = torch.empty(16 * C + 16, dtype=torch.float32, device=dev)
         _lib.pair_bias(bias_t, x, ln[0], ln[1], w_pk[4 * tpg * 128:], scratch, N=N, C=C, H=H, a_inner=a_inner,
                        a_so=a_so, a_si=a_si, scale=LOG2E)
     kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
@@ -191,7 +191,7 @@ def pair_bias(z, *, r, C, H, ln, wb_pk):
     NT = (r + 31) // 32
     bias_t = alloc((H, NT, NT, 1024), z.dtype, z.device, zero=(r % 32) != 0)
     if z.dtype == torch.bfloat16 and C == 128 and H <= 8:
-        scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=z.device)
+        scratch = torch.empty(16 * C + 16, dtype=torch.float32, device=z.device)
         _lib.pair_bias(bias_t, z, ln[0], ln[1], wb_pk, scratch, N=r, C=C, H=H, a_inner=r * r, a_so=0, a_si=C,
                        scale=LOG2E)
         return bias_t

@@ -320,7 +320,7 @@ def test_pair_bias_kernel(dev, r, H):
     gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
     bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
     T = layouts.n_tiles(r)
-    scratch = torch.empty(H * C + 2 * H, dtype=torch.float32, device=dev)
+    scratch = torch.empty(16 * C + 16, dtype=torch.float32, device=dev)
     for transposed in (False, True):
         bt = torch.zeros(H, T, T, 2, 32, 16, dtype=dtype, device=dev)
         kw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else dict(a_inner=r * r, a_so=0, a_si=C)
