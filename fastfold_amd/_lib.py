@@ -247,6 +247,14 @@ def pair_bias(bias_t, z, gamma, beta, w, scratch, *, N, C, H, a_inner, a_so, a_s
          scale, eps, dtype_tag(z.dtype), stream_ptr())
 
 
+SIGNATURES["ffk_opm_fused"] = [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _P]
+
+
+def opm_fused(out, resid, a_t, b_t, w2p, bias, norm, *, r, spad, eps):
+    call("ffk_opm_fused", ptr(out), ptr(resid), ptr(a_t), ptr(b_t), ptr(w2p), ptr(bias), ptr(norm), r, spad, eps,
+         dtype_tag(a_t.dtype), stream_ptr())
+
+
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):
     call("ffk_key_bias", ptr(keybias), ptr(tileflags), ptr(mask), B, N, mask_sb, mask_sn,
          dtype_tag(mask.dtype) if mask is not None else FFK_F32, stream_ptr())

@@ -262,7 +262,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
 
 
 # ------------------------------------------------------------------ outer product mean ----
-def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, bo, budget, eps=1e-3):
+def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, bo, budget, eps=1e-3, wo_ed=None):
     """out = z + (Wo vec(sum_s a[s,i,:] (x) b[s,j,:]) + bo) / (sum_s mask[s,i] mask[s,j] + eps),
     a, b the masked 32-channel projections of LN(m).  m is [s, r, C] rows, mask [s, r]."""
     dt, dev = m.dtype, m.device
@@ -277,6 +277,10 @@ def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, 
     mt[:, :s] = mask.t()
     nrm = torch.empty(r, r, dtype=torch.float32, device=dev)
     _lib.bgemm_nt(mt, mt, nrm, M=r, N=r, K=spad, lda=spad, ldb=spad, out_f32=True)
+    if wo_ed is not None and dt == torch.bfloat16 and Cz == 128 and r % 32 == 0 and spad in (64, 128):
+        # fused core: the [r, r, 1024] outer product never leaves the chip
+        _lib.opm_fused(out, z, ab[0], ab[1], wo_ed, bo, nrm, r=r, spad=spad, eps=eps)
+        return out
     ci = max(1, min(r, budget // (r * 1024 * es)))
     O = torch.empty(ci * r, 1024, dtype=dt, device=dev)
     for i0 in range(0, r, ci):

@@ -192,14 +192,16 @@ class OutProductMean(nn.Module, _PackMixin):
         Cz = Z_raw.shape[-1]
         if not F_.fits_fused(C, dt):
             raise RuntimeError("OutProductMean: unsupported MSA width %d" % C)
-        wab, bab, wo, bo = self._packed(("opm", dt, dev), [self.linear_a.weight, self.linear_a.bias,
+        wab, bab, wo, bo, wo_ed = self._packed(("opm", dt, dev), [self.linear_a.weight, self.linear_a.bias,
                                                           self.linear_b.weight, self.linear_b.bias,
                                                           self.o_linear.weight, self.o_linear.bias], lambda: (
             F_.pack_rows([self.linear_a.weight, self.linear_b.weight], dt, dev),
             F_.pack_vec([self.linear_a.bias, self.linear_b.bias], dt, dev),
-            self.o_linear.weight.detach().to(dt).contiguous(), self.o_linear.bias.detach().to(dt).contiguous()))
+            self.o_linear.weight.detach().to(dt).contiguous(), self.o_linear.bias.detach().to(dt).contiguous(),
+            # the fused kernel contracts over (e, d) instead of (d, e)
+            self.o_linear.weight.detach().to(dt).view(-1, 32, 32).transpose(1, 2).reshape(-1, 1024).contiguous()))
         F_.outer_product_mean(M.contiguous(), _mask_like(M_mask, M), Z_raw, out, s=s, r=r, C=C, Cz=Cz,
-                              ln=_ln_pair(self.layernormM, dt), wab_pk=wab, bab_pk=bab, wo=wo, bo=bo,
+                              ln=_ln_pair(self.layernormM, dt), wab_pk=wab, bab_pk=bab, wo=wo, bo=bo, wo_ed=wo_ed,
                               budget=_budget())
         return out
 

@@ -246,6 +246,18 @@ int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* be
                   float* scratch, int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so,
                   int64_t a_si, float scale, float eps, int dtype, void* stream);
 
+/* Fused core of the outer-product-mean (bf16, 32 projected channels, 128 pair channels):
+ *     out[i, j, c] = resid[i, j, c] + ( sum_{d,e} (sum_s a[s,i,d] b[s,j,e]) * w[c, d, e] + bias[c] ) / (norm[i, j] + eps)
+ * a_t, b_t : [r*32, spad] the masked projections, transposed (row i*32 + d, K = sequences, zero padded
+ *            to spad = 64 or 128); w2p : [128, 1024] with column e*32 + d (the reference weight has d*32 + e);
+ * norm : fp32 [r, r]; resid / out : [r*r, 128] (may alias); r % 32 == 0.
+ * The [r, r, 1024] outer product is never written to memory.
+ * Replaces: the einsum / o_linear / division chain of OutProductMean.forward
+ * (fastfold/model/fastnn/ops.py:156-171; nn/outer_product_mean.py:93-127). */
+int ffk_opm_fused(void* out, const void* resid, const void* a_t, const void* b_t, const void* w2p,
+                  const void* bias, const float* norm, int64_t r, int64_t spad, float eps, int dtype,
+                  void* stream);
+
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the
  * given dtype, or NULL (all keys valid).  tileflags[b, k/32] classifies each 32-key tile (see

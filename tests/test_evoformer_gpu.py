@@ -113,9 +113,9 @@ def test_submodule_updates_fp32(dev, name, s, r, tail):
     assert np.abs(got - ref).max() <= 1e-4 * scale, (name, np.abs(got - ref).max(), scale)
 
 
+@pytest.mark.parametrize("s,r,tail", [(16, 48, 0.1), (128, 64, 0.1), (64, 96, 0.0)])
 @pytest.mark.parametrize("name", SUBMODULES)
-def test_submodule_updates_bf16(dev, name):
-    s, r, tail = 16, 48, 0.1
+def test_submodule_updates_bf16(dev, name, s, r, tail):
     model = _oracle(22, 1)
     fast = _fast(model, dev, torch.bfloat16)
     m, z, mm, pm = synth_inputs(8, s, r, mask_tail_frac=tail)
