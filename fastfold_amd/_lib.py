@@ -255,6 +255,14 @@ def opm_fused(out, resid, a_t, b_t, w2p, bias, norm, *, r, spad, eps):
          dtype_tag(a_t.dtype), stream_ptr())
 
 
+SIGNATURES["ffk_transition_fused"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _P]
+
+
+def transition_fused(out, x, gamma, beta, w1, b1, w2, b2, *, M, C, hidden, eps=1e-5):
+    call("ffk_transition_fused", ptr(out), ptr(x), ptr(gamma), ptr(beta), ptr(w1), ptr(b1), ptr(w2), ptr(b2), M, C, hidden,
+         eps, dtype_tag(x.dtype), stream_ptr())
+
+
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):
     call("ffk_key_bias", ptr(keybias), ptr(tileflags), ptr(mask), B, N, mask_sb, mask_sn,
          dtype_tag(mask.dtype) if mask is not None else FFK_F32, stream_ptr())

@@ -96,6 +96,10 @@ def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
     M, C = x.shape
     dt, dev = x.dtype, x.device
     es = es_of(dt)
+    if dt == torch.bfloat16 and C == 128 and hidden == 512 and ln is not None:
+        # both layers in one kernel, hidden activation kept on chip
+        _lib.transition_fused(out, x, ln[0], ln[1], w1_pk, b1_pk, w2, b2, M=M, C=C, hidden=hidden)
+        return out
     rows = max(128, min(M, (budget // (hidden * es)) // 128 * 128))
     hid = torch.empty(min(rows, M), hidden, dtype=dt, device=dev)
     nt = hidden // 128

@@ -258,6 +258,15 @@ int ffk_opm_fused(void* out, const void* resid, const void* a_t, const void* b_t
                   const void* bias, const float* norm, int64_t r, int64_t spad, float eps, int dtype,
                   void* stream);
 
+/* Fused pair transition (bf16, C = 128, hidden = 512):
+ *     out = x + W2 . relu( W1 . LayerNorm(x; gamma, beta, eps) + b1 ) + b2
+ * x, out : [M, C] row-major (may alias); w1 : [hidden, C]; w2 : [C, hidden]; b1 : [hidden]; b2 : [C].
+ * The hidden activation never leaves the chip.
+ * Replaces: Transition.forward / ChunkTransition.forward (fastfold/model/fastnn/ops.py:79-82,104-123). */
+int ffk_transition_fused(void* out, const void* x, const void* gamma, const void* beta, const void* w1,
+                         const void* b1, const void* w2, const void* b2, int64_t M, int64_t C,
+                         int64_t hidden, float eps, int dtype, void* stream);
+
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the
  * given dtype, or NULL (all keys valid).  tileflags[b, k/32] classifies each 32-key tile (see
