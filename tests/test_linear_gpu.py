@@ -332,3 +332,60 @@ def test_pair_bias_kernel(dev, r, H):
         # padding of ragged tiles is left untouched (zero)
         full = _np(layouts.untile_bias(bt, T * 32, T * 32))
         assert np.abs(full[:, r:, :]).max(initial=0.0) == 0.0 and np.abs(full[:, :, r:]).max(initial=0.0) == 0.0
+
+
+@pytest.mark.parametrize("r,s", [(64, 128), (96, 64)])
+def test_opm_fused_kernel(dev, r, s):
+    """ffk_opm_fused against float64 numpy: out = resid + (sum_{d,e} (a_i^T b_j)[d,e] W[c,d,e] + bias) / (norm + eps)."""
+    from fastfold_amd import _lib
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(r + s)
+    a_t = (torch.randn(r * 32, s, generator=g) * 0.5).to(dev, dtype)       # row i*32 + d, K = sequences
+    b_t = (torch.randn(r * 32, s, generator=g) * 0.5).to(dev, dtype)
+    w = (torch.randn(128, 32, 32, generator=g) / 32).to(dev, dtype)         # [c, d, e] as in the reference weight
+    bias = torch.randn(128, generator=g).to(dev, dtype)
+    norm = (torch.rand(r, r, generator=g) * s + 1).to(dev)
+    resid = torch.randn(r * r, 128, generator=g).to(dev, dtype)
+    out = torch.empty_like(resid)
+    w_ed = w.transpose(1, 2).reshape(128, 1024).contiguous()
+    _lib.opm_fused(out, resid, a_t, b_t, w_ed, bias, norm, r=r, spad=s, eps=1e-3)
+    A = _np(a_t).reshape(r, 32, s)
+    B = _np(b_t).reshape(r, 32, s)
+    O = np.einsum("ids,jes->ijde", A, B)
+    O = _np(torch.from_numpy(O).to(torch.bfloat16))                         # the kernel rounds the outer product to bf16
+    upd = (np.einsum("ijde,cde->ijc", O, _np(w)) + _np(bias)) / (_np(norm)[..., None] + 1e-3)
+    got = _np(out).reshape(r, r, 128) - _np(resid).reshape(r, r, 128)
+    assert _rel(got, upd) < TOL[dtype]
+    # in place
+    res2 = resid.clone()
+    _lib.opm_fused(res2, res2, a_t, b_t, w_ed, bias, norm, r=r, spad=s, eps=1e-3)
+    assert torch.equal(res2, out)
+    with pytest.raises(RuntimeError):
+        _lib.opm_fused(out, resid, a_t, b_t, w_ed, bias, norm, r=r + 8, spad=s, eps=1e-3)
+
+
+@pytest.mark.parametrize("M", [256, 1000, 70000])
+def test_transition_fused_kernel(dev, M):
+    """ffk_transition_fused against float64 numpy, including a ragged last workgroup and in-place use."""
+    from fastfold_amd import _lib
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(M)
+    x = (torch.randn(M, 128, generator=g) * 1.5 + 0.2).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(128, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(128, generator=g)).to(dev, dtype)
+    w1 = (torch.randn(512, 128, generator=g) / 128 ** 0.5).to(dev, dtype)
+    b1 = torch.randn(512, generator=g).to(dev, dtype)
+    w2 = (torch.randn(128, 512, generator=g) / 512 ** 0.5).to(dev, dtype)
+    b2 = torch.randn(128, generator=g).to(dev, dtype)
+    out = torch.full_like(x, 7.0)
+    _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=128, hidden=512)
+    xn = _np(torch.from_numpy(ops_np.layer_norm(_np(x), _np(gam), _np(bet))).to(torch.bfloat16))
+    h = np.maximum(ops_np.linear(xn, _np(w1), _np(b1)), 0)
+    h = _np(torch.from_numpy(h).to(torch.bfloat16))                         # hidden is rounded to bf16 on chip
+    upd = ops_np.linear(h, _np(w2), _np(b2))
+    assert _rel(_np(out) - _np(x), upd) < TOL[dtype]
+    x2 = x.clone()
+    _lib.transition_fused(x2, x2, gam, bet, w1, b1, w2, b2, M=M, C=128, hidden=512)
+    assert torch.equal(x2, out)
+    with pytest.raises(RuntimeError):
+        _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=64, hidden=256)
