@@ -101,9 +101,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     constexpr int TILE_VECS = 1024 / VEC;         // 16-byte vectors per tile
     constexpr int NVL = (NTILES * TILE_VECS + ATT_THREADS - 1) / ATT_THREADS;   // vectors per thread per step
     extern __shared__ __align__(16) unsigned char att_smem[];
-    T* lds = reinterpret_cast<T*>(att_smem);      // [2][NTILES][1024]
+    T* lds = reinterpret_cast<T*>(att_smem);      // [2][NTILES][1024] operand slots, then [ATT_THREADS][16] gate values
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: everything derived from it stays scalar
     const int l32 = lane & 31, half = lane >> 5;
     const int bsel = wave >> 2, qsel = wave & 3;
     const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
@@ -128,13 +129,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     const float* mp = keybias + (long)b2 * KT * 32 + 4 * half;
     const int* fl = tileflags + (long)b2 * KT;
 
-    // cooperative operand fetch: vector slot v = tid + i * ATT_THREADS -> (tile, vector in tile)
-    const T* src[NVL];
-    int dst[NVL];
+    // cooperative operand fetch: vector slot v = tid + i * ATT_THREADS -> (tile, vector in tile).  The
+    // 16-byte vectors go from global memory straight into LDS (no staging registers): the 64 lanes of a
+    // wave cover 64 consecutive vectors of one tile, which the hardware places at  base + 16 * lane.
+    static_assert(NVL * ATT_THREADS == NTILES * TILE_VECS, "every thread fetches the same number of vectors");
+    const T* src[NVL];                            // wave-uniform: start of the wave's 64 vectors in key tile 0
 #pragma unroll
     for (int i = 0; i < NVL; ++i) {
-        int v = tid + i * ATT_THREADS;
-        v = v < NTILES * TILE_VECS ? v : NTILES * TILE_VECS - 1;
+        const int v = wave * 64 + i * ATT_THREADS;
         const int tile = v / TILE_VECS, wv = v % TILE_VECS;
         const T* base;
         if (tile < 4) {
@@ -147,15 +149,16 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
             base = bias_t + ((((long)h * QT + qq) * KT) << 10);
         }
         src[i] = base + wv * VEC;
-        dst[i] = tile * 1024 + wv * VEC;
     }
 
     // gate values of this lane's 16 outputs, fetched now so that their latency is hidden by the loop
     const int q = qt * 32 + l32;
     const int qc = q < Nq ? q : Nq - 1;
     const long rowo = ((long)b2 * Nq + qc) * (H * 32) + h * 32 + 4 * half;
-    T gv[4][4];
+    // They wait in LDS (each lane's own 16 values), not in registers.
+    T* gate_lds = lds + 2 * NTILES * 1024 + tid * 16;
     if (gate) {
+        T gv[4][4];
         if (flags & FFK_ATT_GATE_TILED) {
             // accumulator-order tile: this lane's 16 values are contiguous
             const T* gp = gate + ((bh * QT + qt) << 10) + lane * 16;
@@ -176,6 +179,9 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
                 }
             }
         }
+#pragma unroll
+        for (int i = 0; i < 16 / VEC; ++i)
+            *reinterpret_cast<u32x4*>(gate_lds + i * VEC) = *reinterpret_cast<const u32x4*>(&gv[0][0] + i * VEC);
     }
 
     // trailing key tiles that are completely masked in both batch rows contribute exactly zero
@@ -195,10 +201,11 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     // Online softmax with a lazily updated reference.  Instead of subtracting the running row maximum
     // from every score on the vector pipe, the negated reference  -m_ref[q]  is the C operand of the
     // first MFMA of each tile, so the accumulator already holds  s - m_ref  and exp2 is applied to it
-    // directly.  m_ref is only moved (and O / l rescaled) when a tile contains a score more than
-    // REF_SLACK above it, which bounds  p = exp2(s - m_ref) <= 2^REF_SLACK;  the first tile always
-    // sets it.
+    // directly.  m_ref is only moved (and O / l rescaled) when the probabilities of a tile show that
+    // a score lies more than REF_SLACK above it, which bounds  p = exp2(s - m_ref) <= 2^REF_SLACK
+    // in everything that is accumulated;  the first tile always sets it.
     constexpr float REF_SLACK = 20.0f;
+    constexpr float REF_LIMIT = 1048576.0f;       // 2^REF_SLACK
     constexpr float REF_FLOOR = -1.0e4f;          // keeps m_ref small when the first tile is fully masked
     f32x16 o_acc, negm;
 #pragma unroll
@@ -206,56 +213,96 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     float l_run = 0.0f;                           // partial row sum of this lane's 16 keys per tile
     bool first = true;
 
-    Vec16<T> pre[NVL];
-    auto fetch = [&](int kt) {
+    // The loads are issued from an asm statement on purpose: the compiler orders every later LDS read
+    // after all outstanding loads of this kind it knows of (a full s_waitcnt vmcnt(0) right behind
+    // the issue), while here the slot being filled is never the slot being read.  The explicit wait
+    // at the top of the loop is what orders them.
+    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)att_smem;
+    const unsigned lane_off = lane * 16;          // byte offset of this lane's vector; the base address is scalar
+    auto fetch = [&](int kt, int slot) {
 #pragma unroll
-        for (int i = 0; i < NVL; ++i) pre[i] = ld16(src[i] + ((long)kt << 10));
-    };
-    auto commit = [&](int slot) {
-#pragma unroll
-        for (int i = 0; i < NVL; ++i)
-            if (tid + i * ATT_THREADS < NTILES * TILE_VECS)
-                *reinterpret_cast<Vec16<T>*>(lds + slot * NTILES * 1024 + dst[i]) = pre[i];
+        for (int i = 0; i < NVL; ++i) {
+            const T* gp = src[i] + ((long)kt << 10);
+            const unsigned dst = lds_base + (slot * NTILES * TILE_VECS + wave * 64 + i * ATT_THREADS) * 16;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(gp), "s"(dst)
+                         : "memory", "m0");
+#pragma clang diagnostic pop
+        }
     };
 
-    fetch(0);
-    commit(0);
+    // Every load the compiler knows of (q fragments, gate) is made to complete here: a wait it would
+    // otherwise place at the first use inside the loop would also wait for the operand loads issued
+    // just before that use.
+#pragma unroll
+    for (int i = 0; i < Ops16<T>::NV; ++i) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&qf.v[i])));
+    fetch(0, 0);
     int flag_nxt = fl[0];
     for (int kt = 0; kt < kt_end; ++kt) {
-        // the tile's mask flag was fetched one step ahead, so that its latency is never exposed
+        // wait for this thread's share of tile kt before the barrier that publishes it
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         const int flag = __builtin_amdgcn_readfirstlane(flag_nxt);
         lds_barrier();                            // tile kt is in LDS; nobody still reads the other slot
         const int nxt = kt + 1 < kt_end ? kt + 1 : kt;
-        fetch(nxt);                               // in flight during the MFMAs below
+        fetch(nxt, (kt + 1) & 1);                 // in flight during the MFMAs below
         flag_nxt = fl[nxt];
         const T* buf = lds + (kt & 1) * NTILES * 1024;
-        Ops16<T> kc, vc, bc;
-        kc.load(buf + bsel * 1024 + lane * 16);
+        Ops16<T> vc;
         vc.load(buf + (2 + bsel) * 1024 + lane * 16);
-        if (HAS_BIAS) bc.load(buf + (4 + qsel) * 1024 + lane * 16);
 
         // S^T - m_ref = K . Q^T + Bias^T . I + (-m_ref)   (rows: keys, columns: queries)
-        f32x16 s = negm;
+        f32x16 s;
+        auto score_tile = [&]() {
+            Ops16<T> kc, bc;
+            kc.load(buf + bsel * 1024 + lane * 16);
+            if (HAS_BIAS) bc.load(buf + (4 + qsel) * 1024 + lane * 16);
+            s = negm;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
-        if (HAS_BIAS) {
+            for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
+            if (HAS_BIAS) {
 #pragma unroll
-            for (int i = 0; i < NF; ++i) MM::mma(s, bc.frag(i), ident[i]);
+                for (int i = 0; i < NF; ++i) MM::mma(s, bc.frag(i), ident[i]);
+            }
+            if (flag != 0) {         // some key of this tile is masked or padding: add the key bias
+                f32x4 mk[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) mk[g] = *reinterpret_cast<const f32x4*>(mp + kt * 32 + 8 * g);
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) s[4 * g + e] += mk[g][e];
+            }
+        };
+        // P^T = exp2(S^T - m_ref) rounded to the operand type, and the sum of this lane's 16 rounded values
+        Frag pf[NF];
+        float tsum;
+        auto prob_tile = [&]() {
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) p[v] = fast_exp2(s[v]);
+            tsum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NF; ++i) {
+                pf[i] = PFrag<T>::make(p + i * MM::KLANE);
+                tsum = PFrag<T>::add_sum(pf[i], tsum);
+            }
+        };
+        // No maximum is taken on the common path: probabilities are non-negative, so a partial row sum
+        // within 2^REF_SLACK proves that no score of the tile is more than REF_SLACK above the reference.
+        // Only when some lane's sum exceeds that (or on the first tile, which sets the reference) is
+        // the tile recomputed from its LDS slot, the reference moved to the row maximum and O / l rescaled.
+        score_tile();
+        bool move_ref = first;
+        if (!first) {
+            prob_tile();
+            move_ref = __builtin_amdgcn_ballot_w64(!(tsum <= REF_LIMIT)) != 0;
+            if (move_ref) score_tile();
         }
-        if (flag != 0) {             // some key of this tile is masked or padding: add the key bias
-            f32x4 mk[4];
+        if (move_ref) {
+            float mt = fmaxf(s[0], s[1]);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) mk[g] = *reinterpret_cast<const f32x4*>(mp + kt * 32 + 8 * g);
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) s[4 * g + e] += mk[g][e];
-        }
-        float mt = fmaxf(s[0], s[1]);
-#pragma unroll
-        for (int v = 2; v < 16; ++v) mt = fmaxf(mt, s[v]);
-        if (first || __builtin_amdgcn_ballot_w64(mt > REF_SLACK) != 0) {
-            // move the reference of every row of this wave to its running maximum
+            for (int v = 2; v < 16; ++v) mt = fmaxf(mt, s[v]);
             const float mfull = fmaxf(mt, __shfl_xor(mt, 32, 64));
             const float delta = first ? fmaxf(mfull, REF_FLOOR) : fmaxf(mfull, 0.0f);
             const float alpha = first ? 1.0f : fast_exp2(-delta);   // nothing accumulated before the first tile
@@ -267,25 +314,25 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
             }
             l_run *= alpha;
             first = false;
+            prob_tile();
         }
-        float p[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) p[v] = fast_exp2(s[v]);
+        l_run += tsum;
         // O^T += V^T . P^T   (rows: head dim, columns: queries)
 #pragma unroll
-        for (int i = 0; i < NF; ++i) {
-            const Frag pf = PFrag<T>::make(p + i * MM::KLANE);
-            l_run = PFrag<T>::add_sum(pf, l_run);
-            MM::mma(o_acc, vc.frag(i), pf);
-        }
+        for (int i = 0; i < NF; ++i) MM::mma(o_acc, vc.frag(i), pf[i]);
 
-        commit((kt + 1) & 1);                     // the slot last read in step kt - 1
     }
 
     // rows whose keys are all masked have l == 0 and produce zeros
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     if (live && q < Nq) {
+        T gv[4][4];
+        if (gate) {
+#pragma unroll
+            for (int i = 0; i < 16 / VEC; ++i)
+                *reinterpret_cast<u32x4*>(&gv[0][0] + i * VEC) = *reinterpret_cast<const u32x4*>(gate_lds + i * VEC);
+        }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             T r4[4];
@@ -327,7 +374,7 @@ __global__ void key_bias_kernel(float* kb, int* flags, const T* mask, long N, lo
 template <typename T, bool HAS_BIAS>
 int launch_attention_b(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
                        const int* flags, const void* gate, long B2, long H, long Nq, long Nk, int aflags, hipStream_t st) {
-    const size_t smem = 2 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 * sizeof(T);
+    const size_t smem = (2 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 + ATT_THREADS * 16) * sizeof(T);   // operand slots + gate
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)attention_kernel<T, HAS_BIAS>,

@@ -95,6 +95,39 @@ def test_attention_tiling_invariance_and_masked_keys(dev, dtype, tol):
     assert _rel(_np(out), outs[0]) < tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("slope", [0.05, 0.6, 5.0])
+def test_attention_moving_reference(dev, dtype, tol, slope):
+    """Scores that climb (or fall) steadily along the keys: the kernel's running reference has to move
+    several times, by a little (slope 0.05), by more than its slack per tile (0.6) and by more than the
+    fp32 exponent range per tile (5.0: exp2 overflows before the move).  Half of the queries see the
+    keys in descending order, so only part of a wave asks for the move."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    B2, H, N = 2, 4, 200
+    g = torch.Generator().manual_seed(int(slope * 100))
+    u = torch.nn.functional.normalize(torch.randn(H, 32, generator=g), dim=-1)          # one direction per head
+    ramp = torch.arange(N, dtype=torch.float32) * slope                                   # score of key j ~ +-ramp[j]
+    sign = torch.where(torch.arange(N) % 2 == 0, 1.0, -1.0)
+    q = (sign[None, None, :, None] * u[None, :, None, :] + 0.05 * torch.randn(B2, H, N, 32, generator=g)).to(dev, dtype)
+    k = (ramp[None, None, :, None] * u[None, :, None, :] + 0.05 * torch.randn(B2, H, N, 32, generator=g)).to(dev, dtype)
+    v = torch.randn(B2, H, N, 32, generator=g).to(dev, dtype)
+    mask = torch.ones(B2, N, device=dev, dtype=dtype)
+    mask[1, 150:] = 0
+    NT = layouts.n_tiles(N)
+    kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
+    fl = torch.empty(B2, NT, dtype=torch.int32, device=dev)
+    _lib.key_bias(kb, fl, mask, B=B2, N=N, mask_sb=N, mask_sn=1)
+    out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
+    # q is handed over unscaled: logits are q.k in log2 units, i.e. ln2 * q.k for the oracle
+    _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k), layouts.tile_v(v), None, kb, fl, None,
+                       B2=B2, H=H, Nq=N, Nk=N)
+    ref = ops_np.attention_core(_np(q)[None] * math.log(2.0) * math.sqrt(32), _np(k)[None], _np(v)[None], _np(mask)[None], None)[0]
+    got = _np(out).reshape(B2, N, H * 32)
+    assert np.isfinite(got).all()
+    assert _rel(got, ref) < tol
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("r", [52, 128, 200])
 def test_bgemm_trimul_contraction(dev, dtype, tol, r):
