@@ -101,7 +101,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     constexpr int TILE_VECS = 1024 / VEC;         // 16-byte vectors per tile
     constexpr int NVL = (NTILES * TILE_VECS + ATT_THREADS - 1) / ATT_THREADS;   // vectors per thread per step
     extern __shared__ __align__(16) unsigned char att_smem[];
-    T* lds = reinterpret_cast<T*>(att_smem);      // [2][NTILES][1024] operand slots, then [ATT_THREADS][16] gate values
+    constexpr int NSLOT = 3;                      // operand ring: the tile in use and two in flight behind it
+    T* lds = reinterpret_cast<T*>(att_smem);      // [NSLOT][NTILES][1024] operand slots, then [ATT_THREADS][16] gate values
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: everything derived from it stays scalar
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     const int qc = q < Nq ? q : Nq - 1;
     const long rowo = ((long)b2 * Nq + qc) * (H * 32) + h * 32 + 4 * half;
     // They wait in LDS (each lane's own 16 values), not in registers.
-    T* gate_lds = lds + 2 * NTILES * 1024 + tid * 16;
+    T* gate_lds = lds + NSLOT * NTILES * 1024 + tid * 16;
     if (gate) {
         T gv[4][4];
         if (flags & FFK_ATT_GATE_TILED) {
@@ -238,16 +239,23 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
 #pragma unroll
     for (int i = 0; i < Ops16<T>::NV; ++i) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&qf.v[i])));
     fetch(0, 0);
+    fetch(kt_end > 1 ? 1 : 0, 1);
     int flag_nxt = fl[0];
+    int slot = 0;                                 // ring slot of tile kt
     for (int kt = 0; kt < kt_end; ++kt) {
-        // wait for this thread's share of tile kt before the barrier that publishes it
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // Tile kt was requested two steps ago: wait until only the newest request (tile kt + 1) of this
+        // thread is still in flight, then the barrier publishes tile kt and retires the slot of tile kt - 1.
+        if (NVL == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+        else if (NVL == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         const int flag = __builtin_amdgcn_readfirstlane(flag_nxt);
-        lds_barrier();                            // tile kt is in LDS; nobody still reads the other slot
+        lds_barrier();
         const int nxt = kt + 1 < kt_end ? kt + 1 : kt;
-        fetch(nxt, (kt + 1) & 1);                 // in flight during the MFMAs below
+        const int nxt2 = kt + 2 < kt_end ? kt + 2 : kt_end - 1;
+        fetch(nxt2, slot == 0 ? 2 : slot - 1);    // (slot + 2) % 3: the slot tile kt - 1 was read from
         flag_nxt = fl[nxt];
-        const T* buf = lds + (kt & 1) * NTILES * 1024;
+        const T* buf = lds + slot * NTILES * 1024;
+        slot = slot == 2 ? 0 : slot + 1;
         Ops16<T> vc;
         vc.load(buf + (2 + bsel) * 1024 + lane * 16);
 
@@ -323,6 +331,9 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
 
     }
 
+    // the requests past the last tile must have landed before this workgroup's LDS can be handed on
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
     // rows whose keys are all masked have l == 0 and produce zeros
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
@@ -374,7 +385,7 @@ __global__ void key_bias_kernel(float* kb, int* flags, const T* mask, long N, lo
 template <typename T, bool HAS_BIAS>
 int launch_attention_b(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
                        const int* flags, const void* gate, long B2, long H, long Nq, long Nk, int aflags, hipStream_t st) {
-    const size_t smem = (2 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 + ATT_THREADS * 16) * sizeof(T);   // operand slots + gate
+    const size_t smem = (3 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 + ATT_THREADS * 16) * sizeof(T);   // operand ring + gate
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)attention_kernel<T, HAS_BIAS>,
