@@ -66,7 +66,13 @@ struct WsSlot {
     int kind, act;
     float scale;
     bool masked;
+    bool has_bias;
 };
+
+// sigmoid(acc + b) with the bias table entry pre-multiplied:  bs = -log2(e) * b
+__device__ __forceinline__ float ws_sigmoid_pre(float acc, float bs) {
+    return fast_rcp(1.0f + fast_exp2(__builtin_fmaf(acc, -1.4426950408889634f, bs)));
+}
 
 // tiles stored with channels contiguous (lane = row) vs rows contiguous (lane = channel)
 __host__ __device__ __forceinline__ bool ws_by_rows(const ffk_tile& t) {
@@ -78,16 +84,6 @@ __device__ __forceinline__ void unpack4(const T* p, float (&f)[4]) {
     const T* h = reinterpret_cast<const T*>(&raw);
 #pragma unroll
     for (int e = 0; e < 4; ++e) f[e] = (float)h[e];
-}
-
-__device__ __forceinline__ void ws_activate(float (&x)[16], int act) {
-    if (act == FFK_ACT_RELU) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = fmaxf(x[v], 0.0f);
-    } else if (act == FFK_ACT_SIGMOID) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = sigmoid_f(x[v]);
-    }
 }
 
 // Index permutation tau(8a + 4h + b) = 16h + 4a + b.  An MFMA accumulator register v = 4a + b of
@@ -120,15 +116,33 @@ __device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc
             bv[a] = *reinterpret_cast<const f32x4*>(sb + o);
             if (GLU) bg[a] = *reinterpret_cast<const f32x4*>(sb + 32 + o);
         }
+        if (GLU) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-            x[v] = GLU ? (acc[v] + bv[v >> 2][v & 3]) * sigmoid_f(accg[v] + bg[v >> 2][v & 3]) : acc[v] + bv[v >> 2][v & 3];
+            for (int v = 0; v < 16; ++v) x[v] = (acc[v] + bv[v >> 2][v & 3]) * ws_sigmoid_pre(accg[v], bg[v >> 2][v & 3]);
+        } else if (t.act == FFK_ACT_SIGMOID) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = ws_sigmoid_pre(acc[v], bv[v >> 2][v & 3]);
+        } else if (t.has_bias) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = acc[v] + bv[v >> 2][v & 3];
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = acc[v];
+        }
     }
-    if (!GLU) ws_activate(x, t.act);
-    const float scl = t.scale * rmask;
-    T y[16];
+    if (!GLU && t.act == FFK_ACT_RELU) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * scl);
+        for (int v = 0; v < 16; ++v) x[v] = fmaxf(x[v], 0.0f);
+    }
+    T y[16];
+    if (t.masked || t.scale != 1.0f) {
+        const float scl = t.scale * rmask;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * scl);
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)x[v];
+    }
 
     T* out = t.out;
     if (t.kind == FFK_TILE_ACC) {
@@ -187,9 +201,20 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
                                               const float* sm, long m0g, int M, int l32, int half) {
     const float bv = sb[l32], bg = GLU ? sb[32 + l32] : 0.0f;
     float x[16];
+    if (GLU) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) x[v] = GLU ? (acc[v] + bv) * sigmoid_f(accg[v] + bg) : acc[v] + bv;
-    if (!GLU) ws_activate(x, t.act);
+        for (int v = 0; v < 16; ++v) x[v] = (acc[v] + bv) * ws_sigmoid_pre(accg[v], bg);
+    } else if (t.act == FFK_ACT_SIGMOID) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = ws_sigmoid_pre(acc[v], bv);
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = acc[v] + bv;
+        if (t.act == FFK_ACT_RELU) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = fmaxf(x[v], 0.0f);
+        }
+    }
 
     T* out = t.out;
     const bool vt = t.kind == FFK_TILE_V;
@@ -201,7 +226,8 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
         hi = mc / t.inner;
         lo = mc - hi * t.inner;
     }
-    if (sm && !vt) {
+    // the mask multiply is skipped for row groups without a masked row (the common case)
+    if (sm && !vt && __builtin_amdgcn_ballot_w64(sm[l32] != 1.0f) != 0) {
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const f32x4 mk = *reinterpret_cast<const f32x4*>(sm + 16 * half + 4 * a);
@@ -210,8 +236,13 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
         }
     }
     T y[16];
+    if (t.scale != 1.0f) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
+        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)x[v];
+    }
     if (vt) {
         if (ok && t.ncols_left >= 32) {
             T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + ((half * 32 + l32) << 4);
@@ -246,8 +277,12 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 
     // ---- bias table: no global loads in the epilogues ----
     for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) {
-        const T* bp = (const T*)d.tiles[i >> 7].bias;
-        s_bias[i] = bp ? (float)bp[i & 127] : 0.0f;
+        const ffk_tile& tb = d.tiles[i >> 7];
+        const T* bp = (const T*)tb.bias;
+        // gate halves of a GLU unit ([p 32 | g 32 | p 32 | g 32]) and sigmoid tiles: pre-multiplied for ws_sigmoid_pre
+        const bool sig = tb.glu ? ((i >> 5) & 1) != 0 : tb.act == FFK_ACT_SIGMOID;
+        const float b = bp ? (float)bp[i & 127] : 0.0f;
+        s_bias[i] = sig ? -1.4426950408889634f * b : b;
     }
 
     // ---- this wave's weight slots, resident in registers ----
@@ -279,6 +314,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             sp[s].act = ts.act;
             sp[s].scale = ts.scale;
             sp[s].masked = ts.rowmask != nullptr;
+            sp[s].has_bias = ts.bias != nullptr;
             by_rows[s] = ws_by_rows(ts);
         }
 #pragma unroll
