@@ -1,34 +1,38 @@
 // Fused pair transition (see ffk_transition_fused in include/ffk.h):
 //     out = x + W2 . relu( W1 . LayerNorm(x) + b1 ) + b2        (128 -> 512 -> 128 channels, bf16)
-// with the 512-channel hidden activation kept on chip.
+// with the 512-channel hidden activation never leaving the registers.
 //
-// A workgroup (8 wavefronts) owns 256 rows.  Set-up: the rows are fetched once, normalised in registers
-// (16 lanes per row) and parked in LDS; wave w then lifts the MFMA fragments of its own 32 rows into
-// registers, where they stay.  The hidden layer is walked in 8 chunks of 64 channels:
-//   phase A  hidden[rows of wave w, chunk] = relu(W1[chunk] . x^T + b1): 2 MFMA tiles per wave, results
-//            rounded to bf16 and written to LDS as rows of A2[row][hidden in chunk];
-//   phase B  out[row, c] += A2[row, chunk] . W2[c, chunk]: 8 x 4 MFMA tiles, 2 x 2 per wave, accumulators
-//            in registers across all chunks.
-// W1 / W2 chunks arrive by direct global -> LDS loads (XOR-swizzled unpadded rows) one iteration ahead;
-// phase B of chunk q - 1 and phase A of chunk q share one barrier.  The LDS that held the normalised
-// rows is reused for the rings once the fragments are in registers.
+// A workgroup (4 wavefronts) owns 128 rows, a wavefront 32 of them from start to end.  Set-up: the rows
+// are fetched once, normalised in registers (16 lanes per row) and passed through LDS into the MFMA
+// fragments of their wave, where they stay.  The hidden layer is walked in 8 chunks of 64 channels; per
+// chunk and wave
+//   first GEMM   H^T[hidden, rows] = W1[chunk] . x^T  (+ b1, relu): 2 tiles of 32 hidden channels; lane =
+//                row, registers = hidden channels;
+//   second GEMM  out^T[c, rows] += W2[c, chunk] . H^T: the rounded accumulators of the first GEMM are the
+//                N operand as they stand.  A lane holds hidden channels 8a + 4h + b of a tile (h = its
+//                half-wave) in registers 4a + b, and an MFMA K step wants 8 consecutive K per half-wave,
+//                so the first GEMM's M-operand row i is loaded from weight row sigma(i) such that
+//                registers 8j .. 8j + 7 of half-wave h are hidden channels 16j + 8h .. 16j + 8h + 7.
+// Only the weights go through LDS: W1 / W2 chunks arrive by direct global -> LDS loads (XOR-swizzled
+// unpadded rows) one chunk ahead, shared by the four waves; one barrier per chunk.  Two workgroups fit
+// a CU, so one computes while the other waits for its rows or its barrier.
 #include "ffk_common.h"
 
 namespace {
 
 typedef bf16_t T;
-constexpr int TR_THREADS = 512;
-constexpr int TR_BM = 256;                     // rows per workgroup
+constexpr int TR_THREADS = 256;
+constexpr int TR_BM = 128;                     // rows per workgroup
 constexpr int TR_C = 128, TR_H = 512;
 constexpr int TR_HC = 64;                      // hidden channels per chunk
 constexpr int TR_NCHUNK = TR_H / TR_HC;        // 8
-constexpr int TR_PA = TR_HC * 2 + 16;          // A2 row pitch (bytes)
-constexpr int TR_A2 = TR_BM * TR_PA;           // one A2 buffer (36 864 B)
 constexpr int TR_W1SLOT = TR_HC * TR_C * 2;    // 64 rows of 256 bytes (16 KB)
 constexpr int TR_W2SLOT = TR_C * TR_HC * 2;    // 128 rows of 128 bytes (16 KB)
 constexpr int TR_XP = TR_C * 2 + 16;           // pitch of the normalised rows (set-up only)
 
 __device__ __forceinline__ int tr_tau(int i) { return ((i >> 2) & 1) * 16 + (i >> 3) * 4 + (i & 3); }
+// i = 8a + 4h + b  ->  16 (a / 2) + 8h + 4 (a % 2) + b
+__device__ __forceinline__ int tr_sigma(int i) { return (i >> 4) * 16 + ((i >> 2) & 1) * 8 + ((i >> 3) & 1) * 4 + (i & 3); }
 
 __device__ __forceinline__ void tr_load_lds(const T* src, unsigned char* dst_wave) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
@@ -42,11 +46,10 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
                                                                         long M, float eps) {
     typedef Mma<T> MM;
     extern __shared__ __align__(16) unsigned char smem[];
-    unsigned char* s_a2 = smem;                           // [2][256][TR_PA]
-    unsigned char* s_w2 = smem + 2 * TR_A2;               // [3][128][128 B]
-    unsigned char* s_w1 = s_w2 + 3 * TR_W2SLOT;           // [2][64][256 B]
-    float* s_b1 = reinterpret_cast<float*>(s_w1 + 2 * TR_W1SLOT);   // [512]
-    unsigned char* s_x = smem;                            // [256][TR_XP], set-up only (aliases the above)
+    unsigned char* s_w1 = smem;                           // [2][64][256 B]
+    unsigned char* s_w2 = smem + 2 * TR_W1SLOT;           // [2][128][128 B]
+    float* s_b1 = reinterpret_cast<float*>(s_w2 + 2 * TR_W2SLOT);   // [512]
+    unsigned char* s_x = smem;                            // [128][TR_XP], set-up only (aliases the rings)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -55,12 +58,12 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
 
     // ---- set-up: rows -> LayerNorm in registers -> LDS -> this wave's fragments ----
     {
-        const int c8 = tid & 15, r0 = tid >> 4;           // 16 lanes per row, 32 rows per pass, 8 passes
+        const int c8 = tid & 15, r0 = tid >> 4;           // 16 lanes per row, 16 rows per pass, 8 passes
         const Vec16<T> g = ld16(gamma + c8 * 8), b = ld16(beta + c8 * 8);
         Vec16<T> v[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            long m = m0 + r0 + 32 * i;
+            long m = m0 + r0 + 16 * i;
             m = m < M ? m : M - 1;                        // clamped: rows past the end are never stored
             v[i] = ld16(x + m * TR_C + c8 * 8);
         }
@@ -83,7 +86,7 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
             Vec16<T> y;
 #pragma unroll
             for (int e = 0; e < 8; ++e) y.e[e] = (T)(f[e] * rs * (float)g.e[e] + (float)b.e[e]);
-            *reinterpret_cast<Vec16<T>*>(s_x + (r0 + 32 * i) * TR_XP + c8 * 16) = y;
+            *reinterpret_cast<Vec16<T>*>(s_x + (r0 + 16 * i) * TR_XP + c8 * 16) = y;
         }
     }
     lds_barrier();
@@ -95,38 +98,34 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
     for (int i = tid; i < TR_H; i += TR_THREADS) s_b1[i] = (float)b1[i];
 
     // ---- chunk loaders (direct to LDS; lane L of a wave lands at dst + 16 L) ----
-    // W1 chunk: LDS row rho (0..63) holds weight row 32 * (rho / 32) + tau(rho % 32) of the chunk; 16 columns
-    const T* w1src[2];
+    // W1 chunk: LDS row rho (0..63) holds weight row 32 * (rho / 32) + sigma(rho % 32) of the chunk; 16 columns
+    const T* w1src[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 4; ++i) {
         const int v = i * TR_THREADS + tid, rho = v >> 4, c = v & 15;
-        w1src[i] = w1 + (long)((rho & ~31) + tr_tau(rho & 31)) * TR_C + ((c ^ (rho & 15)) * 8);
+        w1src[i] = w1 + (long)((rho & ~31) + tr_sigma(rho & 31)) * TR_C + ((c ^ (rho & 15)) * 8);
     }
     // W2 chunk: LDS row rho (0..127) holds weight row 32 * (rho / 32) + tau(rho % 32); 8 columns
-    const T* w2src[2];
+    const T* w2src[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 4; ++i) {
         const int v = i * TR_THREADS + tid, rho = v >> 3, c = v & 7;
         w2src[i] = w2 + (long)((rho & ~31) + tr_tau(rho & 31)) * TR_H + ((c ^ ((rho >> 1) & 7)) * 8);
     }
     auto fetch = [&](int q) {
         unsigned char* d1 = s_w1 + (q & 1) * TR_W1SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) tr_load_lds(w1src[i] + (long)q * TR_HC * TR_C, d1 + i * (TR_THREADS * 16));
-        unsigned char* d2 = s_w2 + (q % 3) * TR_W2SLOT + wave * 1024;
+        for (int i = 0; i < 4; ++i) tr_load_lds(w1src[i] + (long)q * TR_HC * TR_C, d1 + i * (TR_THREADS * 16));
+        unsigned char* d2 = s_w2 + (q & 1) * TR_W2SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) tr_load_lds(w2src[i] + q * TR_HC, d2 + i * (TR_THREADS * 16));
+        for (int i = 0; i < 4; ++i) tr_load_lds(w2src[i] + q * TR_HC, d2 + i * (TR_THREADS * 16));
     };
 
-    // ---- phase B roles: m-tiles 2 * (wave % 4) + {0, 1}, c-tiles 2 * (wave / 4) + {0, 1} ----
-    const int mt0 = 2 * (wave & 3), ct0 = 2 * (wave >> 2);
-    f32x16 acc2[2][2];   // [m][c]
+    f32x16 acc2[4];                                        // out^T tiles: channels 32 ct + 16 half + v, row l32
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int c = 0; c < 4; ++c)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc2[a][b][v] = 0.0f;
+        for (int v = 0; v < 16; ++v) acc2[c][v] = 0.0f;
 
     int w1off[8];                                          // W1 fragment of hidden tile 0: row l32, column 2 ks + half
 #pragma unroll
@@ -134,83 +133,63 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
     int w2off[4];                                          // W2 fragment of c-tile 0: row l32, column 2 ks + half
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) w2off[ks] = l32 * 128 + (((2 * ks + half) ^ ((l32 >> 1) & 7)) << 4);
-    const int a2w = (wave * 32 + l32) * TR_PA + 32 * half;   // phase A: row of this lane, hidden 16 half (+ 32 ht)
-    const int a2r = l32 * TR_PA + half * 16;                 // phase B: row mt * 32 + l32, k = 16 ks + 8 half
 
     fetch(0);
-    for (int q = 0; q <= TR_NCHUNK; ++q) {
+    for (int q = 0; q < TR_NCHUNK; ++q) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // chunk q has landed (this wave's part)
-        __builtin_amdgcn_s_barrier();                        // ... everyone's; A2 of chunk q - 1 is complete
+        __builtin_amdgcn_s_barrier();                        // ... everyone's; nobody still reads the other slots
         if (q + 1 < TR_NCHUNK) fetch(q + 1);
-        if (q > 0) {
-            // ---- phase B of chunk q - 1 ----
-            const unsigned char* a2 = s_a2 + ((q - 1) & 1) * TR_A2;
-            const unsigned char* wb = s_w2 + ((q - 1) % 3) * TR_W2SLOT;
+        const unsigned char* wa = s_w1 + (q & 1) * TR_W1SLOT;
+        const unsigned char* wb = s_w2 + (q & 1) * TR_W2SLOT;
+        bf16x8 hf[2][2];                                   // [hidden tile][K step]: the chunk's N operand
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                bf16x8 fa[2], fw[2];
+        for (int ht = 0; ht < 2; ++ht) {
+            f32x16 h;
+            // registers 0..7: hidden 8 half + 0..7 of the tile, registers 8..15: 16 + 8 half + 0..7
+            const float* bp = s_b1 + q * TR_HC + ht * 32 + 8 * half;
 #pragma unroll
-                for (int m = 0; m < 2; ++m) fa[m] = *reinterpret_cast<const bf16x8*>(a2 + (mt0 + m) * 32 * TR_PA + a2r + ks * 32);
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 b4 = *reinterpret_cast<const f32x4*>(bp + (a >> 1) * 16 + (a & 1) * 4);
 #pragma unroll
-                for (int c = 0; c < 2; ++c) fw[c] = *reinterpret_cast<const bf16x8*>(wb + (ct0 + c) * 32 * 128 + w2off[ks]);
-#pragma unroll
-                for (int m = 0; m < 2; ++m)
-#pragma unroll
-                    for (int c = 0; c < 2; ++c) MM::mma(acc2[m][c], fw[c], fa[m]);
+                for (int b = 0; b < 4; ++b) h[4 * a + b] = b4[b];
             }
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+                MM::mma(h, *reinterpret_cast<const bf16x8*>(wa + ht * 32 * 256 + w1off[ks]), xf[ks]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) hf[ht][j][t] = (T)fmaxf(h[8 * j + t], 0.0f);
         }
-        if (q < TR_NCHUNK) {
-            // ---- phase A of chunk q: two hidden tiles for this wave's 32 rows ----
-            const unsigned char* wa = s_w1 + (q & 1) * TR_W1SLOT;
-            unsigned char* a2 = s_a2 + (q & 1) * TR_A2;
 #pragma unroll
-            for (int ht = 0; ht < 2; ++ht) {
-                f32x16 h;
-                const float* bp = s_b1 + q * TR_HC + ht * 32 + 16 * half;
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const f32x4 b4 = *reinterpret_cast<const f32x4*>(bp + 4 * a);
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) h[4 * a + b] = b4[b];
-                }
-#pragma unroll
-                for (int ks = 0; ks < 8; ++ks)
-                    MM::mma(h, *reinterpret_cast<const bf16x8*>(wa + ht * 32 * 256 + w1off[ks]), xf[ks]);
-                T y[16];
-#pragma unroll
-                for (int v = 0; v < 16; ++v) y[v] = (T)fmaxf(h[v], 0.0f);
-                unsigned char* p = a2 + a2w + ht * 64;
-                *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
-                *reinterpret_cast<u32x4*>(p + 16) = *reinterpret_cast<const u32x4*>(&y[8]);
-            }
-        }
+            for (int c = 0; c < 4; ++c)
+                MM::mma(acc2[c], *reinterpret_cast<const bf16x8*>(wb + c * 32 * 128 + w2off[ks]), hf[ks >> 1][ks & 1]);
     }
 
     // ---- epilogue: lane = row, registers = 16 consecutive channels ----
+    const long row = m0 + wave * 32 + l32;
+    const bool ok = row < M;
+    const long rc = ok ? row : M - 1;
 #pragma unroll
-    for (int m = 0; m < 2; ++m) {
-        const long row = m0 + (mt0 + m) * 32 + l32;
-        const bool ok = row < M;
-        const long rc = ok ? row : M - 1;
+    for (int c = 0; c < 4; ++c) {
+        const int ch = c * 32 + 16 * half;
+        const long o = rc * TR_C + ch;
+        u32x4 bv[2], rv[2];
+        bv[0] = *reinterpret_cast<const u32x4*>(b2 + ch);
+        bv[1] = *reinterpret_cast<const u32x4*>(b2 + ch + 8);
+        rv[0] = *reinterpret_cast<const u32x4*>(x + o);
+        rv[1] = *reinterpret_cast<const u32x4*>(x + o + 8);
+        T y[16];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const int ch = (ct0 + c) * 32 + 16 * half;
-            const long o = rc * TR_C + ch;
-            u32x4 bv[2], rv[2];
-            bv[0] = *reinterpret_cast<const u32x4*>(b2 + ch);
-            bv[1] = *reinterpret_cast<const u32x4*>(b2 + ch + 8);
-            rv[0] = *reinterpret_cast<const u32x4*>(x + o);
-            rv[1] = *reinterpret_cast<const u32x4*>(x + o + 8);
-            T y[16];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float u = acc2[m][c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7];
-                y[v] = (T)((float)(T)u + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7]);
-            }
-            if (ok) {
-                *reinterpret_cast<u32x4*>(out + o) = *reinterpret_cast<const u32x4*>(&y[0]);
-                *reinterpret_cast<u32x4*>(out + o + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
-            }
+        for (int v = 0; v < 16; ++v) {
+            const float u = acc2[c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7];
+            y[v] = (T)((float)(T)u + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7]);
+        }
+        if (ok) {
+            *reinterpret_cast<u32x4*>(out + o) = *reinterpret_cast<const u32x4*>(&y[0]);
+            *reinterpret_cast<u32x4*>(out + o + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
     }
 }
@@ -228,7 +207,7 @@ extern "C" int ffk_transition_fused(void* out, const void* x, const void* gamma,
     FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(x) && ffk_aligned16(gamma) && ffk_aligned16(beta) && ffk_aligned16(w1) &&
                     ffk_aligned16(w2) && ffk_aligned16(b2),
                 FFK_ERR_ALIGN, "ffk_transition_fused: buffers must be 16-byte aligned");
-    const size_t smem = 2 * (size_t)TR_A2 + 3 * TR_W2SLOT + 2 * TR_W1SLOT + TR_H * sizeof(float);
+    const size_t smem = 2 * (size_t)TR_W1SLOT + 2 * TR_W2SLOT + TR_H * sizeof(float);
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)transition_fused_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
