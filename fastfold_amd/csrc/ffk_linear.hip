@@ -477,6 +477,13 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
         FFK_REQUIRE((d->a_so * es) % 16 == 0 && (d->a_si * es) % 16 == 0, FFK_ERR_ALIGN,
                     "ffk_fused_linear: row strides of A must be multiples of 16 bytes");
     FFK_REQUIRE(!d->ln_gamma || d->ln_beta, FFK_ERR_NULL, "ffk_fused_linear: ln_beta missing");
+    if (d->a2) {
+        FFK_REQUIRE(d->ln2_gamma && d->ln2_beta, FFK_ERR_NULL, "ffk_fused_linear: the second operand needs ln2_gamma / ln2_beta");
+        FFK_REQUIRE(d->a2_inner > 0, FFK_ERR_SHAPE, "ffk_fused_linear: a2_inner must be positive");
+        FFK_REQUIRE(ffk_aligned16(d->a2) && ffk_aligned16(d->ln2_gamma) && ffk_aligned16(d->ln2_beta) &&
+                        (d->a2_so * es) % 16 == 0 && (d->a2_si * es) % 16 == 0,
+                    FFK_ERR_ALIGN, "ffk_fused_linear: rows of the second operand must be 16-byte aligned");
+    }
     for (int i = 0; i < d->n_tiles; ++i) {
         const ffk_tile& t = d->tiles[i];
         FFK_REQUIRE(t.out, FFK_ERR_NULL, "ffk_fused_linear: tile %d has no output", i);
@@ -509,6 +516,8 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
         int status = FFK_OK;
         if (ffk_linear_ws_try(d, (hipStream_t)stream, &status)) return status;
     }
+    FFK_REQUIRE(!d->a2, FFK_ERR_UNSUPPORTED,
+                "ffk_fused_linear: a second operand needs bf16, K = 128, a channel-major first operand and GLU tiles only");
     if (all_c) return ffk_linear_slab_launch(d, (hipStream_t)stream);
     switch (d->dtype) {
         case FFK_BF16: return launch_linear<bf16_t>(*d, (hipStream_t)stream);

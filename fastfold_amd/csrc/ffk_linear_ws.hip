@@ -256,7 +256,10 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
     }
 }
 
-template <int NS, int WS_K, bool CM>
+// DUAL: the gate halves of the GLU units multiply a second operand (row-major rows, own LayerNorm).  Its
+// slab goes from global memory straight into LDS (unpadded 256-byte rows, 16-byte columns XOR-swizzled
+// with the row index) one slab ahead and is normalised in place by the threads that requested it.
+template <int NS, int WS_K, bool CM, bool DUAL>
 __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs args) {
     typedef Mma<T> MM;
     typedef WsGeo<WS_K> G;
@@ -268,6 +271,11 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     unsigned char* s_a = smem;                                                 // [2][WS_BM][WS_AP]
     float* s_mask = reinterpret_cast<float*>(smem + 2 * WS_BM * WS_AP);        // [2][WS_BM]
     float* s_bias = s_mask + 2 * WS_BM;                                        // [n_tiles][128]
+    unsigned char* s_a2 = reinterpret_cast<unsigned char*>(s_bias + FFK_MAX_TILES * 128);   // DUAL: [2][WS_BM][256 B]
+    static_assert(!DUAL || (WS_K == 128 && WS_BM == 128), "the second operand is built for K = 128");
+    // LayerNorm parameters that are only needed when a slab is committed wait in LDS, not in registers
+    float* s_cmln = reinterpret_cast<float*>(s_a2 + (DUAL ? 2 * WS_BM * 256 : 0));          // CM: gamma[128], beta[128] (fp32)
+    T* s_ln2 = reinterpret_cast<T*>(s_cmln + (CM ? 256 : 0));                               // DUAL: gamma2[128], beta2[128]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
@@ -328,17 +336,20 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const int c8 = tid % LPR, r0 = tid / LPR;
     const bool ln = d.ln_gamma != nullptr;
     Vec16<T> gam, bet;                                   // kept packed: registers are scarce here
-    float cm_g[4], cm_b[4];                              // channel-major A: gamma / beta of this lane's four channels
     if (ln && !CM) {
         gam = ld16((const T*)d.ln_gamma + c8 * 8);
         bet = ld16((const T*)d.ln_beta + c8 * 8);
     }
-    if (ln && CM) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            cm_g[i] = (float)((const T*)d.ln_gamma)[(lane & 31) + 32 * i];
-            cm_b[i] = (float)((const T*)d.ln_beta)[(lane & 31) + 32 * i];
+    if (CM || DUAL) {
+        if (ln && CM && tid < 128) {
+            s_cmln[tid] = (float)((const T*)d.ln_gamma)[tid];
+            s_cmln[128 + tid] = (float)((const T*)d.ln_beta)[tid];
         }
+        if (DUAL && tid < 128) {
+            s_ln2[tid] = ((const T*)d.ln2_gamma)[tid];
+            s_ln2[128 + tid] = ((const T*)d.ln2_beta)[tid];
+        }
+        lds_barrier();
     }
     // row mask of the launch (all masked tiles share it): fetched with the slab, kept in LDS as fp32
     const int mt = args.plan.mask_tile;
@@ -352,7 +363,25 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     // 2w and 2w + 1 of the slab, so the LayerNorm reduction over k stays inside 32 lanes.  The slab is
     // transposed on its way into LDS (2-byte stores, consecutive lanes -> consecutive k of one row).
     const int cm_k = lane & 31, cm_mg = 2 * wave + (lane >> 5);
-    auto fetch = [&](int slab) {
+    // second operand: vector v = i * 512 + tid of a slab is row v / 16, LDS column v % 16, which holds
+    // global column (v % 16) ^ (row % 16); the 16 lanes of a row are adjacent, as the LayerNorm wants them
+    const int a2_col = (tid & 15) ^ ((tid >> 4) & 15);
+    const unsigned lds_a2 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)s_a2;
+    auto fetch = [&](int slab, int tobuf) {
+        if (DUAL) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                long m = (long)slab * WS_BM + i * 32 + (tid >> 4);
+                m = m < M ? m : M - 1;
+                const unsigned hi = (unsigned)m / (unsigned)d.a2_inner, lo = (unsigned)m - hi * (unsigned)d.a2_inner;
+                const T* gp = (const T*)d.a2 + (long)hi * d.a2_so + (long)lo * d.a2_si + a2_col * 8;
+                const unsigned dst = lds_a2 + tobuf * (WS_BM * 256) + (i * WS_THREADS + wave * 64) * 16;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gp), "s"(dst) : "memory", "m0");
+#pragma clang diagnostic pop
+            }
+        }
         if (CM) {
             long m = (long)slab * WS_BM + cm_mg * 8;
             m = m < M ? m : M - 8;                       // M % 8 == 0; clamped groups are never stored
@@ -376,6 +405,33 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     };
     auto commit = [&](int buf) {
         unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
+        if (DUAL) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's vectors of the second operand have landed
+            const Vec16<T> gam2 = *reinterpret_cast<const Vec16<T>*>(s_ln2 + a2_col * 8);
+            const Vec16<T> bet2 = *reinterpret_cast<const Vec16<T>*>(s_ln2 + 128 + a2_col * 8);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                Vec16<T>* px = reinterpret_cast<Vec16<T>*>(s_a2 + buf * (WS_BM * 256) + (i * WS_THREADS + tid) * 16);
+                Vec16<T> x = *px;
+                float f[8], sm = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    f[e] = (float)x.e[e];
+                    sm += f[e];
+                }
+                const float mu = group_sum(sm, 16) * (1.0f / WS_K);
+                float q = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    f[e] -= mu;
+                    q += f[e] * f[e];
+                }
+                const float rs = rsqrtf(group_sum(q, 16) * (1.0f / WS_K) + d.ln_eps);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x.e[e] = (T)(f[e] * rs * (float)gam2.e[e] + (float)bet2.e[e]);
+                *px = x;
+            }
+        }
         if (CM) {
             float f[4][8];
 #pragma unroll
@@ -383,6 +439,12 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 #pragma unroll
                 for (int j = 0; j < 8; ++j) f[i][j] = (float)pre[i].e[j];
             if (ln) {
+                float cm_g[4], cm_b[4];                  // gamma / beta of this lane's four channels
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    cm_g[i] = s_cmln[(lane & 31) + 32 * i];
+                    cm_b[i] = s_cmln[128 + (lane & 31) + 32 * i];
+                }
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float mu = group_sum((f[0][j] + f[1][j]) + (f[2][j] + f[3][j]), 32) * (1.0f / WS_K);
@@ -432,13 +494,13 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 
     const int nslabs = (M + WS_BM - 1) / WS_BM;
     int slab = blockIdx.x;                               // grid <= nslabs
-    fetch(slab);
+    fetch(slab, 0);
     commit(0);
     lds_barrier();
     int buf = 0;
     for (; slab < nslabs; slab += gridDim.x) {
         const int nxt = slab + (int)gridDim.x < nslabs ? slab + (int)gridDim.x : slab;
-        fetch(nxt);                                      // in flight during the products below
+        fetch(nxt, buf ^ 1);                             // in flight during the products below
         const unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
         for (int rg = rg_first; rg < WS_RG; rg += rg_step) {
             const long m0g = (long)slab * WS_BM + rg * 32;
@@ -467,6 +529,19 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
                 const bool rows = by_rows[s];
+                if (DUAL && ALLOW_GLU && glu) {
+                    // gate half: fragments of the second operand's row (row % 16 == l32 % 16 picks the swizzle)
+                    const unsigned a2row = (unsigned)(buf * (WS_BM * 256) + (rg * 32 + n32) * 256 + ((half ^ (n32 & 15)) << 4));
+#pragma unroll
+                    for (int k0 = 0; k0 < WS_KS; k0 += AFC) {
+                        bf16x8 af[AFC];
+#pragma unroll
+                        for (int ks = 0; ks < AFC; ++ks)
+                            af[ks] = *reinterpret_cast<const bf16x8*>(s_a2 + ((a2row + reread) ^ (unsigned)((k0 + ks) * 32)));
+#pragma unroll
+                        for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
+                    }
+                }
 #pragma unroll
                 for (int k0 = 0; k0 < WS_KS; k0 += AFC) {          // AFC K steps of A in registers at a time
                     bf16x8 af[AFC];
@@ -475,7 +550,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                     if (rows) {
 #pragma unroll
                         for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, wf[s][k0 + ks], af[ks]);
-                        if (ALLOW_GLU && glu) {
+                        if (!DUAL && ALLOW_GLU && glu) {
 #pragma unroll
                             for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
                         }
@@ -612,20 +687,21 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p, int rg_per_slab, int max_
     return true;
 }
 
-template <int NS, int K, bool CM>
+template <int NS, int K, bool CM, bool DUAL = false>
 int ws_launch(const WsArgs& args, hipStream_t st) {
     constexpr int WS_BM = WsGeo<K>::BM;
-    const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float);
+    const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float) +
+                        (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) : 0) + (CM ? 256 * sizeof(float) : 0);
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K, CM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K, CM, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess)
             return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
         configured = true;
     }
     const int nslabs = ffk_cdiv(args.d.M, WS_BM);
     const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
-    linear_ws_kernel<NS, K, CM><<<grid, WS_THREADS, smem, st>>>(args);
+    linear_ws_kernel<NS, K, CM, DUAL><<<grid, WS_THREADS, smem, st>>>(args);
     return ffk_check_launch("ffk_fused_linear");
 }
 
@@ -664,7 +740,13 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     args.plan.row_perm = chan_major ? 1 : 0;
     args.plan.mask_tile = mask_tile;
     args.d = *d;
-    if (d->a_chanmajor) {
+    if (d->a2) {
+        // second operand: every unit must be a GLU unit stored [row][channel], first operand channel-major
+        if (!d->a_chanmajor || args.plan.max_slots > 2 || mask_tile >= 0 || d->a2_si % 8 || d->a2_so % 8) return 0;
+        for (int i = 0; i < d->n_tiles; ++i)
+            if (!d->tiles[i].glu || !ws_by_rows(d->tiles[i])) return 0;
+        *status = ws_launch<2, 128, true, true>(args, st);
+    } else if (d->a_chanmajor) {
         if (args.plan.max_slots > 2 || mask_tile >= 0) return 0;
         *status = ws_launch<2, 128, true>(args, st);
     } else if (k256) {

@@ -6,6 +6,7 @@ weight version).  Row-addressing conventions are those of ``ffk_fused_linear``: 
 ``m = hi * inner + lo`` lives at ``hi * s_o + lo * s_i``.
 """
 import math
+import os
 
 import torch
 
@@ -225,16 +226,39 @@ def pack_trimul(proj_w, proj_b, gate_w, gate_b, og_w, og_b, c, dtype, device):
     return torch.cat([w, wg], 0).contiguous(), torch.cat([b, bg], 0).contiguous(), n_glu
 
 
-def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask):
+def pack_trimul_out(out_w, out_b, og_w, og_b, C, dtype, device):
+    """Output stage with the gate computed in the same launch: GLU tiles of 64 channels,
+    [Wout c0..c0+31 | Wog c0..c0+31 | Wout c0+32..c0+63 | Wog c0+32..c0+63] (biases alike)."""
+    ws, bs = [], []
+    for t in range(C // 64):
+        for q in range(2):
+            sl = slice(t * 64 + q * 32, t * 64 + q * 32 + 32)
+            ws += [out_w[sl], og_w[sl]]
+            bs += [out_b[sl], og_b[sl]]
+    return pack_rows(ws, dtype, device), pack_vec(bs, dtype, device)
+
+
+def trimul_gate_in_output_stage(dtype, r, C, c):
+    """The output gate sigmoid(Wg LN(z) + bg) can be computed inside the output stage (second operand
+    of the projection kernel) instead of being written by the first stage and read back."""
+    if os.environ.get("FFK_NO_WS") or os.environ.get("FFK_TRIMUL_GATE_FIRST"):    # debugging knobs: the two-pass form
+        return False
+    return dtype == torch.bfloat16 and C == 128 and c == 128 and r % 8 == 0
+
+
+def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,
+                            dual_pk=None):
     """out = z + sigmoid(Wg LN(z) + bg) * (Wout LN2(p) + b_out),  p[i,j,:] = sum_k a[i,k,:] b[j,k,:]
-    (outgoing) or sum_k a[k,i,:] b[k,j,:] (incoming), a/b the masked gated projections."""
+    (outgoing) or sum_k a[k,i,:] b[k,j,:] (incoming), a/b the masked gated projections.
+    ``dual_pk`` = (weights, biases) of pack_trimul_out: the gate is then computed in the output stage."""
     dt, dev = z.dtype, z.device
     es = es_of(dt)
     M = r * r
     kpad = round_up(r, vec_of(dt))
     zero = kpad != r
     lr = alloc((2, c, r, kpad), dt, dev, zero)
-    g = torch.empty(M, C, dtype=dt, device=dev)
+    dual = dual_pk is not None and trimul_gate_in_output_stage(dt, r, C, c)
+    g = None if dual else torch.empty(M, C, dtype=dt, device=dev)
     tiles = []
     if incoming:      # logical row (a, b) reads z[b, a]
         a_map, m_so, m_si = (r, C, r * C), 1, r
@@ -246,7 +270,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
             tiles.append(make_tile(lr.data_ptr() + (side * c + t * 64) * r * kpad * es,
                                    bias=b_pk.data_ptr() + ti * 128 * es, glu=1, ncols=64, inner=r, s_o=kpad, s_i=1,
                                    s_h=32 * r * kpad, s_d=r * kpad, rowmask=mask, m_so=m_so, m_si=m_si))
-    for t in range((C + 127) // 128):
+    for t in range((C + 127) // 128 if not dual else 0):
         kw = dict(inner=r, s_o=C, s_i=r * C) if incoming else dict(inner=M, s_i=C)
         tiles.append(make_tile(g.data_ptr() + t * 128 * es, bias=b_pk.data_ptr() + (n_glu + t) * 128 * es,
                                act=FFK_ACT_SIGMOID, ncols=min(128, C - t * 128), **kw))
@@ -255,6 +279,13 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     _lib.bgemm_nt(lr[0], lr[1], p, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=c, a_bs=r * kpad, b_bs=r * kpad,
                   o_bs=r * kpad, s_i=kpad)
     del lr
+    if dual:
+        wd, bd = dual_pk
+        tiles = [make_tile(out.data_ptr() + t * 64 * es, bias=bd.data_ptr() + t * 128 * es, glu=1, ncols=64,
+                           resid=z.data_ptr() + t * 64 * es, inner=M, s_i=C) for t in range(C // 64)]
+        _lib.fused_linear(p, wd, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
+                          ln=ln2, a2=z, ln2=ln1, a2_inner=M, a2_si=C)
+        return out
     tiles = []
     for t in range((C + 127) // 128):
         tiles.append(make_tile(out.data_ptr() + t * 128 * es, bias=out_bias_pk.data_ptr() + t * 128 * es,

@@ -329,13 +329,17 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
             w, b, n_glu = F_.pack_trimul(self.left_right_projection.weight, self.left_right_projection.bias,
                                          self.left_right_gate.weight, self.left_right_gate.bias,
                                          self.output_gate.weight, self.output_gate.bias, self.c, dt, dev)
+            dual = None
+            if F_.trimul_gate_in_output_stage(dt, r, C, self.c):
+                dual = F_.pack_trimul_out(self.output_projection.weight, self.output_bias, self.output_gate.weight,
+                                          self.output_gate.bias, C, dt, dev)
             return (w, b, n_glu, F_.pack_rows([self.output_projection.weight], dt, dev),
-                    F_.pack_vec([self.output_bias], dt, dev))
-        w, b, n_glu, wout, bout = self._packed(("tm", dt, dev), ps, build)
+                    F_.pack_vec([self.output_bias], dt, dev), dual)
+        w, b, n_glu, wout, bout, dual = self._packed(("tm", dt, dev, r % 8 == 0), ps, build)
         F_.triangle_multiplication(Z_raw, out, r=r, C=C, c=self.c, incoming=self._incoming,
                                    ln1=_ln_pair(self.layernorm1, dt), w_pk=w, b_pk=b, n_glu=n_glu,
                                    ln2=_ln_pair(self.layernorm2, dt), wout_pk=wout, out_bias_pk=bout,
-                                   mask=_mask_like(Z_mask, Z_raw))
+                                   mask=_mask_like(Z_mask, Z_raw), dual_pk=dual)
         return out
 
     def forward(self, Z_raw, Z_mask):

@@ -167,6 +167,17 @@ typedef struct ffk_linear_desc {
     int32_t dtype;
     const void* w;         /* [n_tiles * 128, K] row-major, zero-padded rows */
     int32_t M, K, n_tiles, reserved;
+    /* Optional second operand (NULL = none): the gate halves of the GLU tiles are then computed from
+       LayerNorm(a2) with ln2_gamma / ln2_beta instead of from the first operand.  a2 is K-contiguous,
+       logical row m at  a2 + (m / a2_inner) * a2_so + (m % a2_inner) * a2_si.  Built for bf16, K = 128
+       and a channel-major first operand (the output stage of the triangle multiplication, whose gate
+       comes from the pair tensor and whose value from the contraction result); other combinations
+       return FFK_ERR_UNSUPPORTED. */
+    const void* a2;
+    const void* ln2_gamma;
+    const void* ln2_beta;
+    int64_t a2_so, a2_si;
+    int32_t a2_inner, reserved2;
     ffk_tile tiles[FFK_MAX_TILES];
 } ffk_linear_desc;
 

@@ -389,3 +389,45 @@ def test_transition_fused_kernel(dev, M):
     assert torch.equal(x2, out)
     with pytest.raises(RuntimeError):
         _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=64, hidden=256)
+
+
+@pytest.mark.parametrize("r", [64, 104])
+def test_fused_linear_second_operand(dev, r):
+    """GLU tiles whose gate halves come from a second operand with its own LayerNorm (the output stage of the
+    triangle multiplication): out = resid + (W_p LN2(p) + b_p) * sigmoid(W_g LN1(z) + b_g), p channel-major."""
+    from fastfold_amd import _lib
+    dtype = torch.bfloat16
+    C, M = 128, r * r
+    g = torch.Generator().manual_seed(r)
+    p_cm = (torch.randn(C, r, r, generator=g) * 2 + 0.3).to(dev, dtype)            # [c, i, j]
+    z = (torch.randn(M, C, generator=g) * 1.5 - 0.2).to(dev, dtype)
+    gam1, gam2 = ((1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype) for _ in range(2))
+    bet1, bet2 = ((0.1 * torch.randn(C, generator=g)).to(dev, dtype) for _ in range(2))
+    wp, wg = ((torch.randn(C, C, generator=g) / C ** 0.5).to(dev, dtype) for _ in range(2))
+    bp, bg = (torch.randn(C, generator=g).to(dev, dtype) for _ in range(2))
+    ws, bs = [], []
+    for t in range(2):
+        for q in range(2):
+            sl = slice(t * 64 + q * 32, t * 64 + q * 32 + 32)
+            ws += [wp[sl], wg[sl]]
+            bs += [bp[sl], bg[sl]]
+    w_pk, b_pk = torch.cat(ws, 0).contiguous(), torch.cat(bs, 0).contiguous()
+    out = torch.empty(M, C, device=dev, dtype=dtype)
+    tiles = [_lib.make_tile(out.data_ptr() + t * 64 * 2, bias=b_pk.data_ptr() + t * 128 * 2, glu=1, ncols=64,
+                            resid=z.data_ptr() + t * 64 * 2, inner=M, s_i=C) for t in range(2)]
+    _lib.fused_linear(p_cm, w_pk, tiles, M=M, K=C, a_inner=r, a_so=r, a_si=1, a_chanmajor=True, a_cs=r * r,
+                      ln=(gam2, bet2), a2=z, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
+    pn = _np(torch.from_numpy(ops_np.layer_norm(_np(p_cm).reshape(C, M).T, _np(gam2), _np(bet2))).to(dtype))
+    zn = _np(torch.from_numpy(ops_np.layer_norm(_np(z), _np(gam1), _np(bet1))).to(dtype))
+    upd = ops_np.linear(pn, _np(wp), _np(bp)) / (1 + np.exp(-ops_np.linear(zn, _np(wg), _np(bg))))
+    assert _rel(_np(out) - _np(z), upd) < TOL[dtype]
+    # in place on the second operand / residual
+    z2 = z.clone()
+    tiles = [_lib.make_tile(z2.data_ptr() + t * 64 * 2, bias=b_pk.data_ptr() + t * 128 * 2, glu=1, ncols=64,
+                            resid=z2.data_ptr() + t * 64 * 2, inner=M, s_i=C) for t in range(2)]
+    _lib.fused_linear(p_cm, w_pk, tiles, M=M, K=C, a_inner=r, a_so=r, a_si=1, a_chanmajor=True, a_cs=r * r,
+                      ln=(gam2, bet2), a2=z2, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
+    assert torch.equal(z2, out)
+    # a second operand without the shapes it is built for is refused, not ignored
+    with pytest.raises(RuntimeError):
+        _lib.fused_linear(z, w_pk, tiles, M=M, K=C, ln=(gam2, bet2), a2=z, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
