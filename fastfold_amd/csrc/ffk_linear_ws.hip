@@ -276,6 +276,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     // LayerNorm parameters that are only needed when a slab is committed wait in LDS, not in registers
     float* s_cmln = reinterpret_cast<float*>(s_a2 + (DUAL ? 2 * WS_BM * 256 : 0));          // CM: gamma[128], beta[128] (fp32)
     T* s_ln2 = reinterpret_cast<T*>(s_cmln + (CM ? 256 : 0));                               // DUAL: gamma2[128], beta2[128]
+    T* s_ln1 = s_ln2 + (DUAL ? 256 : 0);                                                    // !CM: gamma[K], beta[K]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
@@ -335,12 +336,11 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     // ---- slab streaming: thread -> (row tid / LPR + RPP * i, 8 channels starting at 8 * (tid % LPR)) ----
     const int c8 = tid % LPR, r0 = tid / LPR;
     const bool ln = d.ln_gamma != nullptr;
-    Vec16<T> gam, bet;                                   // kept packed: registers are scarce here
-    if (ln && !CM) {
-        gam = ld16((const T*)d.ln_gamma + c8 * 8);
-        bet = ld16((const T*)d.ln_beta + c8 * 8);
-    }
-    if (CM || DUAL) {
+    {
+        if (ln && !CM && tid < WS_K) {
+            s_ln1[tid] = ((const T*)d.ln_gamma)[tid];
+            s_ln1[WS_K + tid] = ((const T*)d.ln_beta)[tid];
+        }
         if (ln && CM && tid < 128) {
             s_cmln[tid] = (float)((const T*)d.ln_gamma)[tid];
             s_cmln[128 + tid] = (float)((const T*)d.ln_beta)[tid];
@@ -470,6 +470,8 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         for (int i = 0; i < 4; ++i) {
             Vec16<T> x = pre[i];
             if (ln) {
+                const Vec16<T> gam = *reinterpret_cast<const Vec16<T>*>(s_ln1 + c8 * 8);
+                const Vec16<T> bet = *reinterpret_cast<const Vec16<T>*>(s_ln1 + WS_K + c8 * 8);
                 float f[8], s = 0.0f;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -691,7 +693,7 @@ template <int NS, int K, bool CM, bool DUAL = false>
 int ws_launch(const WsArgs& args, hipStream_t st) {
     constexpr int WS_BM = WsGeo<K>::BM;
     const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float) +
-                        (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) : 0) + (CM ? 256 * sizeof(float) : 0);
+                        (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) : 0) + (CM ? 256 * sizeof(float) : 2 * K * sizeof(T));
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K, CM, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
