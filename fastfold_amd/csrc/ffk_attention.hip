@@ -311,7 +311,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
             float mt = fmaxf(s[0], s[1]);
 #pragma unroll
             for (int v = 2; v < 16; ++v) mt = fmaxf(mt, s[v]);
-            const float mfull = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float mfull = fmaxf(mt, lane_xor<32>(mt));
             const float delta = first ? fmaxf(mfull, REF_FLOOR) : fmaxf(mfull, 0.0f);
             const float alpha = first ? 1.0f : fast_exp2(-delta);   // nothing accumulated before the first tile
 #pragma unroll
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // rows whose keys are all masked have l == 0 and produce zeros
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float l_tot = l_run + lane_xor<32>(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     if (live && q < Nq) {
         T gv[4][4];

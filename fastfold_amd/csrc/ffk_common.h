@@ -82,13 +82,58 @@ template <typename T> __device__ __forceinline__ void st16_nt(T* p, const Vec16<
 }
 
 // ------------------------------------------------------- wave reductions ----
-// Reduce over groups of `width` adjacent lanes (width a power of two <= 64).
+// lane_xor<W>(v): the value of lane (l ^ W) for a v that is already uniform over aligned groups of W
+// lanes - which is all a butterfly reduction needs.  1 and 2 are quad permutes, 4 and 8 the half-row
+// and row mirrors of the DPP unit (lane i reads lane 7 - i / 15 - i: another lane of the partner group,
+// holding the same value as lane i ^ W), 16 and 32 the row / half-wave swap instructions.  None of them
+// goes through the LDS crossbar, unlike a general shuffle.
+template <int W> __device__ __forceinline__ float lane_xor(float v) {
+    const int x = __builtin_bit_cast(int, v);
+    int r;
+    if (W == 1) r = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false);          // quad_perm [1,0,3,2]
+    else if (W == 2) r = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false);     // quad_perm [2,3,0,1]
+    else if (W == 4) r = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false);    // row_half_mirror
+    else if (W == 8) r = __builtin_amdgcn_update_dpp(x, x, 0x140, 0xF, 0xF, false);    // row_mirror
+    else if (W == 16) {
+        // a = b = v;  swap(a rows 1 / 3, b rows 0 / 2):  a = [r0 r0 r2 r2], b = [r1 r1 r3 r3]
+        typedef unsigned u2 __attribute__((ext_vector_type(2)));
+        const u2 p = __builtin_amdgcn_permlane16_swap((unsigned)x, (unsigned)x, false, false);
+        const int lane_row = (__lane_id() >> 4) & 1;
+        r = (int)(lane_row ? p[0] : p[1]);
+    } else {
+        typedef unsigned u2 __attribute__((ext_vector_type(2)));
+        const u2 p = __builtin_amdgcn_permlane32_swap((unsigned)x, (unsigned)x, false, false);
+        r = (int)((__lane_id() >> 5) ? p[0] : p[1]);
+    }
+    return __builtin_bit_cast(float, r);
+}
+// Reduce over groups of `width` adjacent lanes (width a power of two <= 64); every lane gets the result.
+// The streaming row kernels, whose group size is a run-time value, measured faster with the general
+// shuffles (softmax 59.5 vs 64 us) and keep them.
 __device__ __forceinline__ float group_sum(float v, int width) {
-    for (int off = width >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (!__builtin_constant_p(width)) {     // group size only known at run time (the row kernels): general shuffles
+        for (int off = width >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+        return v;
+    }
+    if (width >= 2) v += lane_xor<1>(v);
+    if (width >= 4) v += lane_xor<2>(v);
+    if (width >= 8) v += lane_xor<4>(v);
+    if (width >= 16) v += lane_xor<8>(v);
+    if (width >= 32) v += lane_xor<16>(v);
+    if (width >= 64) v += lane_xor<32>(v);
     return v;
 }
 __device__ __forceinline__ float group_max(float v, int width) {
-    for (int off = width >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    if (!__builtin_constant_p(width)) {
+        for (int off = width >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+        return v;
+    }
+    if (width >= 2) v = fmaxf(v, lane_xor<1>(v));
+    if (width >= 4) v = fmaxf(v, lane_xor<2>(v));
+    if (width >= 8) v = fmaxf(v, lane_xor<4>(v));
+    if (width >= 16) v = fmaxf(v, lane_xor<8>(v));
+    if (width >= 32) v = fmaxf(v, lane_xor<16>(v));
+    if (width >= 64) v = fmaxf(v, lane_xor<32>(v));
     return v;
 }
 
