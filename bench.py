@@ -219,6 +219,20 @@ def main():
                    "stack_tflops": round(block_gflop(s, r) * args.blocks / ms_per_step, 1)},
         "roofline": roofline,
     }
+    if args.workload == "cfg4" and not args.no_micro:
+        # the same stack at BASELINE configs[2] (N_res = 256), reported beside the headline number
+        w3 = WORKLOADS["cfg3"]
+        m3, z3, mm3, pm3 = (torch.from_numpy(t).to(dev, torch.bfloat16)
+                            for t in synth_inputs(0, w3["n_seq"], w3["n_res"], mask_tail_frac=w3["tail"]))
+        with torch.no_grad():
+            stack(m3, z3, mm3, pm3, chunk_size=None)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                stack(m3, z3, mm3, pm3, chunk_size=None)
+            torch.cuda.synchronize()
+        line["secondary"] = {"workload": w3["name"], "ms_per_block": round((time.perf_counter() - t0) * 1e3 / 3 / args.blocks, 4)}
+        del m3, z3, mm3, pm3
     del stack, out
     torch.cuda.empty_cache()
     if not args.no_micro:
