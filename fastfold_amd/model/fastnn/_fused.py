@@ -5,6 +5,7 @@ C-ABI calls only; torch is used for buffer allocation and for re-packing weights
 weight version).  Row-addressing conventions are those of ``ffk_fused_linear``: logical row
 ``m = hi * inner + lo`` lives at ``hi * s_o + lo * s_i``.
 """
+import contextlib
 import math
 import os
 
@@ -56,6 +57,37 @@ def check_cuda(*ts):
         if t is not None and not t.is_cuda:
             raise RuntimeError("fastfold_amd: the Evoformer modules run on the GPU only "
                                "(got a %s tensor); there is no CPU fallback" % t.device)
+
+
+# ---- values derived from a mask only (key bias + tile flags of an attention, the normaliser of the outer
+# product mean) are the same in every block of a stack: inside `mask_cache()` they are computed once ----
+_MASK_CACHE = None
+
+
+@contextlib.contextmanager
+def mask_cache():
+    """While active, launches whose result depends only on a mask tensor are done once per distinct
+    (storage, view geometry, version) and reused.  Entries keep their mask alive, so its memory cannot be
+    handed to another tensor while the entry exists; the cache dies with the context."""
+    global _MASK_CACHE
+    prev, _MASK_CACHE = _MASK_CACHE, (None if os.environ.get("FFK_NO_MASK_CACHE") else [])
+    try:
+        yield
+    finally:
+        _MASK_CACHE = prev
+
+
+def _mask_derived(mask, what, build):
+    if _MASK_CACHE is None:
+        return build()
+    key = (what, mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype)
+    for k, _, v in _MASK_CACHE:
+        if k == key:
+            return v
+    v = build()
+    if len(_MASK_CACHE) < 32:          # a stack needs about ten; bounded whatever the caller does
+        _MASK_CACHE.append((key, mask, v))
+    return v
 
 
 def fits_fused(K, dtype):
@@ -175,9 +207,12 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         scratch = torch.empty(16 * C + 16, dtype=torch.float32, device=dev)
         _lib.pair_bias(bias_t, x, ln[0], ln[1], w_pk[4 * tpg * 128:], scratch, N=N, C=C, H=H, a_inner=a_inner,
                        a_so=a_so, a_si=a_si, scale=LOG2E)
-    kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
-    flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
-    _lib.key_bias(kb, flags, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
+    def key_bias():
+        kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
+        flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
+        _lib.key_bias(kb, flags, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
+        return kb, flags
+    kb, flags = _mask_derived(mask, ("key_bias", B2, N, mask_sb, mask_sn), key_bias) if mask is not None else key_bias()
     o = torch.empty(M, HC, dtype=dt, device=dev)
     _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, flags, gate, B2=B2, H=H, Nq=N, Nk=N, gate_tiled=acc_order)
     del q_t, k_t, v_t, gate
@@ -308,10 +343,13 @@ def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, 
                      rowmask=mask, m_so=1, m_si=r)
     # logical row (i, s') reads m[s', i]
     _lib.fused_linear(m, wab_pk, [tile], M=s * r, K=C, a_inner=s, a_so=C, a_si=r * C, ln=ln)
-    mt = torch.zeros(r, spad, dtype=dt, device=dev)
-    mt[:, :s] = mask.t()
-    nrm = torch.empty(r, r, dtype=torch.float32, device=dev)
-    _lib.bgemm_nt(mt, mt, nrm, M=r, N=r, K=spad, lda=spad, ldb=spad, out_f32=True)
+    def normaliser():
+        mt = torch.zeros(r, spad, dtype=dt, device=dev)
+        mt[:, :s] = mask.t()
+        nrm = torch.empty(r, r, dtype=torch.float32, device=dev)
+        _lib.bgemm_nt(mt, mt, nrm, M=r, N=r, K=spad, lda=spad, ldb=spad, out_f32=True)
+        return nrm
+    nrm = _mask_derived(mask, ("opm_norm", s, r, spad), normaliser)
     if wo_ed is not None and dt == torch.bfloat16 and Cz == 128 and r % 32 == 0 and spad in (64, 128):
         # fused core: the [r, r, 1024] outer product never leaves the chip
         _lib.opm_fused(out, z, ab[0], ab[1], wo_ed, bo, nrm, r=r, spad=spad, eps=eps)

@@ -15,6 +15,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import _fused as F_
 from .msa import MSACore
 from .ops import Linear, OutProductMean
 from .triangle import PairCore
@@ -109,10 +110,11 @@ class EvoformerStack(nn.Module):
     def _run(self, m, z, msa_mask, pair_mask, inplace_first: bool):
         mm, zz = m.unsqueeze(0), z.unsqueeze(0)
         mk, pk = msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)
-        for i, b in enumerate(self.blocks):
-            if self.clear_cache_between_blocks:
-                torch.cuda.empty_cache()
-            mm, zz = b._core(mm.contiguous(), zz.contiguous(), mk, pk, inplace=(inplace_first or i > 0))
+        with F_.mask_cache():          # key biases / normalisers depend on the masks only: once per stack, not per block
+            for i, b in enumerate(self.blocks):
+                if self.clear_cache_between_blocks:
+                    torch.cuda.empty_cache()
+                mm, zz = b._core(mm.contiguous(), zz.contiguous(), mk, pk, inplace=(inplace_first or i > 0))
         return mm.squeeze(0), zz.squeeze(0)
 
     def forward(self, m: torch.Tensor, z: torch.Tensor, msa_mask: torch.Tensor, pair_mask: torch.Tensor,

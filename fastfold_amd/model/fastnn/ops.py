@@ -64,7 +64,10 @@ def _ln_pair(ln, dtype):
 
 
 def _mask_like(mask, x):
-    return mask.to(dtype=x.dtype).contiguous()
+    if mask.dtype == x.dtype and mask.is_contiguous():
+        return mask
+    # a converted copy is itself derived from the mask only: one per stack, and a stable key for what follows
+    return F_._mask_derived(mask, ("cast", x.dtype), lambda: mask.to(dtype=x.dtype).contiguous())
 
 
 class DropoutRowwise(nn.Module):
