@@ -145,7 +145,7 @@ __global__ void pair_bias_prep_kernel(bf16_t* wop, float* c01, const bf16_t* w, 
 extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w, float* scratch,
                              int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so, int64_t a_si, float scale,
                              float eps, int dtype, void* stream) {
-    FFK_REQUIRE(bias_t && z && gamma && beta && w && scratch, FFK_ERR_NULL, "ffk_pair_bias: null pointer");
+    FFK_REQUIRE(bias_t && z && scratch && (!w || (gamma && beta)), FFK_ERR_NULL, "ffk_pair_bias: null pointer");
     FFK_REQUIRE(dtype == FFK_BF16, FFK_ERR_DTYPE, "ffk_pair_bias: bf16 only (dtype tag %d)", dtype);
     FFK_REQUIRE(C == 128, FFK_ERR_UNSUPPORTED, "ffk_pair_bias: built for 128 pair channels, got %ld", (long)C);
     FFK_REQUIRE(N > 0 && N <= 46340 && H > 0 && H <= PB_MAXH && a_inner > 0, FFK_ERR_SHAPE,
@@ -155,10 +155,12 @@ extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, con
     hipStream_t st = (hipStream_t)stream;
     bf16_t* wop = reinterpret_cast<bf16_t*>(scratch);     // [32][C] bf16 = 16 * C floats
     float* c01 = scratch + 16 * C;                       // [H][2]
-    pair_bias_prep_kernel<<<32, 64, 0, st>>>(wop, c01, (const bf16_t*)w, (const bf16_t*)gamma, (const bf16_t*)beta,
-                                             (int)H, (int)C);
-    int rc = ffk_check_launch("ffk_pair_bias");
-    if (rc != FFK_OK) return rc;
+    if (w) {       // w == NULL: scratch still holds the operand an earlier call built from the same w, gamma, beta
+        pair_bias_prep_kernel<<<32, 64, 0, st>>>(wop, c01, (const bf16_t*)w, (const bf16_t*)gamma, (const bf16_t*)beta,
+                                                 (int)H, (int)C);
+        int rc = ffk_check_launch("ffk_pair_bias");
+        if (rc != FFK_OK) return rc;
+    }
     const size_t smem = 256 * (128 * 2 + 16) + 256 * sizeof(float);
     static bool configured = false;
     if (!configured) {

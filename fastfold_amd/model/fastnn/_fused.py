@@ -90,6 +90,23 @@ def _mask_derived(mask, what, build):
     return v
 
 
+class PairBiasScratch:
+    """Device scratch of ffk_pair_bias together with the fact that it already holds the weight operand
+    (built by the first call from the projection weights and the LayerNorm parameters); modules keep one
+    per packed weight set, so that later calls skip the preparation kernel."""
+
+    def __init__(self, C, device):
+        self.buf = torch.empty(16 * C + 16, dtype=torch.float32, device=device)
+        self.ready = False
+
+
+def _pair_bias_launch(bias_t, x, ln, w, scratch, **kw):
+    if scratch is None:
+        scratch = PairBiasScratch(x.shape[-1], x.device)
+    _lib.pair_bias(bias_t, x, ln[0], ln[1], None if scratch.ready else w, scratch.buf, **kw)
+    scratch.ready = True
+
+
 def fits_fused(K, dtype):
     return K <= 256 and K % 32 == 0
 
@@ -151,7 +168,7 @@ def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
 
 # ---------------------------------------------------------------------- attention ----
 def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_pk, out_bias_pk, c_out,
-              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False):
+              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None):
     """Gated multi-head attention (head dim 32) over N tokens for each of B2 batch rows.
 
     x holds the C-channel rows addressed by ``a_map = (inner, s_o, s_i)``; w_pk is the packed
@@ -204,9 +221,8 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
                           w_row_off=t0 * 128)
     if bias_tile is not None:      # the skinny bias projection has its own pass over x
-        scratch = torch.empty(16 * C + 16, dtype=torch.float32, device=dev)
-        _lib.pair_bias(bias_t, x, ln[0], ln[1], w_pk[4 * tpg * 128:], scratch, N=N, C=C, H=H, a_inner=a_inner,
-                       a_so=a_so, a_si=a_si, scale=LOG2E)
+        _pair_bias_launch(bias_t, x, ln, w_pk[4 * tpg * 128:], pb_scratch, N=N, C=C, H=H, a_inner=a_inner,
+                          a_so=a_so, a_si=a_si, scale=LOG2E)
     def key_bias():
         kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
         flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
@@ -226,14 +242,12 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     return out
 
 
-def pair_bias(z, *, r, C, H, ln, wb_pk):
+def pair_bias(z, *, r, C, H, ln, wb_pk, pb_scratch=None):
     """bias_t[h][q/32][k/32][tile] = log2e * (LN(z)[q, k, :] . Wb[h, :]) in score-accumulator tiles."""
     NT = (r + 31) // 32
     bias_t = alloc((H, NT, NT, 1024), z.dtype, z.device, zero=(r % 32) != 0)
     if z.dtype == torch.bfloat16 and C == 128 and H <= 8:
-        scratch = torch.empty(16 * C + 16, dtype=torch.float32, device=z.device)
-        _lib.pair_bias(bias_t, z, ln[0], ln[1], wb_pk, scratch, N=r, C=C, H=H, a_inner=r * r, a_so=0, a_si=C,
-                       scale=LOG2E)
+        _pair_bias_launch(bias_t, z, ln, wb_pk, pb_scratch, N=r, C=C, H=H, a_inner=r * r, a_so=0, a_si=C, scale=LOG2E)
         return bias_t
     tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=r, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H, scale=LOG2E)
     _lib.fused_linear(z, wb_pk, [tile], M=r * r, K=C, ln=ln)

@@ -45,7 +45,10 @@ class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
                           lambda: F_.pack_rows([self.linear_b_weights], dt, dev))
         ob = self._packed(("ob", dt, dev), [self.out_bias], lambda: F_.pack_vec([self.out_bias], dt, dev))
         w_pk, gb_pk, wo_pk = self.attention.packed(dt, dev)
-        bias_t = F_.pair_bias(Z.contiguous(), r=r, C=Cz, H=self.n_head, ln=_ln_pair(self.layernormZ, dt), wb_pk=wb)
+        pbs = self._packed(("pbs", dt, dev), [self.linear_b_weights, self.layernormZ.weight, self.layernormZ.bias],
+                           lambda: F_.PairBiasScratch(Cz, dev))
+        bias_t = F_.pair_bias(Z.contiguous(), r=r, C=Cz, H=self.n_head, ln=_ln_pair(self.layernormZ, dt), wb_pk=wb,
+                              pb_scratch=pbs)
         mask = _mask_like(M_mask, M_raw)[0]
         F_.attention(M_raw, out, M_raw, B2=s, N=r, C=C, H=self.n_head, a_map=(s * r, 0, C),
                      ln=_ln_pair(self.layernormM, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,

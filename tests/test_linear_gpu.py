@@ -329,6 +329,10 @@ def test_pair_bias_kernel(dev, r, H):
         x = ops_np.layer_norm(zz, _np(gam), _np(bet))
         ref = (ops_np.linear(x, _np(wb)) * _lib.LOG2E).transpose(2, 0, 1)       # [h, q, k]
         assert _rel(_np(layouts.untile_bias(bt, r, r)), ref) < TOL[dtype]
+        # a later call may reuse the weight operand the first one left in scratch (w = None)
+        bt2 = torch.zeros_like(bt)
+        _lib.pair_bias(bt2, z, None, None, None, scratch, N=r, C=C, H=H, scale=_lib.LOG2E, **kw)
+        assert torch.equal(bt2, bt)
         # padding of ragged tiles is left untouched (zero)
         full = _np(layouts.untile_bias(bt, T * 32, T * 32))
         assert np.abs(full[:, r:, :]).max(initial=0.0) == 0.0 and np.abs(full[:, :, r:]).max(initial=0.0) == 0.0
