@@ -78,6 +78,49 @@ def nn_layout_block_shapes(c_m=256, c_z=128, c_hidden_msa_att=32, c_hidden_opm=3
     return out
 
 
+def extra_nn_layout_block_shapes(c_m=64, c_z=128, c_hidden_msa_att=8, c_hidden_opm=32, c_hidden_mul=128,
+                                 c_hidden_pair_att=32, no_heads_msa=8, no_heads_pair=4, transition_n=4):
+    """One extra-MSA block (``fastfold.model.nn.evoformer.ExtraMSABlock``) in draw order: as an Evoformer
+    block, with the column attention replaced by
+      msa_att_col: layer_norm_m, global_attention.linear_{q,k,v}.weight, .linear_g, .linear_o"""
+    base = nn_layout_block_shapes(c_m=c_m, c_z=c_z, c_hidden_msa_att=c_hidden_msa_att, c_hidden_opm=c_hidden_opm,
+                                  c_hidden_mul=c_hidden_mul, c_hidden_pair_att=c_hidden_pair_att,
+                                  no_heads_msa=no_heads_msa, no_heads_pair=no_heads_pair, transition_n=transition_n)
+    hc = c_hidden_msa_att * no_heads_msa
+    g = "msa_att_col.global_attention."
+    col = [("msa_att_col.layer_norm_m.weight", (c_m,), "ln_w"), ("msa_att_col.layer_norm_m.bias", (c_m,), "ln_b"),
+           (g + "linear_q.weight", (hc, c_m), "w"), (g + "linear_k.weight", (c_hidden_msa_att, c_m), "w"),
+           (g + "linear_v.weight", (c_hidden_msa_att, c_m), "w"),
+           (g + "linear_g.weight", (hc, c_m), "w"), (g + "linear_g.bias", (hc,), "b"),
+           (g + "linear_o.weight", (c_m, hc), "w"), (g + "linear_o.bias", (c_m,), "b")]
+    out, done = [], False
+    for ent in base:
+        if ent[0].startswith("msa_att_col."):
+            if not done:
+                out += col
+                done = True
+            continue
+        out.append(ent)
+    return out
+
+
+def synth_extra_nn_state(seed=0, no_blocks=1, std=0.02, fan_in_scaled=False, **dims):
+    """nn-layout state of an ``ExtraMSAStack`` (no final linear), drawn like ``synth_nn_state``."""
+    rng = np.random.RandomState(seed)
+    sd = OrderedDict()
+    for i in range(no_blocks):
+        for name, shape, kind in extra_nn_layout_block_shapes(**dims):
+            x = rng.standard_normal(shape).astype(np.float32)
+            if kind == "ln_w":
+                x = 1.0 + std * x
+            elif kind == "w" and fan_in_scaled:
+                x = x / np.sqrt(shape[1])
+            else:
+                x = std * x
+            sd["blocks.%d.%s" % (i, name)] = x.astype(np.float32)
+    return sd
+
+
 def synth_nn_state(seed=0, no_blocks=1, std=0.02, c_m=256, c_z=128, c_s=384, fan_in_scaled=False, **dims):
     """OrderedDict name -> float32 numpy array, nn layout, for an ``EvoformerStack``.
 

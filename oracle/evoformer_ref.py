@@ -373,10 +373,103 @@ class EvoformerStack(nn.Module):
         return m, z, s
 
 
+# --------------------------------------------------------------------------
+# extra-MSA stack  (reference: fastfold/model/nn/primitives.py:422-504,
+# fastfold/model/nn/msa.py:322-392, fastfold/model/nn/evoformer.py:293-389,538-633)
+# --------------------------------------------------------------------------
+class GlobalAttention(nn.Module):
+    """One query per column (the masked mean over the sequences), one key / value head shared
+    by all query heads (primitives.py:452-504):
+      q = W_q (sum_s mask x / (sum_s mask + eps)) / sqrt(c), k = W_k x, v = W_v x  (c wide),
+      a[h, s] = softmax_s(q[h] . k[s] + inf * (mask[s] - 1)), o[h] = sum_s a[h, s] v[s],
+      out[s] = W_o (sigmoid(W_g x[s] + b_g) * o) + b_o."""
+
+    def __init__(self, c_in, c_hidden, no_heads, inf, eps):
+        super().__init__()
+        self.c_in, self.c_hidden, self.no_heads, self.inf, self.eps = c_in, c_hidden, no_heads, inf, eps
+        self.linear_q = Linear(c_in, c_hidden * no_heads, bias=False, init="glorot")
+        self.linear_k = Linear(c_in, c_hidden, bias=False, init="glorot")
+        self.linear_v = Linear(c_in, c_hidden, bias=False, init="glorot")
+        self.linear_g = Linear(c_in, c_hidden * no_heads, init="gating")
+        self.linear_o = Linear(c_hidden * no_heads, c_in, init="final")
+
+    def forward(self, m, mask):
+        H, D = self.no_heads, self.c_hidden
+        q = (m * mask.unsqueeze(-1)).sum(-2) / (mask.sum(-1)[..., None] + self.eps)     # [*, r, c_in]
+        q = (self.linear_q(q) * D ** -0.5).view(q.shape[:-1] + (H, D))                  # [*, r, H, D]
+        k, v = self.linear_k(m), self.linear_v(m)                                        # [*, r, s, D]
+        a = torch.einsum("...hd,...sd->...hs", q, k) + (self.inf * (mask - 1))[..., :, None, :]
+        a = torch.softmax(a, dim=-1)
+        o = torch.einsum("...hs,...sd->...hd", a, v)                                     # [*, r, H, D]
+        g = torch.sigmoid(self.linear_g(m)).view(m.shape[:-1] + (H, D))                  # [*, r, s, H, D]
+        o = o.unsqueeze(-3) * g
+        return self.linear_o(o.reshape(o.shape[:-2] + (H * D,)))
+
+
+class MSAColumnGlobalAttention(nn.Module):
+    """LayerNorm + GlobalAttention along the sequence axis of every residue column (msa.py:361-392)."""
+
+    def __init__(self, c_in, c_hidden, no_heads, inf=1e9, eps=1e-10):
+        super().__init__()
+        self.layer_norm_m = nn.LayerNorm(c_in)
+        self.global_attention = GlobalAttention(c_in, c_hidden, no_heads, inf, eps)
+
+    def forward(self, m, mask=None, chunk_size=None):
+        if mask is None:
+            mask = m.new_ones(m.shape[:-1])
+        m = self.layer_norm_m(m.transpose(-2, -3))
+        return self.global_attention(m, mask.transpose(-1, -2)).transpose(-2, -3)
+
+
+class ExtraMSABlock(nn.Module):
+    """Evoformer block whose column attention is the global one (evoformer.py:354-389).  The
+    reference calls the core without ``_mask_trans``, i.e. with masked transitions; the argument
+    is exposed here so that a caller can also get the un-masked variant."""
+
+    def __init__(self, c_m, c_z, c_hidden_msa_att, c_hidden_opm, c_hidden_mul, c_hidden_pair_att,
+                 no_heads_msa, no_heads_pair, transition_n, msa_dropout, pair_dropout, inf, eps,
+                 ckpt=False, is_multimer=False):
+        super().__init__()
+        self.ckpt = ckpt
+        self.msa_att_row = MSARowAttentionWithPairBias(c_m, c_z, c_hidden_msa_att, no_heads_msa, inf=inf)
+        self.msa_att_col = MSAColumnGlobalAttention(c_m, c_hidden_msa_att, no_heads_msa, inf=inf, eps=eps)
+        self.core = EvoformerBlockCore(c_m, c_z, c_hidden_opm, c_hidden_mul, c_hidden_pair_att,
+                                       no_heads_msa, no_heads_pair, transition_n, pair_dropout, inf, eps)
+        self.is_multimer = is_multimer
+
+    def forward(self, m, z, msa_mask, pair_mask, chunk_size=None, _mask_trans=True):
+        m = m + self.msa_att_row(m, z=z, mask=msa_mask)
+        m = m + self.msa_att_col(m, mask=msa_mask)
+        return self.core(m, z, msa_mask=msa_mask, pair_mask=pair_mask, _mask_trans=_mask_trans)
+
+
+class ExtraMSAStack(nn.Module):
+    """no_blocks extra-MSA blocks; only the pair representation is returned (evoformer.py:587-633)."""
+
+    def __init__(self, c_m=64, c_z=128, c_hidden_msa_att=8, c_hidden_opm=32, c_hidden_mul=128,
+                 c_hidden_pair_att=32, no_heads_msa=8, no_heads_pair=4, no_blocks=4, transition_n=4,
+                 msa_dropout=0.15, pair_dropout=0.25, inf=1e9, eps=1e-10, ckpt=False,
+                 clear_cache_between_blocks=False, is_multimer=False, **kwargs):
+        super().__init__()
+        self.clear_cache_between_blocks = clear_cache_between_blocks
+        self.blocks = nn.ModuleList([
+            ExtraMSABlock(c_m, c_z, c_hidden_msa_att, c_hidden_opm, c_hidden_mul, c_hidden_pair_att,
+                          no_heads_msa, no_heads_pair, transition_n, msa_dropout, pair_dropout, inf, eps,
+                          ckpt, is_multimer)
+            for _ in range(no_blocks)])
+
+    def forward(self, m, z, chunk_size=None, msa_mask=None, pair_mask=None, _mask_trans=True):
+        for b in self.blocks:
+            m, z = b(m, z, msa_mask, pair_mask, chunk_size=chunk_size, _mask_trans=_mask_trans)
+        return z
+
+
 class OracleModel(nn.Module):
     """Minimal stand-in for the whole-model object the injection routine receives:
     it only has the ``evoformer`` attribute (reference call site: hub/alphafold.py:92-95)."""
 
-    def __init__(self, **stack_kwargs):
+    def __init__(self, extra_msa_kwargs=None, **stack_kwargs):
         super().__init__()
         self.evoformer = EvoformerStack(**stack_kwargs)
+        if extra_msa_kwargs is not None:
+            self.extra_msa_stack = ExtraMSAStack(**extra_msa_kwargs)

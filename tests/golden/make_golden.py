@@ -1,8 +1,9 @@
-"""Writes tests/golden/evoformer_nn_golden.npz by running the REFERENCE's own
-``fastfold.model.nn.evoformer.EvoformerStack`` (plain PyTorch, CPU, fp32) on seeded synthetic
-weights and inputs.  Run only in the build container, where /root/reference is mounted:
+"""Writes tests/golden/evoformer_nn_golden.npz and tests/golden/extra_msa_nn_golden.npz by running
+the REFERENCE's own ``fastfold.model.nn.evoformer.EvoformerStack`` / ``ExtraMSAStack`` (plain
+PyTorch, CPU, fp32) on seeded synthetic weights and inputs.  Run only in the build container, where /root/reference is mounted:
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            # Evoformer stack
+    python tests/golden/make_golden.py extra      # extra-MSA stack
 
 The fixture pins what closed forms cannot: the composition of a block (order of the
 sub-updates, residual placement, OPM reading the updated MSA), the q/k/v and left/right
@@ -20,7 +21,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, "/root/reference")
 
-from fastfold_amd.synthetic import synth_nn_state, synth_inputs  # noqa: E402
+from fastfold_amd.synthetic import synth_extra_nn_state, synth_nn_state, synth_inputs  # noqa: E402
 
 CASES = [
     # name, seed, no_blocks, n_seq, n_res, mask_tail_frac, fan_in_scaled
@@ -56,5 +57,40 @@ def main():
     print("wrote", os.path.join(HERE, "evoformer_nn_golden.npz"))
 
 
+EXTRA_CASES = [
+    # name, seed, no_blocks, n_extra, n_res, mask_tail_frac, fan_in_scaled
+    ("x1_s9_r12_pad", 21, 1, 9, 12, 0.17, True),
+    ("x2_s7_r10_full", 22, 2, 7, 10, 0.0, True),
+    ("x1_s40_r6_std002", 23, 1, 40, 6, 0.34, False),
+]
+
+
+def main_extra():
+    from fastfold.model.nn.evoformer import ExtraMSAStack  # the reference
+
+    out = {}
+    for name, seed, nb, s, r, tail, fis in EXTRA_CASES:
+        torch.manual_seed(0)
+        stack = ExtraMSAStack(c_m=64, c_z=128, c_hidden_msa_att=8, c_hidden_opm=32, c_hidden_mul=128,
+                              c_hidden_pair_att=32, no_heads_msa=8, no_heads_pair=4, no_blocks=nb,
+                              transition_n=4, msa_dropout=0.15, pair_dropout=0.25, inf=1e9, eps=1e-10,
+                              ckpt=False).eval()
+        sd = synth_extra_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=fis)
+        missing, unexpected = stack.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        assert not missing and not unexpected
+        m, z, msa_mask, pair_mask = synth_inputs(seed, s, r, c_m=64, mask_tail_frac=tail)
+        with torch.no_grad():
+            zo = stack(torch.from_numpy(m), torch.from_numpy(z), chunk_size=None,
+                       msa_mask=torch.from_numpy(msa_mask), pair_mask=torch.from_numpy(pair_mask))
+        out[name + ".z"] = zo.numpy()
+        out[name + ".cfg"] = np.array([seed, nb, s, r, int(round(tail * 100)), int(fis)], dtype=np.int64)
+        print(name, "z", float(np.abs(zo.numpy() - z).mean()))
+    np.savez_compressed(os.path.join(HERE, "extra_msa_nn_golden.npz"), **out)
+    print("wrote", os.path.join(HERE, "extra_msa_nn_golden.npz"))
+
+
 if __name__ == "__main__":
-    main()
+    if "extra" in sys.argv[1:]:
+        main_extra()
+    else:
+        main()

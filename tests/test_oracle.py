@@ -148,3 +148,88 @@ def test_ops_np_elementwise_closed_forms():
     xt = torch.from_numpy(np.log(yy)).requires_grad_(True)
     torch.softmax(xt, -1).backward(torch.from_numpy(dy))
     assert np.abs(ops_np.softmax_bwd(dy, yy) - xt.grad.numpy()).max() < 1e-10
+
+
+# ------------------------------------------------------------------ extra-MSA stack ----
+EXTRA_GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "extra_msa_nn_golden.npz")
+
+
+def _extra_stack(seed, nb, fis=True):
+    from fastfold_amd.synthetic import synth_extra_nn_state
+    from oracle.evoformer_ref import ExtraMSAStack
+    st = ExtraMSAStack(no_blocks=nb).eval()
+    sd = synth_extra_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=fis)
+    st.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+    return st
+
+
+def test_extra_msa_golden_vectors_from_reference():
+    g = np.load(EXTRA_GOLDEN)
+    names = sorted({k.split(".")[0] for k in g.files})
+    assert len(names) == 3
+    for name in names:
+        seed, nb, s, r, tail, fis = (int(v) for v in g[name + ".cfg"])
+        st = _extra_stack(seed, nb, bool(fis))
+        m, z, mm, pm = synth_inputs(seed, s, r, c_m=64, mask_tail_frac=tail / 100)
+        with torch.no_grad():
+            zo = st(torch.from_numpy(m), torch.from_numpy(z), msa_mask=torch.from_numpy(mm),
+                    pair_mask=torch.from_numpy(pm)).numpy()
+        ref = g[name + ".z"]
+        assert np.abs(zo - ref).max() <= 2e-5 * max(1.0, np.abs(ref).max()), name
+
+
+def test_global_attention_brute_force():
+    # float64 loops over the published formula (one query per column, shared key / value head)
+    from oracle.evoformer_ref import GlobalAttention
+    torch.manual_seed(3)
+    ga = GlobalAttention(12, 4, 3, inf=1e9, eps=1e-10).double()
+    with torch.no_grad():
+        for p in ga.parameters():
+            p.copy_(torch.randn_like(p) * 0.5)
+    rng = np.random.RandomState(4)
+    R, S = 3, 6
+    m = rng.standard_normal((R, S, 12))
+    mask = np.ones((R, S))
+    mask[1, 2:4] = 0
+    with torch.no_grad():
+        got = ga(torch.from_numpy(m), torch.from_numpy(mask)).numpy()
+    P = {k: v.detach().numpy() for k, v in ga.named_parameters()}
+    for j in range(R):
+        qa = sum(mask[j, s] * m[j, s] for s in range(S)) / (mask[j].sum() + 1e-10)
+        q = (P["linear_q.weight"] @ qa).reshape(3, 4) / 2.0
+        k = [P["linear_k.weight"] @ m[j, s] for s in range(S)]
+        v = [P["linear_v.weight"] @ m[j, s] for s in range(S)]
+        o = np.zeros((3, 4))
+        for h in range(3):
+            lg = np.array([q[h] @ k[s] if mask[j, s] else -np.inf for s in range(S)])
+            w = np.exp(lg - lg.max())
+            w /= w.sum()
+            o[h] = sum(w[s] * v[s] for s in range(S))
+        for s in range(S):
+            gate = 1.0 / (1.0 + np.exp(-(P["linear_g.weight"] @ m[j, s] + P["linear_g.bias"])))
+            out = P["linear_o.weight"] @ (gate * o.reshape(-1)) + P["linear_o.bias"]
+            assert np.abs(out - got[j, s]).max() < 1e-10
+
+
+def test_extra_msa_default_init_is_identity_and_masked_positions_do_not_leak():
+    from oracle.evoformer_ref import ExtraMSAStack
+    torch.manual_seed(0)
+    st = ExtraMSAStack(no_blocks=2).eval()
+    m, z, mm, pm = synth_inputs(8, 5, 7, c_m=64)
+    with torch.no_grad():
+        zo = st(torch.from_numpy(m), torch.from_numpy(z), msa_mask=torch.from_numpy(mm), pair_mask=torch.from_numpy(pm))
+    assert np.array_equal(zo.numpy(), z)
+    st = _extra_stack(9, 1)
+    m, z, mm, pm = synth_inputs(9, 6, 10, c_m=64, mask_tail_frac=0.3)
+    m2, z2 = m.copy(), z.copy()
+    m2[:, 7:] += 3.0
+    z2[7:, :] -= 2.0
+    z2[:, 7:] += 1.5
+    outs = []
+    for mt in (True, False):          # masked transitions only change masked positions
+        for mi, zi in ((m, z), (m2, z2)):
+            with torch.no_grad():
+                outs.append(st(torch.from_numpy(mi), torch.from_numpy(zi), msa_mask=torch.from_numpy(mm),
+                               pair_mask=torch.from_numpy(pm), _mask_trans=mt).numpy()[:7, :7])
+    for o in outs[1:]:
+        assert np.abs(o - outs[0]).max() < 1e-3
