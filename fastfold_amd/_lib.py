@@ -134,7 +134,7 @@ class Tile(ctypes.Structure):
         ("s_o", c_int64), ("s_i", c_int64), ("s_h", c_int64), ("s_d", c_int64),
         ("gate_ld", c_int64), ("m_so", c_int64), ("m_si", c_int64),
         ("inner", c_int), ("kind", c_int), ("act", c_int), ("ncols", c_int), ("glu", c_int),
-        ("scale", c_float),
+        ("scale", c_float), ("gate_rows", c_int), ("reserved", c_int),
     ]
 
 
@@ -157,7 +157,7 @@ SIGNATURES["ffk_fused_linear"] = [ctypes.POINTER(LinearDesc), _P]
 
 def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, gate_ld=0, rowmask=None,
               m_so=0, m_si=0, s_o=0, s_i=0, s_h=32, s_d=1, inner=1, act=FFK_ACT_NONE, ncols=128, glu=0,
-              scale=1.0):
+              scale=1.0, gate_rows=0):
     """Builds one epilogue descriptor; tensors may be passed directly (their data_ptr is taken)."""
     def p(t):
         return None if t is None else (t if isinstance(t, int) else t.data_ptr())
@@ -166,6 +166,7 @@ def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, g
     t.s_o, t.s_i, t.s_h, t.s_d = s_o, s_i, s_h, s_d
     t.gate_ld, t.m_so, t.m_si = gate_ld, m_so, m_si
     t.inner, t.kind, t.act, t.ncols, t.glu, t.scale = inner, kind, act, ncols, glu, scale
+    t.gate_rows = gate_rows
     return t
 
 
@@ -274,3 +275,13 @@ def transition_fused(out, x, gamma, beta, w1, b1, w2, b2, *, M, C, hidden, eps=1
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):
     call("ffk_key_bias", ptr(keybias), ptr(tileflags), ptr(mask), B, N, mask_sb, mask_sn,
          dtype_tag(mask.dtype) if mask is not None else FFK_F32, stream_ptr())
+
+
+SIGNATURES["ffk_global_attention_core"] = [_P, _P, _P, _P, _P, _F, _P, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L,
+                                           _F, _F, _I, _P]
+
+
+def global_attention_core(o, m, mask, gamma, beta, wq, wk, wv, *, S, R, C, H, D, m_ss, m_sr, mask_ss, mask_sr,
+                          scaling, eps, ln_eps=1e-5):
+    call("ffk_global_attention_core", ptr(o), ptr(m), ptr(mask), ptr(gamma), ptr(beta), ln_eps, ptr(wq), ptr(wk),
+         ptr(wv), S, R, C, H, D, m_ss, m_sr, mask_ss, mask_sr, scaling, eps, dtype_tag(m.dtype), stream_ptr())

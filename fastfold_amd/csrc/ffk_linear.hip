@@ -354,7 +354,7 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
                     x[j] = *reinterpret_cast<const Vec16<T>*>(sC + r * CP + c * ES);
                     long mr = m0 + r;
                     mr = mr < M ? mr : M - 1;
-                    if (gate) gv[j] = ld16(gate + mr * t.gate_ld + c);
+                    if (gate) gv[j] = ld16(gate + (t.gate_rows > 0 ? mr % t.gate_rows : mr) * t.gate_ld + c);
                     if (resid) rv[j] = ld16(resid + o[j]);
                 }
 #pragma unroll
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
                     } else {
                         oo = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
                     }
-                    if (gate) y = DT<T>::to_f(DT<T>::from_f(y * DT<T>::to_f(gate[(m0 + r) * t.gate_ld + c])));
+                    if (gate) y = DT<T>::to_f(DT<T>::from_f(y * DT<T>::to_f(gate[(t.gate_rows > 0 ? (m0 + r) % t.gate_rows : (m0 + r)) * t.gate_ld + c])));
                     if (resid) y += DT<T>::to_f(resid[oo]);
                     out[oo] = DT<T>::from_f(y);
                 }

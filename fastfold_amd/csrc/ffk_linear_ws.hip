@@ -596,6 +596,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (t.inner <= 0 || t.ncols <= 0 || !al16(t.out)) return false;
+    if (t.gate && t.gate_rows != 0) return false;      // periodic gate rows: generic kernel only
     if (ws_by_rows(t)) {
         if (t.kind == FFK_TILE_STRIDED) {
             if (t.ncols % 8 != 0 || t.s_o % 8 || t.s_i % 8 || t.s_h % 8) return false;

@@ -168,8 +168,10 @@ def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
 
 # ---------------------------------------------------------------------- attention ----
 def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_pk, out_bias_pk, c_out,
-              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None):
-    """Gated multi-head attention (head dim 32) over N tokens for each of B2 batch rows.
+              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None, head_dim=32):
+    """Gated multi-head attention over N tokens for each of B2 batch rows.  The kernels work on 32-wide
+    heads; a narrower head (``head_dim`` < 32) arrives zero-padded to 32 channels in ``w_pk`` / ``wo_pk``,
+    which changes neither the scores nor the used output channels - only the score scale is its own.
 
     x holds the C-channel rows addressed by ``a_map = (inner, s_o, s_i)``; w_pk is the packed
     [q; k; v; gate(; bias)] weight.  The attention update is projected by wo_pk and written as
@@ -194,7 +196,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     qk_kind = FFK_TILE_ACC if acc_order else FFK_TILE_QK
     gate = torch.empty((B2, H, NT, 1024) if acc_order else (M, HC), dtype=dt, device=dev)
     tpg = HC // 128
-    qscale = LOG2E / math.sqrt(32.0)
+    qscale = LOG2E / math.sqrt(float(head_dim))
     tkw = dict(inner=N, s_o=H * NT * 1024, s_h=NT * 1024)
     tiles = []
     for buf, kind, scale in ((q_t, qk_kind, qscale), (k_t, qk_kind, 1.0), (v_t, FFK_TILE_V, 1.0)):
@@ -376,4 +378,39 @@ def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, 
                       inner=32, s_o=r * 1024, s_i=32, s_h=1024, s_d=1, dtype=dt)
         _lib.bgemm_nt(O, wo, out.data_ptr() + i0 * r * Cz * es, M=n * r, N=Cz, K=1024, lda=1024, ldb=1024, bias=bo,
                       rowdiv=nrm.data_ptr() + i0 * r * 4, div_eps=eps, resid=z.data_ptr() + i0 * r * Cz * es, dtype=dt)
+    return out
+
+
+# --------------------------------------------------------------- global attention ----
+def global_attention(x, out, resid, *, S, R, C, H, D, x_ss, x_sr, out_ss, out_sr, ln, wq, wk, wv, wg_pk, gb_pk,
+                     wo_pk, ob_pk, c_out, mask, mask_ss, mask_sr, eps, budget):
+    """Global column attention (one mean query per column j, shared key / value head):
+    out[s, j] = (resid[s, j] +) Wo (sigmoid(Wg LN(x[s, j]) + bg) * o[j]) + bo, o from
+    ``ffk_global_attention_core``.  Row (s, j) of x is at ``s * x_ss + j * x_sr`` (elements), of out /
+    resid at ``s * out_ss + j * out_sr``; ``ln = None`` takes x as already normalised."""
+    dt, dev = x.dtype, x.device
+    es = es_of(dt)
+    HD = H * D
+    if not fits_fused(C, dt) or not fits_fused(HD, dt) or HD > 128 or c_out % vec_of(dt) != 0:
+        raise RuntimeError("global_attention: unsupported widths C=%d, H*D=%d, out=%d" % (C, HD, c_out))
+    o = torch.empty(R, HD, dtype=dt, device=dev)
+    _lib.global_attention_core(o, x, mask, None if ln is None else ln[0], None if ln is None else ln[1], wq, wk, wv,
+                               S=S, R=R, C=C, H=H, D=D, m_ss=x_ss, m_sr=x_sr, mask_ss=mask_ss, mask_sr=mask_sr,
+                               scaling=D ** -0.5, eps=eps)
+    # gate and output projection, a bounded number of sequences at a time
+    sc = max(1, min(S, budget // max(1, R * HD * es)))
+    tmp = torch.empty(sc * R, HD, dtype=dt, device=dev)
+    for s0 in range(0, S, sc):
+        n = min(sc, S - s0)
+        M = n * R
+        gate_tile = make_tile(tmp, bias=gb_pk, inner=M, s_i=HD, act=FFK_ACT_SIGMOID, ncols=HD, gate=o, gate_ld=HD,
+                              gate_rows=R)
+        _lib.fused_linear(x, wg_pk, [gate_tile], M=M, K=C, a_inner=R, a_so=x_ss, a_si=x_sr, ln=ln, a_off=s0 * x_ss)
+        tiles = []
+        for t in range((c_out + 127) // 128):
+            tiles.append(make_tile(out.data_ptr() + (s0 * out_ss + t * 128) * es,
+                                   bias=None if ob_pk is None else ob_pk.data_ptr() + t * 128 * es,
+                                   resid=None if resid is None else resid.data_ptr() + (s0 * out_ss + t * 128) * es,
+                                   inner=R, s_o=out_ss, s_i=out_sr, ncols=min(128, c_out - t * 128)))
+        _lib.fused_linear(tmp, wo_pk, tiles, M=M, K=HD)
     return out

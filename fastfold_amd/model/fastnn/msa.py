@@ -1,5 +1,6 @@
 """MSA stack of the Evoformer block: row attention with pair bias, column attention,
-transition - same classes and parameters as fastfold/model/fastnn/msa.py:33-151."""
+transition - same classes and parameters as fastfold/model/fastnn/msa.py:33-151 - and the
+extra-MSA core / block / stack (msa.py:154-464), whose column attention is the global one."""
 import math
 
 import torch
@@ -7,7 +8,13 @@ import torch.nn as nn
 
 from fastfold_amd.model.fastnn.kernel import LayerNorm
 from . import _fused as F_
-from .ops import SelfAttention, Transition, _PackMixin, _ln_pair, _mask_like, _no_grad_guard
+from typing import Optional, Tuple
+
+import torch.nn.functional as F
+
+from .ops import (ChunkMSAColumnGlobalAttention, ChunkTransition, OutProductMean, SelfAttention, Transition,
+                  _PackMixin, _ln_pair, _mask_like, _no_grad_guard)
+from .triangle import PairCore
 
 
 class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
@@ -52,12 +59,21 @@ class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
         mask = _mask_like(M_mask, M_raw)[0]
         F_.attention(M_raw, out, M_raw, B2=s, N=r, C=C, H=self.n_head, a_map=(s * r, 0, C),
                      ln=_ln_pair(self.layernormM, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
-                     c_out=C, mask=mask, mask_sb=r, mask_sn=1, bias_t=bias_t)
+                     c_out=C, mask=mask, mask_sb=r, mask_sn=1, bias_t=bias_t, head_dim=self.c)
         return out
 
     def forward(self, M_raw, Z, M_mask):
         M_raw = M_raw.contiguous()
         return self._run(M_raw, Z, M_mask, torch.empty_like(M_raw))
+
+
+class ChunkMSARowAttentionWithPairBias(MSARowAttentionWithPairBias):
+    """Same computation (ops.py:751-867); logits are never materialised, so there is nothing to chunk."""
+
+    def inplace(self, M_raw, Z, M_mask):
+        M_raw[0] = M_raw[0].contiguous()
+        self._run(M_raw[0], Z, M_mask, M_raw[0])
+        return M_raw
 
 
 class MSAColumnAttention(nn.Module, _PackMixin):
@@ -86,7 +102,7 @@ class MSAColumnAttention(nn.Module, _PackMixin):
         # logical row (j, s') reads m[s', j]
         F_.attention(M_raw, out, M_raw, B2=r, N=s, C=C, H=self.n_head, a_map=(s, C, r * C),
                      ln=_ln_pair(self.layernormM, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
-                     c_out=C, mask=mask, mask_sb=1, mask_sn=r)
+                     c_out=C, mask=mask, mask_sb=1, mask_sn=r, head_dim=self.c)
         return out
 
     def forward(self, M_raw, M_mask):
@@ -117,3 +133,139 @@ class MSACore(nn.Module):
         self.MSAColumnAttention._run(node, node_mask, node)
         self.MSATransition._run(node, node)
         return node
+
+
+class ExtraMSACore(nn.Module):
+    """Row attention with pair bias (head dim 8), global column attention, transition (msa.py:154-187)."""
+
+    def __init__(self, d_node, d_pair, p_drop=0.15):
+        super(ExtraMSACore, self).__init__()
+        self.MSARowAttentionWithPairBias = ChunkMSARowAttentionWithPairBias(d_node=d_node, d_pair=d_pair,
+                                                                            p_drop=p_drop, c=8)
+        self.MSAColumnAttention = ChunkMSAColumnGlobalAttention(d_node=d_node, c=8)
+        self.MSATransition = ChunkTransition(d=d_node)
+
+    def forward(self, node, pair, node_mask):
+        node = node.contiguous()
+        out = torch.empty_like(node)
+        self.MSARowAttentionWithPairBias._run(node, pair, node_mask, out)
+        self.MSAColumnAttention._run(out, node_mask, out)
+        self.MSATransition._run(out, out)
+        return out
+
+    def inplace(self, node, pair, node_mask):
+        """``node`` is a one-element list; ``pair`` a tensor (msa.py:176-187)."""
+        node[0] = node[0].contiguous()
+        self.MSARowAttentionWithPairBias._run(node[0], pair, node_mask, node[0])
+        self.MSAColumnAttention._run(node[0], node_mask, node[0])
+        self.MSATransition._run(node[0], node[0])
+        return node
+
+
+class ExtraMSABlock(nn.Module):
+    """One block of the extra-MSA stack (msa.py:190-345).  As for ``Evoformer``, the reference's padding
+    by one sequence and one residue between blocks is kept as an interface (shapes in and out) while the
+    computation runs on the un-padded region, whose results cannot depend on the masked padding."""
+
+    def __init__(self, c_m: int, c_z: int, first_block: bool, last_block: bool, is_multimer=False):
+        super(ExtraMSABlock, self).__init__()
+        self.first_block = first_block
+        self.last_block = last_block
+        self.msa_stack = ExtraMSACore(c_m, c_z, p_drop=0.15)
+        self.communication = OutProductMean(n_feat=c_m, n_feat_out=c_z, n_feat_proj=32)
+        self.pair_stack = PairCore(d_pair=c_z)
+        self.is_multimer = is_multimer
+
+    def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
+        """m [1, s, r, c_m], z [1, r, r, c_z] contiguous, masks [1, s, r] / [1, r, r]."""
+        if self.is_multimer:
+            # msa.py:264-270: outer product mean and pair stack first, MSA stack on the z in between
+            z_new = z if inplace else torch.empty_like(z)
+            self.communication._run(m, msa_mask, z, z_new)
+            z_ori = z_new.clone()
+            self.pair_stack.inplace([z_new], pair_mask)
+            m = self.msa_stack.inplace([m], z_ori, msa_mask)[0] if inplace else self.msa_stack.forward(m, z_ori, msa_mask)
+            return m, z_new
+        if inplace:
+            m = self.msa_stack.inplace([m], z, msa_mask)[0]
+            self.communication._run(m, msa_mask, z, z)
+            self.pair_stack.inplace([z], pair_mask)
+            return m, z
+        m = self.msa_stack.forward(m, z, msa_mask)
+        z = self.communication.forward(m, msa_mask, z)
+        self.pair_stack.inplace([z], pair_mask)
+        return m, z
+
+    def _enter(self, m, z, s, r):
+        if self.first_block:
+            return m.unsqueeze(0).contiguous(), z.unsqueeze(0).contiguous()
+        if m.dim() != 4 or z.dim() != 4 or m.shape[1] != s + 1 or m.shape[2] != r + 1 or z.shape[1] != r + 1:
+            raise RuntimeError("ExtraMSABlock: a non-first block expects padded [1, s+1, r+1, c] / [1, r+1, r+1, c] "
+                               "inputs, got %s / %s" % (tuple(m.shape), tuple(z.shape)))
+        return m[:, :s, :r, :].contiguous(), z[:, :r, :r, :].contiguous()
+
+    def _leave(self, m, z):
+        if self.last_block:
+            return m.squeeze(0), z.squeeze(0)
+        return F.pad(m, (0, 0, 0, 1, 0, 1)), F.pad(z, (0, 0, 0, 1, 0, 1))
+
+    def forward(self, m: torch.Tensor, z: torch.Tensor, msa_mask: torch.Tensor, pair_mask: torch.Tensor,
+                chunk_size: Optional[int] = None, _mask_trans: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+        s, r = msa_mask.size(-2), pair_mask.size(-1)
+        m, z = self._enter(m, z, s, r)
+        m, z = self._core(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0), inplace=not self.first_block)
+        return self._leave(m, z)
+
+    def inplace(self, m, z, msa_mask: torch.Tensor, pair_mask: torch.Tensor, chunk_size: Optional[int] = None,
+                _mask_trans: bool = True):
+        s, r = msa_mask.size(-2), pair_mask.size(-1)
+        mm, zz = self._enter(m[0], z[0], s, r)
+        mm, zz = self._core(mm, zz, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0), inplace=True)
+        m[0], z[0] = self._leave(mm, zz)
+        return m, z
+
+
+class ExtraMSAStack(nn.Module):
+    """Algorithm 18 (msa.py:347-464): ``no_blocks`` extra-MSA blocks; returns the pair representation."""
+
+    def __init__(self, c_m: int, c_z: int, no_blocks: int, clear_cache_between_blocks: bool = False,
+                 is_multimer: bool = False, **kwargs):
+        super(ExtraMSAStack, self).__init__()
+        self.clear_cache_between_blocks = clear_cache_between_blocks
+        self.blocks = nn.ModuleList()
+        for block_id in range(no_blocks):
+            self.blocks.append(ExtraMSABlock(c_m=c_m, c_z=c_z, first_block=(block_id == 0),
+                                             last_block=(block_id == no_blocks - 1), is_multimer=is_multimer))
+
+    def _run(self, m, z, msa_mask, pair_mask, inplace_first: bool):
+        mm, zz = m.unsqueeze(0).contiguous(), z.unsqueeze(0).contiguous()
+        mk, pk = msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)
+        with F_.mask_cache():
+            for i, b in enumerate(self.blocks):
+                mm, zz = b._core(mm, zz, mk, pk, inplace=(inplace_first or i > 0))
+                if self.clear_cache_between_blocks:
+                    torch.cuda.empty_cache()
+        return zz.squeeze(0)
+
+    def forward(self, m: torch.Tensor, z: torch.Tensor, chunk_size: int, msa_mask: Optional[torch.Tensor] = None,
+                pair_mask: Optional[torch.Tensor] = None, _mask_trans: bool = True) -> torch.Tensor:
+        """m [N_extra, N_res, C_m], z [N_res, N_res, C_z], msa_mask [N_extra, N_res], pair_mask
+        [N_res, N_res] -> z.  Inputs are left untouched."""
+        msa_mask, pair_mask = self._masks(m, z, msa_mask, pair_mask)
+        return self._run(m, z, msa_mask, pair_mask, inplace_first=False)
+
+    def inplace(self, m, z, chunk_size: int, msa_mask: Optional[torch.Tensor] = None,
+                pair_mask: Optional[torch.Tensor] = None, _mask_trans: bool = True):
+        """``m`` / ``z`` are one-element lists; returns the list ``z`` as the reference does (msa.py:433-464)."""
+        msa_mask, pair_mask = self._masks(m[0], z[0], msa_mask, pair_mask)
+        contiguous = m[0].is_contiguous() and z[0].is_contiguous()
+        z[0] = self._run(m[0], z[0], msa_mask, pair_mask, inplace_first=contiguous)
+        return z
+
+    @staticmethod
+    def _masks(m, z, msa_mask, pair_mask):
+        if msa_mask is None:
+            msa_mask = m.new_ones(m.shape[:-1])
+        if pair_mask is None:
+            pair_mask = z.new_ones(z.shape[:-1])
+        return msa_mask, pair_mask

@@ -218,9 +218,19 @@ class OutProductMean(nn.Module, _PackMixin):
         return Z_raw
 
 
+def _pad_heads(w, n_head, c, dim):
+    """Index h * c + d along ``dim`` -> h * 32 + d, new entries zero (a head narrower than the kernels'
+    32 channels contributes nothing through its padding: zero q / k / v channels and zero o_linear columns)."""
+    if c == 32:
+        return w
+    w = w.detach().unflatten(dim, (n_head, c))
+    pad = [0, 0] * (w.dim() - dim - 2) + [0, 32 - c]
+    return torch.nn.functional.pad(w, pad).flatten(dim, dim + 1)
+
+
 class SelfAttention(nn.Module, _PackMixin):
     """Multi-head self attention over [batch_size1, batch_size2, len, dim] tensors with gating
-    (ops.py:259-363).  Head dimension ``c`` must be 32 and ``n_head`` a multiple of 4."""
+    (ops.py:259-363).  Head dimension ``c`` at most 32 and ``n_head`` a multiple of 4."""
 
     def __init__(self, qkv_dim, c, n_head, out_dim, gating=True, last_bias_fuse=False):
         super(SelfAttention, self).__init__()
@@ -238,8 +248,8 @@ class SelfAttention(nn.Module, _PackMixin):
         self.o_linear = Linear(n_head * c, out_dim, initializer='zero', use_bias=(not last_bias_fuse))
 
     def _check(self, dtype):
-        if self.c != 32 or not self.gating:
-            raise RuntimeError("SelfAttention: the kernel path needs head dim 32 and gating=True")
+        if self.c > 32 or self.n_head % 4 != 0 or not self.gating:
+            raise RuntimeError("SelfAttention: the kernel path needs head dim <= 32, n_head % 4 == 0 and gating=True")
         if not F_.fits_fused(self.qkv_dim, dtype):
             raise RuntimeError("SelfAttention: unsupported input width %d" % self.qkv_dim)
 
@@ -250,11 +260,14 @@ class SelfAttention(nn.Module, _PackMixin):
         params += list(extra_params)
 
         def build():
-            mats = [self.to_qkv.weight, self.gating_linear.weight]
+            H, c = self.n_head, self.c
+            mats = [_pad_heads(self.to_qkv.weight.detach().unflatten(0, (3, H * c)), H, c, 1).flatten(0, 1),
+                    _pad_heads(self.gating_linear.weight, H, c, 0)]
             w = F_.pack_rows(mats, dtype, device)
             if extra_rows is not None:
                 w = torch.cat([w, F_.pack_rows([extra_rows()], dtype, device)], 0).contiguous()
-            return (w, F_.pack_vec([self.gating_bias], dtype, device), F_.pack_rows([self.o_linear.weight], dtype, device))
+            return (w, F_.pack_vec([_pad_heads(self.gating_bias, H, c, 0)], dtype, device),
+                    F_.pack_rows([_pad_heads(self.o_linear.weight, H, c, 1)], dtype, device))
         return self._packed(key, params, build)
 
     def forward(self, in_data, mask, nonbatched_bias=None):
@@ -289,8 +302,95 @@ class SelfAttention(nn.Module, _PackMixin):
         out = torch.empty(1, B2, N, self.out_dim, dtype=dt, device=dev)
         F_.attention(x, out, None, B2=B2, N=N, C=C, H=self.n_head, a_map=(B2 * N, 0, C), ln=None, w_pk=w_pk,
                      gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob, c_out=self.out_dim, mask=mk, mask_sb=sb,
-                     mask_sn=sn, bias_t=bias_t)
+                     mask_sn=sn, bias_t=bias_t, head_dim=self.c)
         return out
+
+
+class GlobalAttention(nn.Module, _PackMixin):
+    """Global attention over [batch_size1, batch_size2, len, dim] tensors (ops.py:1148-1236): one query
+    per (batch_size1, batch_size2) entry - the masked mean over ``len`` - and a single key / value head."""
+
+    def __init__(self, qkv_dim, c, n_head, out_dim):
+        super(GlobalAttention, self).__init__()
+        self.qkv_dim = qkv_dim
+        self.c = c
+        self.n_head = n_head
+        self.out_dim = out_dim
+        self.scaling = self.c ** (-0.5)
+        self.eps = 1e-10
+        self.inf = 1e9
+        self.to_q = Linear(qkv_dim, c * self.n_head, use_bias=False)
+        self.to_kv = Linear(qkv_dim, 2 * c, initializer="linear", use_bias=False)
+        self.gating_bias = nn.parameter.Parameter(data=torch.ones((n_head * c,)))
+        self.gating_linear = Linear(qkv_dim, n_head * c, initializer="zero", use_bias=False)
+        self.o_linear = Linear(n_head * c, out_dim, initializer="zero")
+
+    def _pk(self, dt, dev):
+        ps = [self.to_q.weight, self.to_kv.weight, self.gating_linear.weight, self.gating_bias,
+              self.o_linear.weight, self.o_linear.bias]
+        return self._packed(("ga", dt, dev), ps, lambda: (
+            self.to_q.weight.detach().to(dt).contiguous(),
+            self.to_kv.weight.detach()[:self.c].to(dt).contiguous(),
+            self.to_kv.weight.detach()[self.c:].to(dt).contiguous(),
+            F_.pack_rows([self.gating_linear.weight], dt, dev), F_.pack_vec([self.gating_bias], dt, dev),
+            F_.pack_rows([self.o_linear.weight], dt, dev), F_.pack_vec([self.o_linear.bias], dt, dev)))
+
+    def _run(self, x, out, resid, *, S, R, x_ss, x_sr, out_ss, out_sr, ln, mask, mask_ss, mask_sr):
+        """Rows (s, j), s < S along the attended axis, j < R columns; see ``_fused.global_attention``."""
+        dt, dev = x.dtype, x.device
+        wq, wk, wv, wg, gb, wo, ob = self._pk(dt, dev)
+        return F_.global_attention(x, out, resid, S=S, R=R, C=self.qkv_dim, H=self.n_head, D=self.c, x_ss=x_ss,
+                                   x_sr=x_sr, out_ss=out_ss, out_sr=out_sr, ln=ln, wq=wq, wk=wk, wv=wv, wg_pk=wg,
+                                   gb_pk=gb, wo_pk=wo, ob_pk=ob, c_out=self.out_dim, mask=mask, mask_ss=mask_ss,
+                                   mask_sr=mask_sr, eps=self.eps, budget=_budget())
+
+    def forward(self, m, mask):
+        """m [1, batch_size2, len, qkv_dim] (already normalised), mask [1, batch_size2, len] ->
+        [1, batch_size2, len, out_dim]."""
+        F_.check_cuda(m, mask)
+        _no_grad_guard(self, m)
+        if m.dim() != 4 or m.shape[0] != 1 or m.shape[-1] != self.qkv_dim:
+            raise RuntimeError("GlobalAttention: expected [1, B2, N, %d] input, got %s" % (self.qkv_dim, tuple(m.shape)))
+        _, R, S, C = m.shape
+        if m.stride(-1) != 1 or m.stride(1) % 8 or m.stride(2) % 8:
+            m = m.contiguous()
+        mk = mask.to(m.dtype)[0]
+        out = torch.empty(1, R, S, self.out_dim, dtype=m.dtype, device=m.device)
+        self._run(m, out, None, S=S, R=R, x_ss=m.stride(2), x_sr=m.stride(1), out_ss=self.out_dim,
+                  out_sr=S * self.out_dim, ln=None, mask=mk, mask_ss=mk.stride(1), mask_sr=mk.stride(0))
+        return out
+
+
+class ChunkMSAColumnGlobalAttention(nn.Module):
+    """M_raw + GlobalAttention(LayerNorm(M_raw) along the sequence axis) (ops.py:992-1043)."""
+
+    def __init__(self, d_node, c=8, n_head=8):
+        super(ChunkMSAColumnGlobalAttention, self).__init__()
+        self.d_node = d_node
+        self.c = c
+        self.n_head = n_head
+        self.layernormM = LayerNorm(d_node)
+        self.global_attention = GlobalAttention(qkv_dim=d_node, c=c, n_head=n_head, out_dim=d_node)
+
+    def _run(self, M_raw, M_mask, out):
+        F_.check_cuda(M_raw, M_mask)
+        _no_grad_guard(self, M_raw)
+        if M_raw.dim() != 4 or M_raw.shape[0] != 1:
+            raise RuntimeError("ChunkMSAColumnGlobalAttention: expected [1, s, r, C], got %s" % (tuple(M_raw.shape),))
+        _, s, r, C = M_raw.shape
+        mask = _mask_like(M_mask, M_raw)[0]               # [s, r]
+        self.global_attention._run(M_raw, out, M_raw, S=s, R=r, x_ss=r * C, x_sr=C, out_ss=r * C, out_sr=C,
+                                   ln=_ln_pair(self.layernormM, M_raw.dtype), mask=mask, mask_ss=r, mask_sr=1)
+        return out
+
+    def forward(self, M_raw, M_mask):
+        M_raw = M_raw.contiguous()
+        return self._run(M_raw, M_mask, torch.empty_like(M_raw))
+
+    def inplace(self, M_raw, M_mask):
+        M_raw[0] = M_raw[0].contiguous()
+        self._run(M_raw[0], M_mask, M_raw[0])
+        return M_raw
 
 
 def permute_final_dims(tensor, inds):
@@ -423,3 +523,12 @@ class ChunkTriangleAttentionStartingNode(_TriangleAttention):
 class ChunkTriangleAttentionEndingNode(_TriangleAttention):
     """Algorithm 14 (ops.py:869-989): attention along each column."""
     _ending = True
+
+
+def __getattr__(name):
+    # the reference keeps the chunked row attention in this module (ops.py:751-867); here it lives
+    # beside the un-chunked one, which this module cannot import at load time
+    if name == "ChunkMSARowAttentionWithPairBias":
+        from .msa import ChunkMSARowAttentionWithPairBias
+        return ChunkMSARowAttentionWithPairBias
+    raise AttributeError("module %r has no attribute %r" % (__name__, name))

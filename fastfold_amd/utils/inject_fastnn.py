@@ -12,11 +12,13 @@ path (``inject_fastnn``, ``inject_evoformer``, ``copy_*``; reference lines 24-15
   tri-mul a_p|b_p, a_g|b_g -> ``left_right_projection`` / ``left_right_gate`` (left rows first),
   linear_g -> ``output_gate``, linear_z.{weight,bias} -> ``output_projection.weight`` / ``output_bias``
   OPM linear_1/2/out       -> ``linear_a`` / ``linear_b`` / ``o_linear``
-Extra-MSA, template and embedder stages are outside this build and are left as they are.
+The extra-MSA stack (``inject_extramsa``, reference lines 154-236,341-355) follows the same re-layout,
+with the global column attention's linear_q -> ``to_q``, linear_k | linear_v -> rows of ``to_kv``.
+Template and embedder stages are outside this build and are left as they are.
 """
 import torch
 
-from fastfold_amd.model.fastnn import EvoformerStack
+from fastfold_amd.model.fastnn import EvoformerStack, ExtraMSAStack
 
 
 def copy_layernorm(model_fast, model_ori):
@@ -40,6 +42,18 @@ def copy_attention(model_fast, model_ori):
     copy_linear(model_fast.o_linear, model_ori.linear_o)
     if getattr(model_fast, "gating_bias", None) is not None and model_ori.linear_g is not None:
         model_fast.gating_bias.copy_(model_ori.linear_g.bias)
+
+
+def copy_kv_linear(model_fast, ori_k, ori_v):
+    model_fast.weight.copy_(torch.cat((ori_k.weight, ori_v.weight), dim=0))
+
+
+def copy_global_attention(model_fast, model_ori):
+    copy_linear(model_fast.to_q, model_ori.linear_q)
+    copy_kv_linear(model_fast.to_kv, model_ori.linear_k, model_ori.linear_v)
+    copy_linear(model_fast.gating_linear, model_ori.linear_g)
+    copy_linear(model_fast.o_linear, model_ori.linear_o)
+    model_fast.gating_bias.copy_(model_ori.linear_g.bias)
 
 
 def copy_left_right(model_fast, ori_left, ori_right):
@@ -97,6 +111,53 @@ def copy_evoformer_para(block_fast, block_ori):
     copy_transition(block_fast.pair.PairTransition, block_ori.core.pair_transition)
 
 
+def copy_extra_msa_para(block_fast, block_ori):
+    row_f, row_o = block_fast.msa_stack.MSARowAttentionWithPairBias, block_ori.msa_att_row
+    copy_layernorm(row_f.layernormM, row_o.layer_norm_m)
+    copy_layernorm(row_f.layernormZ, row_o.layer_norm_z)
+    copy_attention(row_f.attention, row_o.mha)
+    row_f.linear_b_weights.copy_(row_o.linear_z.weight)
+    row_f.out_bias.copy_(row_o.mha.linear_o.bias)
+
+    col_f, col_o = block_fast.msa_stack.MSAColumnAttention, block_ori.msa_att_col
+    copy_layernorm(col_f.layernormM, col_o.layer_norm_m)
+    copy_global_attention(col_f.global_attention, col_o.global_attention)
+
+    copy_transition(block_fast.msa_stack.MSATransition, block_ori.core.msa_transition)
+
+    opm_f, opm_o = block_fast.communication, block_ori.core.outer_product_mean
+    copy_layernorm(opm_f.layernormM, opm_o.layer_norm)
+    copy_linear(opm_f.linear_a, opm_o.linear_1)
+    copy_linear(opm_f.linear_b, opm_o.linear_2)
+    copy_linear(opm_f.o_linear, opm_o.linear_out)
+
+    copy_triangle(block_fast.pair_stack.TriangleMultiplicationOutgoing, block_ori.core.tri_mul_out)
+    copy_triangle(block_fast.pair_stack.TriangleMultiplicationIncoming, block_ori.core.tri_mul_in)
+    copy_triangle_att(block_fast.pair_stack.TriangleAttentionStartingNode, block_ori.core.tri_att_start)
+    copy_triangle_att(block_fast.pair_stack.TriangleAttentionEndingNode, block_ori.core.tri_att_end)
+    copy_transition(block_fast.pair_stack.PairTransition, block_ori.core.pair_transition)
+
+
+def inject_extramsa(model):
+    with torch.no_grad():
+        target_module = model.extra_msa_stack
+        ref_param = next(target_module.parameters())
+        fast_module = ExtraMSAStack(
+            c_m=target_module.blocks[0].msa_att_row.c_in,
+            c_z=target_module.blocks[0].msa_att_row.c_z,
+            no_blocks=len(target_module.blocks),
+            clear_cache_between_blocks=target_module.clear_cache_between_blocks,
+            is_multimer=target_module.blocks[0].is_multimer,
+        ).to(device=ref_param.device, dtype=ref_param.dtype)
+        for target_block, fast_block in zip(target_module.blocks, fast_module.blocks):
+            copy_extra_msa_para(fast_block, target_block)
+            if target_block.training is False:
+                fast_block.eval()
+        if target_module.training is False:
+            fast_module.eval()
+        model.extra_msa_stack = fast_module
+
+
 def inject_evoformer(model):
     with torch.no_grad():
         target_module = model.evoformer
@@ -121,8 +182,11 @@ def inject_evoformer(model):
 
 
 def inject_fastnn(model):
-    """Replaces ``model.evoformer``; returns the model (reference: inject_fastnn.py:418-423)."""
+    """Replaces ``model.evoformer`` and, where the model has one, ``model.extra_msa_stack``; returns the
+    model (reference: inject_fastnn.py:418-423)."""
     inject_evoformer(model)
+    if getattr(model, "extra_msa_stack", None) is not None:
+        inject_extramsa(model)
     return model
 
 

@@ -143,7 +143,9 @@ typedef struct ffk_tile {
     void* out;
     const void* bias;      /* 128 values of the activation dtype (packed tile order) or NULL */
     const void* resid;     /* same addressing as out (may alias out) or NULL; STRIDED with s_d == 1 only */
-    const void* gate;      /* [M, gate_ld] in logical row order, or NULL; STRIDED with s_d == 1 only */
+    const void* gate;      /* [M, gate_ld] in logical row order (gate_rows == 0) or [gate_rows, gate_ld] read at
+                              row m % gate_rows (one multiplier row shared by every gate_rows-th logical row),
+                              or NULL; STRIDED with s_d == 1 only */
     const void* rowmask;   /* 0/1 per logical row at (m / inner) * m_so + (m % inner) * m_si, or NULL */
     int64_t s_o, s_i, s_h, s_d;
     int64_t gate_ld;
@@ -154,6 +156,8 @@ typedef struct ffk_tile {
     int32_t ncols;         /* valid output channels of this tile (<= 128, <= 64 with glu) */
     int32_t glu;
     float scale;
+    int32_t gate_rows;     /* 0, or the period of the gate's row index (see gate) */
+    int32_t reserved;
 } ffk_tile;
 
 typedef struct ffk_linear_desc {
@@ -279,6 +283,25 @@ int ffk_opm_fused(void* out, const void* resid, const void* a_t, const void* b_t
 int ffk_transition_fused(void* out, const void* x, const void* gamma, const void* beta, const void* w1,
                          const void* b1, const void* w2, const void* b2, int64_t M, int64_t C,
                          int64_t hidden, float eps, int dtype, void* stream);
+
+/* Global column attention core of the extra-MSA stack: one query per residue column (the masked mean
+ * of the normalised rows), one key / value head of width D shared by the H query heads.
+ *     x_s = LayerNorm(m[s, j, :]; gamma, beta, ln_eps)
+ *     q[h] = scaling * Wq[h] (sum_s mask[s, j] x_s / (sum_s mask[s, j] + eps))
+ *     o[j, h*D + d] = sum_s softmax_s(q[h] . Wk x_s, masked s replaced by -1e9) (Wv x_s)[d]
+ * Row (s, j) of m lives at  m + s * m_ss + j * m_sr  (elements; its C channels, C in {32, 64, 128},
+ * contiguous), mask[s, j] (activation dtype, 0 / 1; NULL = all ones) at  mask + s * mask_ss + j * mask_sr.
+ * ln_gamma == NULL: the rows are taken as already normalised.
+ * wq : [H*D, C]; wk, wv : [D, C]; o : [R, H*D]; H <= 8, H*D <= 128.  fp32 or bf16; the sums run in
+ * fp32.  A column whose rows are all masked gets the plain mean of v (the softmax of equal logits),
+ * as in the reference.
+ * Replaces: LayerNorm + the q / k / v / softmax / weighted-average part of GlobalAttention.forward
+ * (fastfold/model/fastnn/ops.py:1006-1009,1179-1195; nn/primitives.py:452-486). */
+int ffk_global_attention_core(void* o, const void* m, const void* mask, const void* ln_gamma,
+                              const void* ln_beta, float ln_eps, const void* wq, const void* wk,
+                              const void* wv, int64_t S, int64_t R, int64_t C, int64_t H, int64_t D,
+                              int64_t m_ss, int64_t m_sr, int64_t mask_ss, int64_t mask_sr,
+                              float scaling, float eps, int dtype, void* stream);
 
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the

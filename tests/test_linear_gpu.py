@@ -435,3 +435,27 @@ def test_fused_linear_second_operand(dev, r):
     # a second operand without the shapes it is built for is refused, not ignored
     with pytest.raises(RuntimeError):
         _lib.fused_linear(z, w_pk, tiles, M=M, K=C, ln=(gam2, bet2), a2=z, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("K,N,P", [(64, 64, 37), (128, 128, 16)])
+def test_periodic_gate_rows(dev, dtype, K, N, P):
+    """gate_rows = P: logical row m is multiplied by gate row m % P (one multiplier row per column of an
+    [S, P] grid of rows, as the global column attention uses it)."""
+    from fastfold_amd import _lib
+    S = 9
+    M = S * P
+    g = torch.Generator().manual_seed(K + P)
+    a = torch.randn(M, K, generator=g).to(dev, dtype)
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).to(dev, dtype)
+    b = torch.randn(N, generator=g).to(dev, dtype)
+    gate = torch.randn(P, N, generator=g).to(dev, dtype)
+    out = torch.empty(M, N, dtype=dtype, device=dev)
+    bp = torch.zeros(128, dtype=dtype, device=dev)
+    bp[:N] = b
+    tiles = [_lib.make_tile(out, bias=bp, gate=gate, gate_ld=N, gate_rows=P, inner=M, s_i=N, ncols=N,
+                            act=_lib.FFK_ACT_SIGMOID)]
+    _lib.fused_linear(a, _pack(w, 1), tiles, M=M, K=K)
+    y = 1.0 / (1.0 + np.exp(-ops_np.linear(_np(a), _np(w), _np(b))))
+    ref = y.reshape(S, P, N) * _np(gate)[None]
+    assert _rel(_np(out).reshape(S, P, N), ref) < TOL[dtype]
