@@ -2,16 +2,14 @@
 transition - same classes and parameters as fastfold/model/fastnn/msa.py:33-151 - and the
 extra-MSA core / block / stack (msa.py:154-464), whose column attention is the global one."""
 import math
+from typing import Optional, Tuple
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from fastfold_amd.model.fastnn.kernel import LayerNorm
 from . import _fused as F_
-from typing import Optional, Tuple
-
-import torch.nn.functional as F
-
 from .ops import (ChunkMSAColumnGlobalAttention, ChunkTransition, OutProductMean, SelfAttention, Transition,
                   _PackMixin, _ln_pair, _mask_like, _no_grad_guard)
 from .triangle import PairCore

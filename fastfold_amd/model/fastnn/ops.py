@@ -502,7 +502,8 @@ class _TriangleAttention(nn.Module, _PackMixin):
             a_map, sb, sn = (r * r, 0, C), r, 1
         F_.attention(Z_raw, out, Z_raw, B2=r, N=r, C=C, H=self.n_head, a_map=a_map,
                      ln=_ln_pair(self.layernorm1, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
-                     c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=bias_t, bias_in_launch=True, pb_scratch=pbs)
+                     c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=bias_t, bias_in_launch=True, pb_scratch=pbs,
+                     head_dim=self.c)
         return out
 
     def forward(self, Z_raw, Z_mask):

@@ -121,6 +121,40 @@ def synth_extra_nn_state(seed=0, no_blocks=1, std=0.02, fan_in_scaled=False, **d
     return sd
 
 
+def template_nn_layout_block_shapes(c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_heads=4, pair_transition_n=2):
+    """One ``TemplatePairStackBlock`` in draw order: tri_att_start, tri_att_end (layer_norm, linear.weight,
+    mha.linear_{q,k,v}.weight, mha.linear_o, mha.linear_g), tri_mul_out, tri_mul_in (layer_norm_in, linear_a_p,
+    linear_a_g, linear_b_p, linear_b_g, linear_g, linear_z, layer_norm_out), pair_transition."""
+    base = nn_layout_block_shapes(c_m=c_t, c_z=c_t, c_hidden_mul=c_hidden_tri_mul, c_hidden_pair_att=c_hidden_tri_att,
+                                  no_heads_pair=no_heads, transition_n=pair_transition_n)
+    out = []
+    for prefix in ("core.tri_att_start.", "core.tri_att_end.", "core.tri_mul_out.", "core.tri_mul_in.",
+                   "core.pair_transition."):
+        out += [(n[len("core."):], sh, k) for n, sh, k in base if n.startswith(prefix)]
+    return out
+
+
+def synth_template_nn_state(seed=0, no_blocks=2, std=0.02, fan_in_scaled=False, c_t=64, **dims):
+    """nn-layout state of a ``TemplatePairStack`` (blocks, then ``layer_norm``), drawn like ``synth_nn_state``."""
+    rng = np.random.RandomState(seed)
+    sd = OrderedDict()
+
+    def draw(shape, kind):
+        x = rng.standard_normal(shape).astype(np.float32)
+        if kind == "ln_w":
+            return (1.0 + std * x).astype(np.float32)
+        if kind == "w" and fan_in_scaled:
+            return (x / np.sqrt(shape[1])).astype(np.float32)
+        return (std * x).astype(np.float32)
+
+    for i in range(no_blocks):
+        for name, shape, kind in template_nn_layout_block_shapes(c_t=c_t, **dims):
+            sd["blocks.%d.%s" % (i, name)] = draw(shape, kind)
+    sd["layer_norm.weight"] = draw((c_t,), "ln_w")
+    sd["layer_norm.bias"] = draw((c_t,), "ln_b")
+    return sd
+
+
 def synth_nn_state(seed=0, no_blocks=1, std=0.02, c_m=256, c_z=128, c_s=384, fan_in_scaled=False, **dims):
     """OrderedDict name -> float32 numpy array, nn layout, for an ``EvoformerStack``.
 
@@ -161,3 +195,10 @@ def synth_inputs(seed, n_seq, n_res, c_m=256, c_z=128, mask_tail_frac=0.0):
     msa_mask = np.ones((n_seq, 1), np.float32) * seq_mask[None, :]
     pair_mask = seq_mask[:, None] * seq_mask[None, :]
     return m, z, msa_mask, pair_mask
+
+
+def synth_template_inputs(seed, n_templ, n_res, c_t=64, mask_tail_frac=0.0):
+    """t [n_templ, r, r, c_t] ~ N(0,1) fp32 and the pair mask [r, r] shared by the templates."""
+    t = synth_inputs(seed, n_templ, n_res * n_res, c_m=c_t, c_z=1)[0].reshape(n_templ, n_res, n_res, c_t)
+    pair_mask = synth_inputs(seed, 1, n_res, c_m=1, c_z=1, mask_tail_frac=mask_tail_frac)[3]
+    return t, pair_mask

@@ -14,11 +14,13 @@ path (``inject_fastnn``, ``inject_evoformer``, ``copy_*``; reference lines 24-15
   OPM linear_1/2/out       -> ``linear_a`` / ``linear_b`` / ``o_linear``
 The extra-MSA stack (``inject_extramsa``, reference lines 154-236,341-355) follows the same re-layout,
 with the global column attention's linear_q -> ``to_q``, linear_k | linear_v -> rows of ``to_kv``.
-Template and embedder stages are outside this build and are left as they are.
+Of the template stage only the pair stack is built (``inject_template_pair_stack``, same triangle /
+transition re-layout); the embedders are left as they are.
 """
 import torch
 
 from fastfold_amd.model.fastnn import EvoformerStack, ExtraMSAStack
+from fastfold_amd.model.fastnn.template import TemplatePairStack
 
 
 def copy_layernorm(model_fast, model_ori):
@@ -156,6 +158,44 @@ def inject_extramsa(model):
         if target_module.training is False:
             fast_module.eval()
         model.extra_msa_stack = fast_module
+
+
+def copy_template_pair_stack_para(block_fast, block_ori):
+    copy_triangle(block_fast.TriangleMultiplicationOutgoing, block_ori.tri_mul_out)
+    copy_triangle(block_fast.TriangleMultiplicationIncoming, block_ori.tri_mul_in)
+    copy_triangle_att(block_fast.TriangleAttentionStartingNode, block_ori.tri_att_start)
+    copy_triangle_att(block_fast.TriangleAttentionEndingNode, block_ori.tri_att_end)
+    copy_transition(block_fast.PairTransition, block_ori.pair_transition)
+
+
+def copy_template_pair_block_para(fast_module, target_module):
+    with torch.no_grad():
+        for ori_block, fast_block in zip(target_module.blocks, fast_module.blocks):
+            copy_template_pair_stack_para(fast_block, ori_block)
+            if ori_block.training is False:
+                fast_block.eval()
+
+
+def inject_template_pair_stack(template_embedder):
+    """Swaps ``template_embedder.template_pair_stack`` (nn layout) for the HIP-backed stack.  The
+    reference's ``inject_template`` (inject_fastnn.py:358-374) replaces the whole template embedder;
+    its embedders and point-wise attention are outside this build and stay as they are."""
+    with torch.no_grad():
+        target = template_embedder.template_pair_stack
+        blk = target.blocks[0]
+        ref_param = next(target.parameters())
+        fast = TemplatePairStack(
+            c_t=blk.tri_att_start.c_in, c_hidden_tri_att=blk.tri_att_start.c_hidden,
+            c_hidden_tri_mul=blk.tri_mul_out.c_hidden, no_blocks=len(target.blocks),
+            no_heads=blk.tri_att_start.no_heads, pair_transition_n=blk.pair_transition.n,
+            dropout_rate=getattr(blk, "dropout_rate", 0.25), blocks_per_ckpt=target.blocks_per_ckpt,
+            inf=blk.tri_att_start.inf).to(device=ref_param.device, dtype=ref_param.dtype)
+        copy_template_pair_block_para(fast, target)
+        copy_layernorm(fast.layer_norm, target.layer_norm)
+        if target.training is False:
+            fast.eval()
+        template_embedder.template_pair_stack = fast
+    return template_embedder
 
 
 def inject_evoformer(model):

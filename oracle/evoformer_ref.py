@@ -464,6 +464,55 @@ class ExtraMSAStack(nn.Module):
         return z
 
 
+# --------------------------------------------------------------------------
+# template pair stack  (reference: fastfold/model/nn/template.py:139-363)
+# --------------------------------------------------------------------------
+class TemplatePairStackBlock(nn.Module):
+    """Per template: tri-att start, tri-att end, tri-mul out, tri-mul in, pair transition, each added
+    to its input (template.py:205-242; dropout is the identity in eval mode)."""
+
+    def __init__(self, c_t, c_hidden_tri_att, c_hidden_tri_mul, no_heads, pair_transition_n, dropout_rate,
+                 inf, is_multimer=False, **kwargs):
+        super().__init__()
+        self.tri_att_start = TriangleAttentionStartingNode(c_t, c_hidden_tri_att, no_heads, inf=inf)
+        self.tri_att_end = TriangleAttentionEndingNode(c_t, c_hidden_tri_att, no_heads, inf=inf)
+        self.tri_mul_out = TriangleMultiplicationOutgoing(c_t, c_hidden_tri_mul)
+        self.tri_mul_in = TriangleMultiplicationIncoming(c_t, c_hidden_tri_mul)
+        self.pair_transition = PairTransition(c_t, pair_transition_n)
+
+    def forward(self, z, mask, chunk_size=None, _mask_trans=True):
+        outs = []
+        for single, single_mask in zip(torch.unbind(z, dim=-4), torch.unbind(mask, dim=-3)):
+            single, single_mask = single.unsqueeze(-4), single_mask.unsqueeze(-3)
+            single = single + self.tri_att_start(single, mask=single_mask)
+            single = single + self.tri_att_end(single, mask=single_mask)
+            single = single + self.tri_mul_out(single, mask=single_mask)
+            single = single + self.tri_mul_in(single, mask=single_mask)
+            single = single + self.pair_transition(single, mask=single_mask if _mask_trans else None)
+            outs.append(single)
+        return torch.cat(outs, dim=-4)
+
+
+class TemplatePairStack(nn.Module):
+    """no_blocks blocks, then a LayerNorm (template.py:326-363)."""
+
+    def __init__(self, c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_blocks=2, no_heads=4,
+                 pair_transition_n=2, dropout_rate=0.25, blocks_per_ckpt=None, inf=1e9, **kwargs):
+        super().__init__()
+        self.blocks_per_ckpt = blocks_per_ckpt
+        self.blocks = nn.ModuleList([
+            TemplatePairStackBlock(c_t, c_hidden_tri_att, c_hidden_tri_mul, no_heads, pair_transition_n,
+                                   dropout_rate, inf) for _ in range(no_blocks)])
+        self.layer_norm = LayerNorm(c_t)
+
+    def forward(self, t, mask, chunk_size=None, _mask_trans=True):
+        if mask.shape[-3] == 1:
+            mask = mask.expand(*mask.shape[:-3], t.shape[-4], *mask.shape[-2:])
+        for b in self.blocks:
+            t = b(t, mask, _mask_trans=_mask_trans)
+        return self.layer_norm(t)
+
+
 class OracleModel(nn.Module):
     """Minimal stand-in for the whole-model object the injection routine receives:
     it only has the ``evoformer`` attribute (reference call site: hub/alphafold.py:92-95)."""

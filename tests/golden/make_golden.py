@@ -1,9 +1,11 @@
-"""Writes tests/golden/evoformer_nn_golden.npz and tests/golden/extra_msa_nn_golden.npz by running
-the REFERENCE's own ``fastfold.model.nn.evoformer.EvoformerStack`` / ``ExtraMSAStack`` (plain
-PyTorch, CPU, fp32) on seeded synthetic weights and inputs.  Run only in the build container, where /root/reference is mounted:
+"""Writes tests/golden/evoformer_nn_golden.npz, extra_msa_nn_golden.npz and template_pair_nn_golden.npz by
+running the REFERENCE's own ``fastfold.model.nn.evoformer.EvoformerStack`` / ``ExtraMSAStack`` and
+``fastfold.model.nn.template.TemplatePairStack`` (plain PyTorch, CPU, fp32) on seeded synthetic weights
+and inputs.  Run only in the build container, where /root/reference is mounted:
 
     python tests/golden/make_golden.py            # Evoformer stack
     python tests/golden/make_golden.py extra      # extra-MSA stack
+    python tests/golden/make_golden.py template   # template pair stack
 
 The fixture pins what closed forms cannot: the composition of a block (order of the
 sub-updates, residual placement, OPM reading the updated MSA), the q/k/v and left/right
@@ -21,7 +23,8 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, "/root/reference")
 
-from fastfold_amd.synthetic import synth_extra_nn_state, synth_nn_state, synth_inputs  # noqa: E402
+from fastfold_amd.synthetic import (synth_extra_nn_state, synth_nn_state, synth_inputs,  # noqa: E402
+                                    synth_template_inputs, synth_template_nn_state)
 
 CASES = [
     # name, seed, no_blocks, n_seq, n_res, mask_tail_frac, fan_in_scaled
@@ -89,8 +92,39 @@ def main_extra():
     print("wrote", os.path.join(HERE, "extra_msa_nn_golden.npz"))
 
 
+TEMPLATE_CASES = [
+    # name, seed, no_blocks, n_templ, n_res, mask_tail_frac, fan_in_scaled
+    ("t2_n1_r12_pad", 31, 2, 1, 12, 0.17, True),
+    ("t2_n3_r9_full", 32, 2, 3, 9, 0.0, True),
+    ("t1_n2_r10_std002", 33, 1, 2, 10, 0.2, False),
+]
+
+
+def main_template():
+    from fastfold.model.nn.template import TemplatePairStack  # the reference
+
+    out = {}
+    for name, seed, nb, nt, r, tail, fis in TEMPLATE_CASES:
+        torch.manual_seed(0)
+        stack = TemplatePairStack(c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_blocks=nb, no_heads=4,
+                                  pair_transition_n=2, dropout_rate=0.25, blocks_per_ckpt=None, inf=1e9).eval()
+        sd = synth_template_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=fis)
+        missing, unexpected = stack.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        assert not missing and not unexpected
+        t, pair_mask = synth_template_inputs(seed, nt, r, mask_tail_frac=tail)
+        with torch.no_grad():
+            to = stack(torch.from_numpy(t), torch.from_numpy(pair_mask)[None], chunk_size=None, _mask_trans=False)
+        out[name + ".t"] = to.numpy()
+        out[name + ".cfg"] = np.array([seed, nb, nt, r, int(round(tail * 100)), int(fis)], dtype=np.int64)
+        print(name, "t", float(np.abs(to.numpy() - t).mean()))
+    np.savez_compressed(os.path.join(HERE, "template_pair_nn_golden.npz"), **out)
+    print("wrote", os.path.join(HERE, "template_pair_nn_golden.npz"))
+
+
 if __name__ == "__main__":
-    if "extra" in sys.argv[1:]:
+    if "template" in sys.argv[1:]:
+        main_template()
+    elif "extra" in sys.argv[1:]:
         main_extra()
     else:
         main()

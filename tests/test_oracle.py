@@ -233,3 +233,24 @@ def test_extra_msa_default_init_is_identity_and_masked_positions_do_not_leak():
                                pair_mask=torch.from_numpy(pm), _mask_trans=mt).numpy()[:7, :7])
     for o in outs[1:]:
         assert np.abs(o - outs[0]).max() < 1e-3
+
+
+# -------------------------------------------------------------- template pair stack ----
+TEMPLATE_GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "template_pair_nn_golden.npz")
+
+
+def test_template_pair_stack_golden_vectors_from_reference():
+    from fastfold_amd.synthetic import synth_template_inputs, synth_template_nn_state
+    from oracle.evoformer_ref import TemplatePairStack
+    g = np.load(TEMPLATE_GOLDEN)
+    names = sorted({k.split(".")[0] for k in g.files})
+    assert len(names) == 3
+    for name in names:
+        seed, nb, nt, r, tail, fis = (int(v) for v in g[name + ".cfg"])
+        st = TemplatePairStack(no_blocks=nb).eval()
+        sd = synth_template_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=bool(fis))
+        st.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        t, pm = synth_template_inputs(seed, nt, r, mask_tail_frac=tail / 100)
+        with torch.no_grad():
+            to = st(torch.from_numpy(t), torch.from_numpy(pm)[None], _mask_trans=False).numpy()
+        assert np.abs(to - g[name + ".t"]).max() <= 2e-5, name

@@ -1,0 +1,159 @@
+"""GPU parity of the template pair stack (the pair modules at c_t = 64, 4 heads of 16, multiplication
+width 64, transition factor 2) against the CPU oracle, itself pinned by golden vectors written by the
+reference's fastfold.model.nn.template.TemplatePairStack.
+
+Tolerances: fp32 max-abs <= 1e-4; bf16 relative L2 <= 2e-2 against the fp32 oracle."""
+import copy
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from fastfold_amd.synthetic import synth_template_inputs, synth_template_nn_state
+from oracle.evoformer_ref import TemplatePairStack as OracleStack
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "template_pair_nn_golden.npz")
+
+
+class _Embedder(torch.nn.Module):
+    def __init__(self, stack):
+        super().__init__()
+        self.template_pair_stack = stack
+
+
+def _t(x, dev, dtype):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev, dtype)
+
+
+def _f(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _rel_l2(a, b):
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-12))
+
+
+def _oracle(seed, nb, fis=True):
+    st = OracleStack(no_blocks=nb).eval()
+    sd = synth_template_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=fis)
+    st.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+    return st
+
+
+def _fast(oracle, dev, dtype):
+    from fastfold_amd.utils.inject_fastnn import inject_template_pair_stack
+    e = inject_template_pair_stack(_Embedder(copy.deepcopy(oracle)))
+    return e.template_pair_stack.to(device=dev, dtype=dtype).eval()
+
+
+SUB = ["tas", "tae", "tmo", "tmi", "ptrans"]
+
+
+def _oracle_sub(blk, name, z, pm):
+    with torch.no_grad():
+        if name == "tas":
+            return blk.tri_att_start(z, mask=pm)
+        if name == "tae":
+            return blk.tri_att_end(z, mask=pm)
+        if name == "tmo":
+            return blk.tri_mul_out(z, mask=pm)
+        if name == "tmi":
+            return blk.tri_mul_in(z, mask=pm)
+        return blk.pair_transition(z, mask=None)
+
+
+def _fast_sub(blk, name, z, pm):
+    with torch.no_grad():
+        if name == "tas":
+            return blk.TriangleAttentionStartingNode(z, pm) - z
+        if name == "tae":
+            return blk.TriangleAttentionEndingNode(z, pm) - z
+        if name == "tmo":
+            return blk.TriangleMultiplicationOutgoing(z, pm) - z
+        if name == "tmi":
+            return blk.TriangleMultiplicationIncoming(z, pm) - z
+        return blk.PairTransition(z) - z
+
+
+@pytest.mark.parametrize("r,tail", [(40, 0.2), (33, 0.0), (64, 0.1)])
+@pytest.mark.parametrize("name", SUB)
+def test_template_submodule_updates_fp32(dev, name, r, tail):
+    oracle = _oracle(51, 1)
+    fast = _fast(oracle, dev, torch.float32)
+    t, pm = synth_template_inputs(19, 1, r, mask_tail_frac=tail)
+    ref = _oracle_sub(oracle.blocks[0], name, torch.from_numpy(t), torch.from_numpy(pm)[None])[0].numpy()
+    got = _f(_fast_sub(fast.blocks[0], name, _t(t, dev, torch.float32), _t(pm[None], dev, torch.float32)))[0]
+    nv = r - int(round(tail * r))
+    got, ref = got[:nv, :nv], ref[:nv, :nv]
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert np.abs(got - ref).max() <= 1e-4 * scale, (name, np.abs(got - ref).max(), scale)
+
+
+@pytest.mark.parametrize("r,tail", [(64, 0.1), (96, 0.0)])
+@pytest.mark.parametrize("name", SUB)
+def test_template_submodule_updates_bf16(dev, name, r, tail):
+    oracle = _oracle(52, 1)
+    fast = _fast(oracle, dev, torch.bfloat16)
+    t, pm = synth_template_inputs(20, 1, r, mask_tail_frac=tail)
+    tb = _f(_t(t, dev, torch.bfloat16))
+    ref = _oracle_sub(oracle.blocks[0], name, torch.from_numpy(tb), torch.from_numpy(pm)[None])[0].numpy()
+    out = _f(_fast_sub(fast.blocks[0], name, _t(tb, dev, torch.bfloat16), _t(pm[None], dev, torch.bfloat16)))[0]
+    nv = r - int(round(tail * r))
+    got, ref, base = out[:nv, :nv], ref[:nv, :nv], tb[0, :nv, :nv]
+    err = np.linalg.norm(got - ref)
+    bound = 2e-2 * np.linalg.norm(ref) + 2.0 ** -8 * np.linalg.norm(base + ref)
+    assert err <= bound, (name, err, bound)
+
+
+def test_template_golden_vectors_fp32(dev):
+    g = np.load(GOLDEN)
+    for name in sorted({k.split(".")[0] for k in g.files}):
+        seed, nb, nt, r, tail, fis = (int(v) for v in g[name + ".cfg"])
+        fast = _fast(_oracle(seed, nb, bool(fis)), dev, torch.float32)
+        t, pm = synth_template_inputs(seed, nt, r, mask_tail_frac=tail / 100)
+        tt, tpm = _t(t, dev, torch.float32), _t(pm[None], dev, torch.float32)
+        keep = tt.clone()
+        with torch.no_grad():
+            to = fast(tt, tpm, chunk_size=None)
+        assert torch.equal(tt, keep), "forward must not modify its input"
+        nv = r - int(round(tail / 100 * r))
+        got, ref = _f(to)[:, :nv, :nv], g[name + ".t"][:, :nv, :nv]
+        assert np.abs(got - ref).max() <= 1e-4, (name, np.abs(got - ref).max())
+        tl = [tt.clone()]
+        with torch.no_grad():
+            tl = fast.inplace(tl, tpm, chunk_size=None)
+        assert torch.equal(tl[0], to)
+
+
+def test_template_block_interface_padding_and_chaining(dev):
+    oracle = _oracle(53, 3)
+    fast = _fast(oracle, dev, torch.float32)
+    r = 24
+    t, pm = synth_template_inputs(53, 1, r, mask_tail_frac=0.1)
+    tt, tpm = _t(t, dev, torch.float32), _t(pm[None], dev, torch.float32)
+    with torch.no_grad():
+        want = fast(tt, tpm, chunk_size=None)
+        a = fast.blocks[0](tt, tpm)
+        assert a.shape == (1, r + 1, r + 1, 64)
+        a = fast.blocks[1](a, tpm)
+        assert a.shape == (1, r + 1, r + 1, 64)
+        a = fast.blocks[2](a, tpm)
+        assert a.shape == (1, r, r, 64)
+        a = fast.layer_norm(a)
+    assert torch.equal(a, want)
+
+
+def test_template_stack_bf16_rel_l2(dev):
+    nb, nt, r, tail = 2, 2, 72, 0.1
+    oracle = _oracle(54, nb)
+    fast = _fast(oracle, dev, torch.bfloat16)
+    t, pm = synth_template_inputs(54, nt, r, mask_tail_frac=tail)
+    tb = _f(_t(t, dev, torch.bfloat16))
+    with torch.no_grad():
+        ref = oracle(torch.from_numpy(tb), torch.from_numpy(pm)[None], _mask_trans=False).numpy()
+        got = _f(fast(_t(tb, dev, torch.bfloat16), _t(pm[None], dev, torch.bfloat16), chunk_size=None))
+    nv = r - int(round(tail * r))
+    assert _rel_l2(got[:, :nv, :nv], ref[:, :nv, :nv]) <= 2e-2
