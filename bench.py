@@ -127,6 +127,51 @@ def micro_ops(dev):
     return res
 
 
+def feeder_stacks(dev, r):
+    """The two stacks that run before the Evoformer (hub/alphafold.py:262-362) at their own widths, random
+    weights: the 4-block extra-MSA stack on 1024 extra sequences and the 2-block template pair stack on one
+    template; milliseconds per block."""
+    import torch
+    from fastfold_amd.model.fastnn import ExtraMSAStack, TemplatePairStack
+
+    def init(mod):
+        g = torch.Generator().manual_seed(0)
+        with torch.no_grad():
+            for n, p in mod.named_parameters():
+                ln_w = ("norm" in n) and n.endswith("weight")
+                p.copy_((1.0 if ln_w else 0.0) + 0.02 * torch.randn(p.shape, generator=g))
+        return mod.to(dev, torch.bfloat16).eval()
+
+    def timed(fn, blocks, reps=2):
+        with torch.no_grad():
+            fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                out = fn()
+            torch.cuda.synchronize()
+        assert bool(torch.isfinite(out.float()).all())
+        return round((time.perf_counter() - t0) * 1e3 / reps / blocks, 4)
+
+    res = {}
+    se = 1024
+    g = torch.Generator().manual_seed(1)
+    ex = init(ExtraMSAStack(c_m=64, c_z=128, no_blocks=4))
+    m = torch.randn(se, r, 64, generator=g).to(dev, torch.bfloat16)
+    z = torch.randn(r, r, 128, generator=g).to(dev, torch.bfloat16)
+    mm = torch.ones(se, r, device=dev, dtype=torch.bfloat16)
+    pm = torch.ones(r, r, device=dev, dtype=torch.bfloat16)
+    res["extra_msa_stack"] = {"workload": "4 blocks, N_extra=%d, N_res=%d, c_e=64" % (se, r),
+                              "ms_per_block": timed(lambda: ex(m, z, chunk_size=None, msa_mask=mm, pair_mask=pm), 4)}
+    del ex, m, z, mm
+    tp = init(TemplatePairStack(c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_blocks=2, no_heads=4,
+                                pair_transition_n=2, dropout_rate=0.25, blocks_per_ckpt=None))
+    t = torch.randn(1, r, r, 64, generator=g).to(dev, torch.bfloat16)
+    res["template_pair_stack"] = {"workload": "2 blocks, 1 template, N_res=%d, c_t=64" % r,
+                                  "ms_per_block": timed(lambda: tp(t, pm[None], chunk_size=None), 2)}
+    return res
+
+
 def cpu_baseline(threads):
     """The CPU oracle timed on the host cores: one fp32 block at N_seq=128, N_res=256."""
     import numpy as np
@@ -239,6 +284,7 @@ def main():
     del stack, out
     torch.cuda.empty_cache()
     if not args.no_micro:
+        line["feeders"] = feeder_stacks(dev, r)
         line["ops"] = micro_ops(dev)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))

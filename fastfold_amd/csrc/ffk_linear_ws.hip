@@ -1,6 +1,7 @@
 // Weights-stationary variant of the fused linear layer (see ffk_fused_linear in include/ffk.h),
-// bf16, K = 128 or 256: the projections of the pair and MSA stacks, where M is 10^5 .. 10^6 rows and
-// the whole weight matrix is a few hundred KB.
+// bf16, K = 64, 128 or 256: the projections of the pair and MSA stacks (and of the extra-MSA and
+// template stacks at 64 channels), where M is 10^5 .. 10^6 rows and the whole weight matrix is a few
+// hundred KB.
 //
 // One persistent workgroup of 8 wavefronts per CU.  The weight matrix is split into "slots" of 32
 // output rows; every wave keeps the MFMA fragments of up to three slots in registers for the whole
@@ -23,7 +24,7 @@ namespace {
 
 constexpr int WS_WAVES = 8;
 constexpr int WS_THREADS = 64 * WS_WAVES;
-constexpr int WS_NS = 3;                 // weight slots per wave (two with K = 256, where a slot costs 64 registers)
+constexpr int WS_NS = 4;                 // weight slots per wave: up to 4 (K = 64), 3 (K = 128), 2 (K = 256, 64 registers a slot)
 constexpr int WS_MAX_GRID = 256;         // one workgroup per CU
 // Per-K geometry: a slab is as many rows as 512 threads fetch with four 16-byte loads each.
 template <int K> struct WsGeo {
@@ -62,6 +63,7 @@ struct WsSlot {
     const T* gate;
     long s_o, s_i, s_d, gate_ld;
     unsigned inner;
+    unsigned gate_rows;      // 0, or the period of the gate's row index
     int ncols_left;          // valid channels from the unit's first channel on
     int kind, act;
     float scale;
@@ -165,7 +167,7 @@ __device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc
         if (t.gate || t.resid) {
             // every load first (clamped, unconditional), then combine and store
             u32x4 gv[2], rv[2];
-            const T* gate = t.gate ? t.gate + (long)mc * t.gate_ld + cl : nullptr;
+            const T* gate = t.gate ? t.gate + (long)(t.gate_rows ? mc % t.gate_rows : mc) * t.gate_ld + cl : nullptr;
             const T* resid = t.resid ? t.resid + off : nullptr;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -264,7 +266,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     typedef Mma<T> MM;
     typedef WsGeo<WS_K> G;
     constexpr int WS_KS = G::KS, WS_AP = G::AP, WS_BM = G::BM, WS_RG = G::RG, LPR = G::LPR, RPP = G::RPP;
-    constexpr bool ALLOW_GLU = NS >= 2 && WS_K == 128;
+    constexpr bool ALLOW_GLU = NS >= 2 && WS_K <= 128;
     constexpr int AFC = WS_K == 128 ? 8 : 4;               // A fragments held at a time (register budget)
     const ffk_linear_desc& d = args.d;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -317,6 +319,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             sp[s].s_i = ts.s_i;
             sp[s].s_d = ts.s_d;
             sp[s].gate_ld = ts.gate_ld;
+            sp[s].gate_rows = (unsigned)ts.gate_rows;
             sp[s].inner = (unsigned)ts.inner;
             sp[s].ncols_left = ts.ncols - s_chan[s];
             sp[s].kind = ts.kind;
@@ -596,7 +599,6 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (t.inner <= 0 || t.ncols <= 0 || !al16(t.out)) return false;
-    if (t.gate && t.gate_rows != 0) return false;      // periodic gate rows: generic kernel only
     if (ws_by_rows(t)) {
         if (t.kind == FFK_TILE_STRIDED) {
             if (t.ncols % 8 != 0 || t.s_o % 8 || t.s_i % 8 || t.s_h % 8) return false;
@@ -713,7 +715,7 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
 // Launches the weights-stationary kernel if it can take this (already validated) descriptor and
 // returns 1 with the launch status in *status; returns 0 if the caller has to use another variant.
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
-    if (d->dtype != FFK_BF16 || (d->K != 128 && d->K != 256)) return 0;
+    if (d->dtype != FFK_BF16 || (d->K != 64 && d->K != 128 && d->K != 256)) return 0;
     if (d->a_chanmajor && (d->K != 128 || d->a_si != 1 || d->a_inner % 8 || d->a_so % 8 || d->a_cs % 8 || d->M % 8)) return 0;
     const bool k256 = d->K == 256;
     if (getenv("FFK_NO_WS")) return 0;
@@ -735,7 +737,10 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     }
     if (chan_major && v_tiles) return 0;          // they need different row orders within a group
     WsArgs args;
-    if (!ws_make_plan(*d, args.plan, k256 ? WsGeo<256>::RG : WsGeo<128>::RG, k256 ? 2 : WS_NS)) return 0;
+    const bool k64 = d->K == 64;
+    if (!ws_make_plan(*d, args.plan, k256 ? WsGeo<256>::RG : (k64 ? WsGeo<64>::RG : WsGeo<128>::RG),
+                      k256 ? 2 : (k64 ? 4 : 3)))
+        return 0;
     if (k256) {
         for (int i = 0; i < d->n_tiles; ++i)
             if (d->tiles[i].glu) return 0;                   // GLU units are only built for K = 128
@@ -754,6 +759,8 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
         *status = ws_launch<2, 128, true>(args, st);
     } else if (k256) {
         *status = ws_launch<2, 256, false>(args, st);
+    } else if (k64) {
+        *status = args.plan.max_slots <= 2 ? ws_launch<2, 64, false>(args, st) : ws_launch<4, 64, false>(args, st);
     } else {
         *status = args.plan.max_slots <= 2 ? ws_launch<2, 128, false>(args, st) : ws_launch<3, 128, false>(args, st);
     }

@@ -192,7 +192,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     v_t = alloc((B2, H, NT, 1024), dt, dev, zero)
     # With bf16, 128 input channels and whole key tiles the projection runs on the weights-stationary
     # kernel, which writes q, k and the gate in accumulator order straight from its registers.
-    acc_order = dt == torch.bfloat16 and C in (128, 256) and N % 32 == 0
+    acc_order = dt == torch.bfloat16 and C in (64, 128, 256) and N % 32 == 0
     qk_kind = FFK_TILE_ACC if acc_order else FFK_TILE_QK
     gate = torch.empty((B2, H, NT, 1024) if acc_order else (M, HC), dtype=dt, device=dev)
     tpg = HC // 128
@@ -222,9 +222,12 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     for t0 in range(0, len(tiles), per):
         _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
                           w_row_off=t0 * 128)
-    if bias_tile is not None:      # the skinny bias projection has its own pass over x
+    if bias_tile is not None and C == 128:      # the skinny bias projection has its own pass over x
         _pair_bias_launch(bias_t, x, ln, w_pk[4 * tpg * 128:], pb_scratch, N=N, C=C, H=H, a_inner=a_inner,
                           a_so=a_so, a_si=a_si, scale=LOG2E)
+    elif bias_tile is not None:
+        _lib.fused_linear(x, w_pk, [bias_tile], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
+                          w_row_off=4 * tpg * 128)
     def key_bias():
         kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
         flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
