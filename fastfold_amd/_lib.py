@@ -285,3 +285,12 @@ def global_attention_core(o, m, mask, gamma, beta, wq, wk, wv, *, S, R, C, H, D,
                           scaling, eps, ln_eps=1e-5):
     call("ffk_global_attention_core", ptr(o), ptr(m), ptr(mask), ptr(gamma), ptr(beta), ln_eps, ptr(wq), ptr(wk),
          ptr(wv), S, R, C, H, D, m_ss, m_sr, mask_ss, mask_sr, scaling, eps, dtype_tag(m.dtype), stream_ptr())
+
+
+FFK_EMBED_RELPOS, FFK_EMBED_DISTOGRAM = 0, 1
+SIGNATURES["ffk_pair_embed"] = [_P, _P, _P, _P, _F, _P, _P, _P, _P, _I, _P, _P, _F, _L, _L, _L, _I, _P]
+
+
+def pair_embed(out, z, gamma, beta, table, bias, row, col, *, mode, pos, edges=None, inf=1e8, r, C, nb, ln_eps=1e-5):
+    call("ffk_pair_embed", ptr(out), ptr(z), ptr(gamma), ptr(beta), ln_eps, ptr(table), ptr(bias), ptr(row), ptr(col),
+         mode, ptr(pos), ptr(edges), inf, r, C, nb, dtype_tag(out.dtype), stream_ptr())

@@ -527,9 +527,11 @@ class ChunkTriangleAttentionEndingNode(_TriangleAttention):
 
 
 def __getattr__(name):
-    # the reference keeps the chunked row attention in this module (ops.py:751-867); here it lives
-    # beside the un-chunked one, which this module cannot import at load time
+    # the reference keeps these classes in this module; here they live in modules that import this one
     if name == "ChunkMSARowAttentionWithPairBias":
         from .msa import ChunkMSARowAttentionWithPairBias
         return ChunkMSARowAttentionWithPairBias
+    if name in ("InputEmbedder", "RecyclingEmbedder"):      # ops.py:1046-1145,1238-1334
+        from . import embedders
+        return getattr(embedders, name)
     raise AttributeError("module %r has no attribute %r" % (__name__, name))

@@ -15,11 +15,12 @@ path (``inject_fastnn``, ``inject_evoformer``, ``copy_*``; reference lines 24-15
 The extra-MSA stack (``inject_extramsa``, reference lines 154-236,341-355) follows the same re-layout,
 with the global column attention's linear_q -> ``to_q``, linear_k | linear_v -> rows of ``to_kv``.
 Of the template stage only the pair stack is built (``inject_template_pair_stack``, same triangle /
-transition re-layout); the embedders are left as they are.
+transition re-layout); ``inject_embedder`` swaps the input and recycling embedders (plain copies).
 """
 import torch
 
 from fastfold_amd.model.fastnn import EvoformerStack, ExtraMSAStack
+from fastfold_amd.model.fastnn.embedders import InputEmbedder, RecyclingEmbedder
 from fastfold_amd.model.fastnn.template import TemplatePairStack
 
 
@@ -198,6 +199,39 @@ def inject_template_pair_stack(template_embedder):
     return template_embedder
 
 
+def copy_native_linear(model_fast, model_ori):
+    model_fast.weight.copy_(model_ori.weight)
+    model_fast.bias.copy_(model_ori.bias)
+
+
+def inject_embedder(model):
+    """Swaps ``model.recycling_embedder`` and ``model.input_embedder`` (inject_fastnn.py:376-416); nothing is
+    done for a multimer model, as in the reference."""
+    if model.evoformer.blocks[0].is_multimer:
+        return
+    with torch.no_grad():
+        target = model.recycling_embedder
+        ref_param = next(target.parameters())
+        fast = RecyclingEmbedder(c_m=target.c_m, c_z=target.c_z, min_bin=target.min_bin, max_bin=target.max_bin,
+                                 no_bins=target.no_bins, inf=target.inf).to(device=ref_param.device, dtype=ref_param.dtype)
+        copy_native_linear(fast.linear, target.linear)
+        copy_layernorm(fast.layer_norm_m, target.layer_norm_m)
+        copy_layernorm(fast.layer_norm_z, target.layer_norm_z)
+        if target.training is False:
+            fast.eval()
+        model.recycling_embedder = fast
+
+        target = model.input_embedder
+        ref_param = next(target.parameters())
+        fast = InputEmbedder(tf_dim=target.tf_dim, msa_dim=target.msa_dim, c_z=target.c_z, c_m=target.c_m,
+                             relpos_k=target.relpos_k).to(device=ref_param.device, dtype=ref_param.dtype)
+        for name in ("linear_tf_z_i", "linear_tf_z_j", "linear_tf_m", "linear_msa_m", "linear_relpos"):
+            copy_linear(getattr(fast, name), getattr(target, name))
+        if target.training is False:
+            fast.eval()
+        model.input_embedder = fast
+
+
 def inject_evoformer(model):
     with torch.no_grad():
         target_module = model.evoformer
@@ -222,11 +256,16 @@ def inject_evoformer(model):
 
 
 def inject_fastnn(model):
-    """Replaces ``model.evoformer`` and, where the model has one, ``model.extra_msa_stack``; returns the
-    model (reference: inject_fastnn.py:418-423)."""
+    """Replaces ``model.evoformer`` and, where the model has them, ``model.extra_msa_stack``, the template
+    embedder's pair stack and the input / recycling embedders; returns the model (reference:
+    inject_fastnn.py:418-423)."""
     inject_evoformer(model)
     if getattr(model, "extra_msa_stack", None) is not None:
         inject_extramsa(model)
+    if getattr(model, "template_embedder", None) is not None and hasattr(model.template_embedder, "template_pair_stack"):
+        inject_template_pair_stack(model.template_embedder)
+    if getattr(model, "input_embedder", None) is not None and getattr(model, "recycling_embedder", None) is not None:
+        inject_embedder(model)
     return model
 
 

@@ -303,6 +303,26 @@ int ffk_global_attention_core(void* o, const void* m, const void* mask, const vo
                               int64_t m_ss, int64_t m_sr, int64_t mask_ss, int64_t mask_sr,
                               float scaling, float eps, int dtype, void* stream);
 
+/* Pair-representation part of the input embedder and of the recycling embedder:
+ *     out[i, j, :] = [LayerNorm(z[i, j, :])] + table[bin(i, j), :] + [bias] + [row[i, :]] + [col[j, :]]
+ * (terms in brackets are skipped when their pointer is NULL; a pair that falls in no bin gets no table row).
+ * A Linear applied to a one-hot vector picks one column of its weight: `table` is that weight transposed,
+ * [nb, C], and the one-hot tensor is never formed.
+ *   FFK_EMBED_RELPOS     pos : [r] residue indices (fp32); bin = nearest of the offsets -k .. k (nb = 2k + 1)
+ *                        to pos[i] - pos[j], the lower one on a tie
+ *   FFK_EMBED_DISTOGRAM  pos : [r, 3] coordinates (fp32); edges : [nb] squared lower bin edges (fp32);
+ *                        bin = the b with edges[b] < |pos_i - pos_j|^2 < edges[b + 1] (inf after the last),
+ *                        open intervals as in the reference: a distance on an edge is in no bin
+ * out, z : [r, r, C] (may alias), C in {64, 128, 256}; row, col : [r, C]; fp32 or bf16.
+ * Replaces: InputEmbedder.forward's relpos / one_hot / linear_relpos / broadcast adds and
+ * RecyclingEmbedder.forward's distogram one-hot / linear / layer_norm_z
+ * (fastfold/model/fastnn/ops.py:1306-1324, 1108-1145; nn/embedders.py:82-127, 208-230). */
+enum { FFK_EMBED_RELPOS = 0, FFK_EMBED_DISTOGRAM = 1 };
+int ffk_pair_embed(void* out, const void* z, const void* ln_gamma, const void* ln_beta, float ln_eps,
+                   const void* table, const void* bias, const void* row, const void* col, int mode,
+                   const float* pos, const float* edges, float inf, int64_t r, int64_t C, int64_t nb,
+                   int dtype, void* stream);
+
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the
  * given dtype, or NULL (all keys valid).  tileflags[b, k/32] classifies each 32-key tile (see

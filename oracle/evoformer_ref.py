@@ -513,6 +513,69 @@ class TemplatePairStack(nn.Module):
         return self.layer_norm(t)
 
 
+# --------------------------------------------------------------------------
+# input and recycling embedders  (reference: fastfold/model/nn/embedders.py:35-232,
+# one_hot: fastfold/utils/tensor_utils.py:63-67)
+# --------------------------------------------------------------------------
+def one_hot_nearest(x, v_bins):
+    """One-hot of the bin centre nearest to x (first one on a tie)."""
+    diffs = x[..., None] - v_bins.view(((1,) * x.dim()) + (len(v_bins),))
+    am = torch.argmin(torch.abs(diffs), dim=-1)
+    return F.one_hot(am, num_classes=len(v_bins)).float()
+
+
+class InputEmbedder(nn.Module):
+    """Algorithms 3 and 4 (embedders.py:99-135): pair_emb[i, j] = W_i tf[i] + W_j tf[j] + W_rel
+    onehot(clip(ri[i] - ri[j], +-k)), msa_emb[s, i] = W_msa msa[s, i] + W_tf tf[i] (biases included)."""
+
+    def __init__(self, tf_dim, msa_dim, c_z, c_m, relpos_k, **kwargs):
+        super().__init__()
+        self.tf_dim, self.msa_dim, self.c_z, self.c_m = tf_dim, msa_dim, c_z, c_m
+        self.linear_tf_z_i = Linear(tf_dim, c_z)
+        self.linear_tf_z_j = Linear(tf_dim, c_z)
+        self.linear_tf_m = Linear(tf_dim, c_m)
+        self.linear_msa_m = Linear(msa_dim, c_m)
+        self.relpos_k = relpos_k
+        self.no_bins = 2 * relpos_k + 1
+        self.linear_relpos = Linear(self.no_bins, c_z)
+
+    def relpos(self, ri):
+        d = ri[..., None] - ri[..., None, :]
+        boundaries = torch.arange(start=-self.relpos_k, end=self.relpos_k + 1, device=d.device)
+        return self.linear_relpos(one_hot_nearest(d, boundaries).type(ri.dtype))
+
+    def forward(self, tf, ri, msa):
+        tf_emb_i = self.linear_tf_z_i(tf)
+        tf_emb_j = self.linear_tf_z_j(tf)
+        pair_emb = tf_emb_i[..., None, :] + tf_emb_j[..., None, :, :]
+        pair_emb = pair_emb + self.relpos(ri.type(pair_emb.dtype))
+        tf_m = self.linear_tf_m(tf).unsqueeze(-3)
+        msa_emb = self.linear_msa_m(msa) + tf_m
+        return msa_emb, pair_emb
+
+
+class RecyclingEmbedder(nn.Module):
+    """Algorithm 32 (embedders.py:183-232): m_update = LN(m); z_update = LN(z) + W onehot(bin of
+    |x_i - x_j|^2 among the squared bin edges, open intervals: a distance on an edge or below the first
+    one falls in no bin) + b."""
+
+    def __init__(self, c_m, c_z, min_bin, max_bin, no_bins, inf=1e8, **kwargs):
+        super().__init__()
+        self.c_m, self.c_z, self.min_bin, self.max_bin, self.no_bins, self.inf = c_m, c_z, min_bin, max_bin, no_bins, inf
+        self.linear = Linear(no_bins, c_z)
+        self.layer_norm_m = LayerNorm(c_m)
+        self.layer_norm_z = LayerNorm(c_z)
+
+    def forward(self, m, z, x):
+        bins = torch.linspace(self.min_bin, self.max_bin, self.no_bins, dtype=x.dtype, device=x.device)
+        m_update = self.layer_norm_m(m)
+        squared_bins = bins ** 2
+        upper = torch.cat([squared_bins[1:], squared_bins.new_tensor([self.inf])], dim=-1)
+        d = torch.sum((x[..., None, :] - x[..., None, :, :]) ** 2, dim=-1, keepdims=True)
+        d = ((d > squared_bins) * (d < upper)).type(x.dtype)
+        return m_update, self.linear(d) + self.layer_norm_z(z)
+
+
 class OracleModel(nn.Module):
     """Minimal stand-in for the whole-model object the injection routine receives:
     it only has the ``evoformer`` attribute (reference call site: hub/alphafold.py:92-95)."""

@@ -254,3 +254,60 @@ def test_template_pair_stack_golden_vectors_from_reference():
         with torch.no_grad():
             to = st(torch.from_numpy(t), torch.from_numpy(pm)[None], _mask_trans=False).numpy()
         assert np.abs(to - g[name + ".t"]).max() <= 2e-5, name
+
+
+# ------------------------------------------------------------------------ embedders ----
+def test_embedders_brute_force():
+    """No golden vectors here: the reference's nn/embedders.py imports dm-tree, which this image lacks.
+    A linear layer on a one-hot vector is a column pick, so both embedders have closed forms that the
+    float64 loops below restate independently (indices by explicit comparison, not by one_hot)."""
+    from oracle.evoformer_ref import InputEmbedder, RecyclingEmbedder
+    torch.manual_seed(0)
+    ie = InputEmbedder(tf_dim=22, msa_dim=49, c_z=16, c_m=24, relpos_k=4).double()
+    with torch.no_grad():
+        for p in ie.parameters():
+            p.copy_(torch.randn_like(p))
+    rng = np.random.RandomState(0)
+    r, s = 9, 3
+    tf, msa = rng.standard_normal((r, 22)), rng.standard_normal((s, r, 49))
+    ri = np.array([0, 1, 2, 3, 10, 11, 12, 40, 41], dtype=np.float64)      # gaps beyond the +-4 window
+    with torch.no_grad():
+        m_emb, z_emb = (t.numpy() for t in ie(torch.from_numpy(tf), torch.from_numpy(ri), torch.from_numpy(msa)))
+    P = {k: v.detach().numpy() for k, v in ie.named_parameters()}
+    for i in range(r):
+        for j in range(r):
+            b = int(min(max(ri[i] - ri[j], -4), 4)) + 4
+            want = (P["linear_tf_z_i.weight"] @ tf[i] + P["linear_tf_z_i.bias"] + P["linear_tf_z_j.weight"] @ tf[j]
+                    + P["linear_tf_z_j.bias"] + P["linear_relpos.weight"][:, b] + P["linear_relpos.bias"])
+            assert np.abs(z_emb[i, j] - want).max() < 1e-10
+        for q in range(s):
+            want = (P["linear_msa_m.weight"] @ msa[q, i] + P["linear_msa_m.bias"] + P["linear_tf_m.weight"] @ tf[i]
+                    + P["linear_tf_m.bias"])
+            assert np.abs(m_emb[q, i] - want).max() < 1e-10
+    re_ = RecyclingEmbedder(c_m=24, c_z=16, min_bin=3.25, max_bin=20.75, no_bins=15).double()
+    with torch.no_grad():
+        for p in re_.parameters():
+            p.copy_(torch.randn_like(p))
+    x = rng.standard_normal((r, 3)) * 8.0
+    x[1] = x[0] + np.array([3.25, 0.0, 0.0])       # exactly on the first edge: no bin
+    m, z = rng.standard_normal((r, 24)), rng.standard_normal((r, r, 16))
+    with torch.no_grad():
+        mu, zu = (t.numpy() for t in re_(torch.from_numpy(m), torch.from_numpy(z), torch.from_numpy(x)))
+    P = {k: v.detach().numpy() for k, v in re_.named_parameters()}
+    edges = np.linspace(3.25, 20.75, 15)
+
+    def ln(v, g, b):
+        return (v - v.mean()) / np.sqrt(v.var() + 1e-5) * g + b
+    none_hit = 0
+    for i in range(r):
+        assert np.abs(mu[i] - ln(m[i], P["layer_norm_m.weight"], P["layer_norm_m.bias"])).max() < 1e-10
+        for j in range(r):
+            d2 = float(((x[i] - x[j]) ** 2).sum())
+            hit = [b for b in range(15) if d2 > edges[b] ** 2 and d2 < (edges[b + 1] ** 2 if b < 14 else 1e8)]
+            assert len(hit) <= 1
+            none_hit += not hit
+            want = ln(z[i, j], P["layer_norm_z.weight"], P["layer_norm_z.bias"]) + P["linear.bias"]
+            if hit:
+                want = want + P["linear.weight"][:, hit[0]]
+            assert np.abs(zu[i, j] - want).max() < 1e-10
+    assert none_hit >= r + 2        # the diagonal and the pair on the edge
