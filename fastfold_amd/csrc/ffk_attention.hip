@@ -27,6 +27,13 @@ template <typename T> struct Ops16 {   // the 16 elements one lane owns of a 102
 #pragma unroll
         for (int i = 0; i < NV; ++i) v[i] = ld16(p + i * DT<T>::VEC);
     }
+    // the same 16 elements from a tile kept in LDS vector-interleaved: vector i of lane l at (i * 64 + l)
+    // * 16 bytes, so that the 64 lanes of one read touch 1 KB of consecutive addresses (the tile's own
+    // order, 32 or 64 bytes from lane to lane, makes every 16-byte read a two- or four-way bank conflict)
+    __device__ __forceinline__ void load_lds(const T* tile, int lane) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) v[i] = ld16(tile + (i * 64 + lane) * DT<T>::VEC);
+    }
     __device__ __forceinline__ float f(int j) const { return DT<T>::to_f(v[j / DT<T>::VEC].e[j % DT<T>::VEC]); }
     // MFMA fragment number i (KLANE elements each)
     __device__ __forceinline__ typename Mma<T>::Frag frag(int i) const {
@@ -131,8 +138,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     const int* fl = tileflags + (long)b2 * KT;
 
     // cooperative operand fetch: vector slot v = tid + i * ATT_THREADS -> (tile, vector in tile).  The
-    // 16-byte vectors go from global memory straight into LDS (no staging registers): the 64 lanes of a
-    // wave cover 64 consecutive vectors of one tile, which the hardware places at  base + 16 * lane.
+    // 16-byte vectors go from global memory straight into LDS (no staging registers); the hardware places
+    // the 64 vectors of a request at  base + 16 * lane,  while the source address is per lane: a request
+    // gathers vector c of each lane's 16 elements (stride 16 * NV bytes), which leaves the tile in LDS
+    // vector-interleaved (see Ops16::load_lds).
     static_assert(NVL * ATT_THREADS == NTILES * TILE_VECS, "every thread fetches the same number of vectors");
     const T* src[NVL];                            // wave-uniform: start of the wave's 64 vectors in key tile 0
 #pragma unroll
@@ -149,7 +158,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
             qq = qq < QT ? qq : QT - 1;
             base = bias_t + ((((long)h * QT + qq) * KT) << 10);
         }
-        src[i] = base + wv * VEC;
+        // the wave's 64 vectors of this request: vector number wv / 64 of every lane's 16 elements
+        src[i] = base + (wv / 64) * VEC;
     }
 
     // gate values of this lane's 16 outputs, fetched now so that their latency is hidden by the loop
@@ -219,7 +229,7 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     // the issue), while here the slot being filled is never the slot being read.  The explicit wait
     // at the top of the loop is what orders them.
     const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)att_smem;
-    const unsigned lane_off = lane * 16;          // byte offset of this lane's vector; the base address is scalar
+    const unsigned lane_off = lane * 16 * Ops16<T>::NV;   // byte offset of this lane's 16 elements; the base address is scalar
     auto fetch = [&](int kt, int slot) {
 #pragma unroll
         for (int i = 0; i < NVL; ++i) {
@@ -257,14 +267,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
         const T* buf = lds + slot * NTILES * 1024;
         slot = slot == 2 ? 0 : slot + 1;
         Ops16<T> vc;
-        vc.load(buf + (2 + bsel) * 1024 + lane * 16);
+        vc.load_lds(buf + (2 + bsel) * 1024, lane);
 
         // S^T - m_ref = K . Q^T + Bias^T . I + (-m_ref)   (rows: keys, columns: queries)
         f32x16 s;
         auto score_tile = [&]() {
             Ops16<T> kc, bc;
-            kc.load(buf + bsel * 1024 + lane * 16);
-            if (HAS_BIAS) bc.load(buf + (4 + qsel) * 1024 + lane * 16);
+            kc.load_lds(buf + bsel * 1024, lane);
+            if (HAS_BIAS) bc.load_lds(buf + (4 + qsel) * 1024, lane);
             s = negm;
 #pragma unroll
             for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
