@@ -33,7 +33,7 @@ WORKLOADS = {
                  attn_traffic=None),
     "cfg4": dict(n_seq=128, n_res=1024, tail=0.05,
                  name="configs[3]: 48-block stack bf16 N_seq=128 N_res=1024, last 5% of residues masked",
-                 attn_traffic=1.453e9),
+                 attn_traffic=1.417e9),
 }
 
 
@@ -205,6 +205,8 @@ def main():
     ap.add_argument("--blocks", type=int, default=48)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
+    ap.add_argument("--only-feeders", action="store_true",
+                    help="time only the extra-MSA and template pair stacks (for profiling them on their own)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the Evoformer on ONE GPU (DAP size 1, no collectives); "
@@ -218,6 +220,9 @@ def main():
     dev = torch.device("cuda:0")
     wl = WORKLOADS[args.workload]
     s, r = wl["n_seq"], wl["n_res"]
+    if args.only_feeders:
+        print(json.dumps({"feeders": feeder_stacks(dev, r)}))
+        return
     stack = build_stack(args.blocks, dev, torch.bfloat16)
     m, z, mm, pm = (torch.from_numpy(t).to(dev, torch.bfloat16) for t in synth_inputs(0, s, r, mask_tail_frac=wl["tail"]))
 
