@@ -19,6 +19,7 @@
 // attention kernel loads them.
 #include "ffk_common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
@@ -76,6 +77,9 @@ __device__ __forceinline__ float ws_sigmoid_pre(float acc, float bs) {
     return fast_rcp(1.0f + fast_exp2(__builtin_fmaf(acc, -1.4426950408889634f, bs)));
 }
 
+// max(x, 0) as one instruction (fmaxf also canonicalises its argument first)
+__device__ __forceinline__ float ws_relu(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, 3.0e38f); }
+
 // tiles stored with channels contiguous (lane = row) vs rows contiguous (lane = channel)
 __host__ __device__ __forceinline__ bool ws_by_rows(const ffk_tile& t) {
     return t.kind == FFK_TILE_QK || t.kind == FFK_TILE_ACC || (t.kind == FFK_TILE_STRIDED && t.s_d == 1);
@@ -101,12 +105,18 @@ __device__ __forceinline__ void unpack8(const T* p, float* f) {
     for (int e = 0; e < 8; ++e) f[e] = (float)h[e];
 }
 
+// Two forms of each epilogue.  The "compact" one funnels every bias / activation / scale combination
+// through one intermediate array; the other gives each combination its own straight-line path from the
+// accumulators to the rounded outputs, which executes about 30 vector instructions fewer per 32x32 block
+// (no register copies where paths join, no cleared gate accumulator for plain units) but needs more
+// registers.  The kernel variants with three or four weight slots or K = 256 have no registers to spare -
+// there the second form spills, and a spill costs far more than it saves - so they keep the compact form.
 // ---- lane = row (n32 = its row within the group), registers = channels -----------------------
 // STRIDED tiles: weight rows were loaded through tau, registers hold channels 16*half + v.
 // ACC / QK tiles: natural weight order, registers hold channels 8a + 4*half + b.
 // sb: this slot's 32 (GLU: 64) bias values in LDS (fp32); rmask: the row's mask value.
 template <bool GLU>
-__device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+__device__ __forceinline__ void ws_store_rows_compact(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
                                               bool valid, unsigned mc, unsigned hi, unsigned lo, float rmask, int half) {
     const bool strided = t.kind == FFK_TILE_STRIDED;
     float x[16];
@@ -199,7 +209,7 @@ __device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc
 // 16*half + v: sixteen consecutive rows, which never straddle `inner` (inner % 16 == 0, M % 16 == 0).
 // sm: mask values (fp32, LDS) of the group's 32 rows, or nullptr.
 template <bool GLU>
-__device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+__device__ __forceinline__ void ws_store_cols_compact(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
                                               const float* sm, long m0g, int M, int l32, int half) {
     const float bv = sb[l32], bg = GLU ? sb[32 + l32] : 0.0f;
     float x[16];
@@ -258,6 +268,166 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
     }
 }
 
+// ---- lane = row (n32 = its row within the group), registers = channels -----------------------
+// STRIDED tiles: weight rows were loaded through tau, registers hold channels 16*half + v.
+// ACC / QK tiles: natural weight order, registers hold channels 8a + 4*half + b.
+// sb: this slot's 32 (GLU: 64) bias values in LDS (fp32); rmask: the row's mask value.
+template <bool GLU>
+__device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+                                              bool valid, unsigned mc, unsigned hi, unsigned lo, float rmask, int half) {
+    const bool strided = t.kind == FFK_TILE_STRIDED;
+    // Every combination of bias / activation / scale is its own straight-line path from the accumulators
+    // to the rounded outputs: a shared intermediate array makes the compiler copy the 16 registers where
+    // the paths join, and the vector instruction count is what this kernel's time follows.
+    T y[16];
+    const bool scaled = t.masked || t.scale != 1.0f;
+    const float scl = t.scale * rmask;
+    auto emit = [&](auto value) {
+        if (scaled) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = (T)(value(v) * scl);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = (T)value(v);
+        }
+    };
+    if (GLU || t.has_bias || t.act == FFK_ACT_SIGMOID) {
+        f32x4 bv[4], bg[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int o = strided ? 16 * half + 4 * a : 4 * half + 8 * a;
+            bv[a] = *reinterpret_cast<const f32x4*>(sb + o);
+            if (GLU) bg[a] = *reinterpret_cast<const f32x4*>(sb + 32 + o);
+        }
+        if (GLU) {
+            emit([&](int v) { return (acc[v] + bv[v >> 2][v & 3]) * ws_sigmoid_pre(accg[v], bg[v >> 2][v & 3]); });
+        } else if (t.act == FFK_ACT_SIGMOID) {
+            emit([&](int v) { return ws_sigmoid_pre(acc[v], bv[v >> 2][v & 3]); });
+        } else if (t.act == FFK_ACT_RELU) {
+            emit([&](int v) { return ws_relu(acc[v] + bv[v >> 2][v & 3]); });
+        } else {
+            emit([&](int v) { return acc[v] + bv[v >> 2][v & 3]; });
+        }
+    } else if (t.act == FFK_ACT_RELU) {
+        emit([&](int v) { return ws_relu(acc[v]); });
+    } else {
+        emit([&](int v) { return acc[v]; });
+    }
+
+    T* out = t.out;
+    if (t.kind == FFK_TILE_ACC) {
+        if (valid && t.ncols_left >= 32) {
+            T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + ((half * 32 + (lo & 31)) << 4);
+            *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+            *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+        }
+    } else if (t.kind == FFK_TILE_QK) {
+        if (valid && t.ncols_left >= 32) {
+            T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + (lo & 31) * 16 + 4 * half;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)      // d = 8a + 4 half + b  ->  (d >> 4) * 512 + n * 16 + (d & 15)
+                *reinterpret_cast<u32x2*>(p + (a >> 1) * 512 + (a & 1) * 8) = *reinterpret_cast<const u32x2*>(&y[4 * a]);
+        }
+    } else {
+        const int cl = 16 * half;                        // this lane's 16 channels, relative to the unit
+        const long off = (long)hi * t.s_o + (long)lo * t.s_i + cl;
+        const bool ok0 = valid && cl + 8 <= t.ncols_left, ok1 = valid && cl + 16 <= t.ncols_left;
+        if (t.gate || t.resid) {
+            // every load first (clamped, unconditional), then combine and store
+            u32x4 gv[2], rv[2];
+            const T* gate = t.gate ? t.gate + (long)(t.gate_rows ? mc % t.gate_rows : mc) * t.gate_ld + cl : nullptr;
+            const T* resid = t.resid ? t.resid + off : nullptr;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int cj = cl + 8 * j + 8 <= t.ncols_left ? 8 * j : (cl + 8 <= t.ncols_left ? 0 : -cl);
+                if (gate) gv[j] = *reinterpret_cast<const u32x4*>(gate + cj);
+                if (resid) rv[j] = *reinterpret_cast<const u32x4*>(resid + cj);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const T* gh = reinterpret_cast<const T*>(&gv[j]);
+                const T* rh = reinterpret_cast<const T*>(&rv[j]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float f = (float)y[8 * j + e];
+                    if (gate) f = (float)(T)(f * (float)gh[e]);
+                    if (resid) f += (float)rh[e];
+                    y[8 * j + e] = (T)f;
+                }
+            }
+        }
+        if (ok0) *reinterpret_cast<u32x4*>(out + off) = *reinterpret_cast<const u32x4*>(&y[0]);
+        if (ok1) *reinterpret_cast<u32x4*>(out + off + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+    }
+}
+
+// ---- lane = channel, registers = rows ----------------------------------------------------------
+// V tiles: natural row order (registers hold rows 8a + 4*half + b of the group).
+// STRIDED (channel-major) tiles: the A fragments were loaded through tau, registers hold rows
+// 16*half + v: sixteen consecutive rows, which never straddle `inner` (inner % 16 == 0, M % 16 == 0).
+// sm: mask values (fp32, LDS) of the group's 32 rows, or nullptr.
+template <bool GLU>
+__device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+                                              const float* sm, long m0g, int M, int l32, int half) {
+    const float bv = sb[l32], bg = GLU ? sb[32 + l32] : 0.0f;
+    float x[16];
+    if (GLU) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = (acc[v] + bv) * ws_sigmoid_pre(accg[v], bg);
+    } else if (t.act == FFK_ACT_SIGMOID) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = ws_sigmoid_pre(acc[v], bv);
+    } else if (t.act == FFK_ACT_RELU) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = ws_relu(acc[v] + bv);
+    } else if (t.has_bias) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = acc[v] + bv;
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = acc[v];
+    }
+
+    T* out = t.out;
+    const bool vt = t.kind == FFK_TILE_V;
+    const long mr = vt ? m0g : m0g + 16 * half;          // V: the group is one whole key tile (inner % 32 == 0)
+    const bool ok = mr < M;
+    const unsigned mc = (unsigned)(ok ? mr : 0);
+    unsigned hi = 0, lo = mc;
+    if (t.inner < (unsigned)M) {
+        hi = mc / t.inner;
+        lo = mc - hi * t.inner;
+    }
+    // the mask multiply is skipped for row groups without a masked row (the common case)
+    if (sm && !vt && __builtin_amdgcn_ballot_w64(sm[l32] != 1.0f) != 0) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const f32x4 mk = *reinterpret_cast<const f32x4*>(sm + 16 * half + 4 * a);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) x[4 * a + b] *= mk[b];
+        }
+    }
+    T y[16];
+    if (t.scale != 1.0f) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)(x[v] * t.scale);
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[v] = (T)x[v];
+    }
+    if (vt) {
+        if (ok && t.ncols_left >= 32) {
+            T* p = out + (long)hi * t.s_o + (long)(lo >> 5) * 1024 + ((half * 32 + l32) << 4);
+            *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+            *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+        }
+    } else if (ok && l32 < t.ncols_left) {
+        T* p = out + (long)hi * t.s_o + lo + (long)l32 * t.s_d;
+        *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
+        *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+    }
+}
+
 // DUAL: the gate halves of the GLU units multiply a second operand (row-major rows, own LayerNorm).  Its
 // slab goes from global memory straight into LDS (unpadded 256-byte rows, 16-byte columns XOR-swizzled
 // with the row index) one slab ahead and is normalised in place by the threads that requested it.
@@ -267,6 +437,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     typedef WsGeo<WS_K> G;
     constexpr int WS_KS = G::KS, WS_AP = G::AP, WS_BM = G::BM, WS_RG = G::RG, LPR = G::LPR, RPP = G::RPP;
     constexpr bool ALLOW_GLU = NS >= 2 && WS_K <= 128;
+    constexpr bool LEAN = NS == 2 && WS_K <= 128 && !DUAL;   // straight-line epilogues where the registers allow them
     constexpr int AFC = WS_K == 128 ? 8 : 4;               // A fragments held at a time (register budget)
     const ffk_linear_desc& d = args.d;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -530,62 +701,138 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                 // reload with a full vector-memory wait into every epilogue.
                 int reread = 0;
                 asm volatile("" : "+v"(reread));                   // opaque zero: keeps the compiler from reusing the loads
-                f32x16 acc, accg;
+                if constexpr (LEAN) {
+                    const bool rows = by_rows[s];
+                    // One straight-line body per (store order, GLU or not): the gate accumulator only exists
+                    // where it is used, and no accumulator has to be copied or cleared where paths would join.
+                    auto slot_body = [&](auto rows_tag, auto glu_tag) {
+                        constexpr bool ROWS = decltype(rows_tag)::value, G = decltype(glu_tag)::value;
+                        f32x16 acc, accg;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
-                const bool rows = by_rows[s];
-                if (DUAL && ALLOW_GLU && glu) {
-                    // gate half: fragments of the second operand's row (row % 16 == l32 % 16 picks the swizzle)
-                    const unsigned a2row = (unsigned)(buf * (WS_BM * 256) + (rg * 32 + n32) * 256 + ((half ^ (n32 & 15)) << 4));
+                        for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+                        if (G) {
 #pragma unroll
-                    for (int k0 = 0; k0 < WS_KS; k0 += AFC) {
-                        bf16x8 af[AFC];
+                            for (int v = 0; v < 16; ++v) accg[v] = 0.0f;
+                        }
+                        if (DUAL && G) {
+                            // gate half: fragments of the second operand's row (row % 16 == l32 % 16 picks the swizzle)
+                            const unsigned a2row = (unsigned)(buf * (WS_BM * 256) + (rg * 32 + n32) * 256 + ((half ^ (n32 & 15)) << 4));
 #pragma unroll
-                        for (int ks = 0; ks < AFC; ++ks)
-                            af[ks] = *reinterpret_cast<const bf16x8*>(s_a2 + ((a2row + reread) ^ (unsigned)((k0 + ks) * 32)));
+                            for (int k0 = 0; k0 < WS_KS; k0 += AFC) {
+                                bf16x8 af[AFC];
 #pragma unroll
-                        for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
+                                for (int ks = 0; ks < AFC; ++ks)
+                                    af[ks] = *reinterpret_cast<const bf16x8*>(s_a2 + ((a2row + reread) ^ (unsigned)((k0 + ks) * 32)));
+#pragma unroll
+                                for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
+                            }
+                        }
+#pragma unroll
+                        for (int k0 = 0; k0 < WS_KS; k0 += AFC) {          // AFC K steps of A in registers at a time
+                            bf16x8 af[AFC];
+#pragma unroll
+                            for (int ks = 0; ks < AFC; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + (k0 + ks) * 32);
+                            if (ROWS) {
+#pragma unroll
+                                for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, wf[s][k0 + ks], af[ks]);
+                                if (!DUAL && G) {
+#pragma unroll
+                                    for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
+                                }
+                            } else {
+#pragma unroll
+                                for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, af[ks], wf[s][k0 + ks]);
+                                if (G) {
+#pragma unroll
+                                    for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, af[ks], wf[sg][k0 + ks]);
+                                }
+                            }
+                        }
+                        if (ROWS) {
+                            if (t.inner != c_inner) {
+                                c_inner = t.inner;
+                                if (c_inner < (unsigned)M) {
+                                    c_hi = mc / c_inner;
+                                    c_lo = mc - c_hi * c_inner;
+                                } else {
+                                    c_hi = 0;
+                                    c_lo = mc;
+                                }
+                            }
+                            const float rmask = t.masked ? smk[n32] : 1.0f;
+                            ws_store_rows<G>(t, acc, G ? accg : acc, sb, valid, mc, c_hi, c_lo, rmask, half);
+                        } else {
+                            const float* sm = t.masked ? smk : nullptr;
+                            ws_store_cols<G>(t, acc, G ? accg : acc, sb, sm, m0g, M, l32, half);
+                        }
+                    };
+                    typedef std::integral_constant<bool, true> Yes;
+                    typedef std::integral_constant<bool, false> No;
+                    if (ALLOW_GLU && glu) {
+                        if (rows) slot_body(Yes(), Yes());
+                        else slot_body(No(), Yes());
+                    } else {
+                        if (rows) slot_body(Yes(), No());
+                        else slot_body(No(), No());
                     }
-                }
+                } else {
+                    f32x16 acc, accg;
 #pragma unroll
-                for (int k0 = 0; k0 < WS_KS; k0 += AFC) {          // AFC K steps of A in registers at a time
-                    bf16x8 af[AFC];
+                    for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
+                    const bool rows = by_rows[s];
+                    if (DUAL && ALLOW_GLU && glu) {
+                        // gate half: fragments of the second operand's row (row % 16 == l32 % 16 picks the swizzle)
+                        const unsigned a2row = (unsigned)(buf * (WS_BM * 256) + (rg * 32 + n32) * 256 + ((half ^ (n32 & 15)) << 4));
 #pragma unroll
-                    for (int ks = 0; ks < AFC; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + (k0 + ks) * 32);
-                    if (rows) {
+                        for (int k0 = 0; k0 < WS_KS; k0 += AFC) {
+                            bf16x8 af[AFC];
 #pragma unroll
-                        for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, wf[s][k0 + ks], af[ks]);
-                        if (!DUAL && ALLOW_GLU && glu) {
+                            for (int ks = 0; ks < AFC; ++ks)
+                                af[ks] = *reinterpret_cast<const bf16x8*>(s_a2 + ((a2row + reread) ^ (unsigned)((k0 + ks) * 32)));
 #pragma unroll
                             for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
                         }
-                    } else {
-#pragma unroll
-                        for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, af[ks], wf[s][k0 + ks]);
-                        if (ALLOW_GLU && glu) {
-#pragma unroll
-                            for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, af[ks], wf[sg][k0 + ks]);
-                        }
                     }
-                }
-                if (rows) {
-                    if (t.inner != c_inner) {
-                        c_inner = t.inner;
-                        if (c_inner < (unsigned)M) {
-                            c_hi = mc / c_inner;
-                            c_lo = mc - c_hi * c_inner;
+#pragma unroll
+                    for (int k0 = 0; k0 < WS_KS; k0 += AFC) {          // AFC K steps of A in registers at a time
+                        bf16x8 af[AFC];
+#pragma unroll
+                        for (int ks = 0; ks < AFC; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + (k0 + ks) * 32);
+                        if (rows) {
+#pragma unroll
+                            for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, wf[s][k0 + ks], af[ks]);
+                            if (!DUAL && ALLOW_GLU && glu) {
+#pragma unroll
+                                for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
+                            }
                         } else {
-                            c_hi = 0;
-                            c_lo = mc;
+#pragma unroll
+                            for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, af[ks], wf[s][k0 + ks]);
+                            if (ALLOW_GLU && glu) {
+#pragma unroll
+                                for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, af[ks], wf[sg][k0 + ks]);
+                            }
                         }
                     }
-                    const float rmask = t.masked ? smk[n32] : 1.0f;
-                    if (ALLOW_GLU && glu) ws_store_rows<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
-                    else ws_store_rows<false>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
-                } else {
-                    const float* sm = t.masked ? smk : nullptr;
-                    if (ALLOW_GLU && glu) ws_store_cols<true>(t, acc, accg, sb, sm, m0g, M, l32, half);
-                    else ws_store_cols<false>(t, acc, accg, sb, sm, m0g, M, l32, half);
+                    if (rows) {
+                        if (t.inner != c_inner) {
+                            c_inner = t.inner;
+                            if (c_inner < (unsigned)M) {
+                                c_hi = mc / c_inner;
+                                c_lo = mc - c_hi * c_inner;
+                            } else {
+                                c_hi = 0;
+                                c_lo = mc;
+                            }
+                        }
+                        const float rmask = t.masked ? smk[n32] : 1.0f;
+                        if (ALLOW_GLU && glu) ws_store_rows_compact<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                        else ws_store_rows_compact<false>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                    } else {
+                        const float* sm = t.masked ? smk : nullptr;
+                        if (ALLOW_GLU && glu) ws_store_cols_compact<true>(t, acc, accg, sb, sm, m0g, M, l32, half);
+                        else ws_store_cols_compact<false>(t, acc, accg, sb, sm, m0g, M, l32, half);
+                    }
                 }
             }
         }
