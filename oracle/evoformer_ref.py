@@ -11,9 +11,14 @@ it is the mathematics of the eval-mode forward pass only (dropout = identity).
 Pinning (what each part is checked against, see tests/test_oracle.py):
   * Attention, LayerNorm, Linear, softmax      library routines / float64 brute force
   * tri-mul / OPM contractions                 einsum forms + triple-loop brute force
-  * composition of a block                     golden vectors written by importing the
+  * composition of a block (Evoformer,
+    extra-MSA, template pair stack)            golden vectors written by importing the
                                                reference's fastfold.model.nn in the
                                                build container (tests/golden/)
+  * global attention                           float64 loops over the published formula
+  * input / recycling embedders                float64 loops (a Linear on a one-hot vector is a
+                                               column pick); no golden vectors: the reference's
+                                               nn/embedders.py needs dm-tree, absent here
   * identity at default init, permutation
     equivariance, masked-key invariance        mathematical invariants
 """
