@@ -145,7 +145,7 @@ class LinearDesc(ctypes.Structure):
         ("a_inner", c_int), ("a_chanmajor", c_int),
         ("ln_gamma", c_void_p), ("ln_beta", c_void_p), ("ln_eps", c_float), ("dtype", c_int),
         ("w", c_void_p),
-        ("M", c_int), ("K", c_int), ("n_tiles", c_int), ("reserved", c_int),
+        ("M", c_int), ("K", c_int), ("n_tiles", c_int), ("ln_folded", c_int),
         ("a2", c_void_p), ("ln2_gamma", c_void_p), ("ln2_beta", c_void_p),
         ("a2_so", c_int64), ("a2_si", c_int64), ("a2_inner", c_int), ("reserved2", c_int),
         ("tiles", Tile * FFK_MAX_TILES),
@@ -171,10 +171,13 @@ def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, g
 
 
 def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanmajor=False, a_cs=0,
-                 ln=None, eps=1e-5, a_off=0, w_row_off=0, a2=None, ln2=None, a2_inner=None, a2_so=0, a2_si=None):
+                 ln=None, eps=1e-5, a_off=0, w_row_off=0, a2=None, ln2=None, a2_inner=None, a2_so=0, a2_si=None,
+                 ln_rowsums=None):
     """Launches ``ffk_fused_linear``.  ``a`` / ``w`` are tensors (``w`` packed [>= n_tiles*128, K]);
     ``ln`` is ``(gamma, beta)`` or None; ``a_off`` (elements) / ``w_row_off`` (rows) offset the bases.
-    ``a2`` / ``ln2`` give the second operand the gate halves of GLU tiles are computed from."""
+    ``a2`` is the second operand the gate halves of GLU tiles are computed from; it goes with ``ln_rowsums``
+    (fp32 [n_tiles * 128]) instead of ``ln``: both LayerNorms folded into ``w`` and the tile biases
+    (``ln_folded`` in include/ffk.h).  ``ln2`` is accepted for symmetry and ignored."""
     d = LinearDesc()
     d.a = a.data_ptr() + a_off * a.element_size()
     d.a_inner = M if a_inner is None else a_inner
@@ -184,12 +187,18 @@ def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanma
     d.a_chanmajor = 1 if a_chanmajor else 0
     if ln is not None:
         d.ln_gamma, d.ln_beta = ln[0].data_ptr(), ln[1].data_ptr()
+    if ln_rowsums is not None:
+        if ln is not None or ln_rowsums.dtype != torch.float32 or ln_rowsums.numel() < 128 * len(tiles):
+            raise RuntimeError("fused_linear: ln_rowsums must be fp32 [n_tiles * 128] and excludes ln")
+        d.ln_gamma, d.ln_folded = ln_rowsums.data_ptr(), 1
     d.ln_eps = eps
     d.dtype = dtype_tag(a.dtype)
     d.w = w.data_ptr() + w_row_off * K * w.element_size()
     d.M, d.K, d.n_tiles = M, K, len(tiles)
     if a2 is not None:
-        d.a2, d.ln2_gamma, d.ln2_beta = a2.data_ptr(), ln2[0].data_ptr(), ln2[1].data_ptr()
+        if ln_rowsums is None:
+            raise RuntimeError("fused_linear: a second operand needs folded LayerNorms (ln_rowsums)")
+        d.a2 = a2.data_ptr()
         d.a2_inner = M if a2_inner is None else a2_inner
         d.a2_so = a2_so
         d.a2_si = K if a2_si is None else a2_si

@@ -476,12 +476,13 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
     if (!d->a_chanmajor)
         FFK_REQUIRE((d->a_so * es) % 16 == 0 && (d->a_si * es) % 16 == 0, FFK_ERR_ALIGN,
                     "ffk_fused_linear: row strides of A must be multiples of 16 bytes");
-    FFK_REQUIRE(!d->ln_gamma || d->ln_beta, FFK_ERR_NULL, "ffk_fused_linear: ln_beta missing");
+    FFK_REQUIRE(d->ln_folded || !d->ln_gamma || d->ln_beta, FFK_ERR_NULL, "ffk_fused_linear: ln_beta missing");
+    FFK_REQUIRE((d->ln_folded != 0) == (d->a2 != nullptr), FFK_ERR_UNSUPPORTED,
+                "ffk_fused_linear: the second operand and folded LayerNorms (ln_folded) go together");
     if (d->a2) {
-        FFK_REQUIRE(d->ln2_gamma && d->ln2_beta, FFK_ERR_NULL, "ffk_fused_linear: the second operand needs ln2_gamma / ln2_beta");
+        FFK_REQUIRE(d->ln_gamma, FFK_ERR_NULL, "ffk_fused_linear: folded LayerNorms need the row-sum table in ln_gamma");
         FFK_REQUIRE(d->a2_inner > 0, FFK_ERR_SHAPE, "ffk_fused_linear: a2_inner must be positive");
-        FFK_REQUIRE(ffk_aligned16(d->a2) && ffk_aligned16(d->ln2_gamma) && ffk_aligned16(d->ln2_beta) &&
-                        (d->a2_so * es) % 16 == 0 && (d->a2_si * es) % 16 == 0,
+        FFK_REQUIRE(ffk_aligned16(d->a2) && (d->a2_so * es) % 16 == 0 && (d->a2_si * es) % 16 == 0,
                     FFK_ERR_ALIGN, "ffk_fused_linear: rows of the second operand must be 16-byte aligned");
     }
     for (int i = 0; i < d->n_tiles; ++i) {

@@ -428,6 +428,49 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
     }
 }
 
+// GLU unit of a [row][channel] tile of a second-operand launch, where both LayerNorms are folded into the
+// weights (see a2 in include/ffk.h): with W' = W * gamma the normalised product is
+//     W LN(x) + b = rstd * (W' x - mean * c1) + c2,   c1[n] = sum_k W'[n][k],  c2[n] = sum_k W[n][k] beta[k] + b[n],
+// so the slab needs no normalisation pass at all: mean and rstd of the lane's row come from the fragments the
+// products use, c2 sits in the bias table, c1 in a table of its own; the gate half does the same with the
+// second operand's row.  out = resid + value * sigmoid(gate), rounded once.  sb / sc1: this unit's 64 bias
+// values / 64 row sums in LDS (fp32), value half first.
+__device__ __forceinline__ void ws_store_rows_folded(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
+                                                     const float* sc1, float rstd, float nmr, float rstd_g, float nmr_g,
+                                                     bool valid, unsigned hi, unsigned lo, int half) {
+    // rstd_g / nmr_g (the second operand's statistics) arrive multiplied by -log2(e), as the gate's bias table is
+    f32x4 bv[4], bg[4], cv[4], cg[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int o = 16 * half + 4 * a;
+        bv[a] = *reinterpret_cast<const f32x4*>(sb + o);
+        bg[a] = *reinterpret_cast<const f32x4*>(sb + 32 + o);
+        cv[a] = *reinterpret_cast<const f32x4*>(sc1 + o);
+        cg[a] = *reinterpret_cast<const f32x4*>(sc1 + 32 + o);
+    }
+    const int cl = 16 * half;
+    const long off = (long)hi * t.s_o + (long)lo * t.s_i + cl;
+    u32x4 rv[2];
+    if (t.resid) {
+        rv[0] = *reinterpret_cast<const u32x4*>(t.resid + off);
+        rv[1] = *reinterpret_cast<const u32x4*>(t.resid + off + 8);
+    }
+    T y[16];
+    const T* rh = reinterpret_cast<const T*>(&rv[0]);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const float val = __builtin_fmaf(acc[v], rstd, __builtin_fmaf(cv[v >> 2][v & 3], nmr, bv[v >> 2][v & 3]));
+        const float garg = __builtin_fmaf(accg[v], rstd_g, __builtin_fmaf(cg[v >> 2][v & 3], nmr_g, bg[v >> 2][v & 3]));
+        float x = val * fast_rcp(1.0f + fast_exp2(garg));
+        if (t.resid) x += (float)rh[v];
+        y[v] = (T)x;
+    }
+    if (valid) {
+        *reinterpret_cast<u32x4*>(t.out + off) = *reinterpret_cast<const u32x4*>(&y[0]);
+        *reinterpret_cast<u32x4*>(t.out + off + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
+    }
+}
+
 // DUAL: the gate halves of the GLU units multiply a second operand (row-major rows, own LayerNorm).  Its
 // slab goes from global memory straight into LDS (unpadded 256-byte rows, 16-byte columns XOR-swizzled
 // with the row index) one slab ahead and is normalised in place by the threads that requested it.
@@ -450,6 +493,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     float* s_cmln = reinterpret_cast<float*>(s_a2 + (DUAL ? 2 * WS_BM * 256 : 0));          // CM: gamma[128], beta[128] (fp32)
     T* s_ln2 = reinterpret_cast<T*>(s_cmln + (CM ? 256 : 0));                               // DUAL: gamma2[128], beta2[128]
     T* s_ln1 = s_ln2 + (DUAL ? 256 : 0);                                                    // !CM: gamma[K], beta[K]
+    float* s_c1 = reinterpret_cast<float*>(s_ln1 + (CM ? 0 : 2 * WS_K));                    // DUAL: folded LayerNorm row sums
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
@@ -509,8 +553,14 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 
     // ---- slab streaming: thread -> (row tid / LPR + RPP * i, 8 channels starting at 8 * (tid % LPR)) ----
     const int c8 = tid % LPR, r0 = tid / LPR;
-    const bool ln = d.ln_gamma != nullptr;
+    // DUAL launches carry both LayerNorms folded into the weights: ln_gamma is the fp32 table of row sums and
+    // both slabs are used as they arrive (see ws_store_rows_folded)
+    const bool folded = DUAL;
+    const bool ln = d.ln_gamma != nullptr && !folded;
     {
+        if (folded) {
+            for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) s_c1[i] = ((const float*)d.ln_gamma)[i];
+        }
         if (ln && !CM && tid < WS_K) {
             s_ln1[tid] = ((const T*)d.ln_gamma)[tid];
             s_ln1[WS_K + tid] = ((const T*)d.ln_beta)[tid];
@@ -518,10 +568,6 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         if (ln && CM && tid < 128) {
             s_cmln[tid] = (float)((const T*)d.ln_gamma)[tid];
             s_cmln[128 + tid] = (float)((const T*)d.ln_beta)[tid];
-        }
-        if (DUAL && tid < 128) {
-            s_ln2[tid] = ((const T*)d.ln2_gamma)[tid];
-            s_ln2[128 + tid] = ((const T*)d.ln2_beta)[tid];
         }
         lds_barrier();
     }
@@ -579,34 +625,16 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     };
     auto commit = [&](int buf) {
         unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
-        if (DUAL) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's vectors of the second operand have landed
-            const Vec16<T> gam2 = *reinterpret_cast<const Vec16<T>*>(s_ln2 + a2_col * 8);
-            const Vec16<T> bet2 = *reinterpret_cast<const Vec16<T>*>(s_ln2 + 128 + a2_col * 8);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                Vec16<T>* px = reinterpret_cast<Vec16<T>*>(s_a2 + buf * (WS_BM * 256) + (i * WS_THREADS + tid) * 16);
-                Vec16<T> x = *px;
-                float f[8], sm = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    f[e] = (float)x.e[e];
-                    sm += f[e];
-                }
-                const float mu = group_sum(sm, 16) * (1.0f / WS_K);
-                float q = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    f[e] -= mu;
-                    q += f[e] * f[e];
-                }
-                const float rs = rsqrtf(group_sum(q, 16) * (1.0f / WS_K) + d.ln_eps);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) x.e[e] = (T)(f[e] * rs * (float)gam2.e[e] + (float)bet2.e[e]);
-                *px = x;
-            }
-        }
+        if (DUAL) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's vectors of the second operand have landed
         if (CM) {
+            if (!ln) {       // nothing to normalise here: the transposition is a plain copy
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        *reinterpret_cast<T*>(sa + (cm_mg * 8 + j) * WS_AP + (cm_k + 32 * i) * 2) = pre[i].e[j];
+                return;
+            }
             float f[4][8];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -779,6 +807,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                     f32x16 acc, accg;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) acc[v] = accg[v] = 0.0f;
+                    float st1 = 0.0f, st2 = 0.0f, su1 = 0.0f, su2 = 0.0f;   // row statistics of the two operands (DUAL)
                     const bool rows = by_rows[s];
                     if (DUAL && ALLOW_GLU && glu) {
                         // gate half: fragments of the second operand's row (row % 16 == l32 % 16 picks the swizzle)
@@ -789,6 +818,18 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 #pragma unroll
                             for (int ks = 0; ks < AFC; ++ks)
                                 af[ks] = *reinterpret_cast<const bf16x8*>(s_a2 + ((a2row + reread) ^ (unsigned)((k0 + ks) * 32)));
+                            {
+                                typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                                const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+#pragma unroll
+                                for (int ks = 0; ks < AFC; ++ks)
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) {
+                                        const bf16x2 pr = {af[ks][2 * e], af[ks][2 * e + 1]};
+                                        su1 = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, su1, false);
+                                        su2 = __builtin_amdgcn_fdot2_f32_bf16(pr, pr, su2, false);
+                                    }
+                            }
 #pragma unroll
                             for (int ks = 0; ks < AFC; ++ks) MM::mma(accg, wf[sg][k0 + ks], af[ks]);
                         }
@@ -798,6 +839,19 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                         bf16x8 af[AFC];
 #pragma unroll
                         for (int ks = 0; ks < AFC; ++ks) af[ks] = *reinterpret_cast<const bf16x8*>(ap + reread + (k0 + ks) * 32);
+                        if (DUAL && folded) {
+                            // sum and sum of squares of this lane's half of its row, from the fragments themselves
+                            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                            const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+#pragma unroll
+                            for (int ks = 0; ks < AFC; ++ks)
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const bf16x2 pr = {af[ks][2 * e], af[ks][2 * e + 1]};
+                                    st1 = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, st1, false);
+                                    st2 = __builtin_amdgcn_fdot2_f32_bf16(pr, pr, st2, false);
+                                }
+                        }
                         if (rows) {
 #pragma unroll
                             for (int ks = 0; ks < AFC; ++ks) MM::mma(acc, wf[s][k0 + ks], af[ks]);
@@ -826,7 +880,18 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                             }
                         }
                         const float rmask = t.masked ? smk[n32] : 1.0f;
-                        if (ALLOW_GLU && glu) ws_store_rows_compact<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                        if (DUAL && folded) {
+                            st1 += lane_xor<32>(st1);
+                            st2 += lane_xor<32>(st2);
+                            const float mean = st1 * (1.0f / WS_K);
+                            const float rstd = rsqrtf(fmaxf(st2 * (1.0f / WS_K) - mean * mean, 0.0f) + d.ln_eps);
+                            su1 += lane_xor<32>(su1);
+                            su2 += lane_xor<32>(su2);
+                            const float mean_g = su1 * (1.0f / WS_K);
+                            const float rstd_g = -1.4426950408889634f * rsqrtf(fmaxf(su2 * (1.0f / WS_K) - mean_g * mean_g, 0.0f) + d.ln_eps);
+                            ws_store_rows_folded(t, acc, accg, sb, s_c1 + s_wrow[s], rstd, -rstd * mean, rstd_g, -rstd_g * mean_g,
+                                                 valid, c_hi, c_lo, half);
+                        } else if (ALLOW_GLU && glu) ws_store_rows_compact<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                         else ws_store_rows_compact<false>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                     } else {
                         const float* sm = t.masked ? smk : nullptr;
@@ -943,7 +1008,8 @@ template <int NS, int K, bool CM, bool DUAL = false>
 int ws_launch(const WsArgs& args, hipStream_t st) {
     constexpr int WS_BM = WsGeo<K>::BM;
     const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float) +
-                        (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) : 0) + (CM ? 256 * sizeof(float) : 2 * K * sizeof(T));
+                        (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) + FFK_MAX_TILES * 128 * sizeof(float) : 0) +
+                        (CM ? 256 * sizeof(float) : 2 * K * sizeof(T));
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K, CM, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -963,6 +1029,7 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
 // returns 1 with the launch status in *status; returns 0 if the caller has to use another variant.
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->dtype != FFK_BF16 || (d->K != 64 && d->K != 128 && d->K != 256)) return 0;
+    if ((d->ln_folded != 0) != (d->a2 != nullptr)) return 0;    // folded LayerNorms and the second operand go together
     if (d->a_chanmajor && (d->K != 128 || d->a_si != 1 || d->a_inner % 8 || d->a_so % 8 || d->a_cs % 8 || d->M % 8)) return 0;
     const bool k256 = d->K == 256;
     if (getenv("FFK_NO_WS")) return 0;
@@ -998,8 +1065,12 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->a2) {
         // second operand: every unit must be a GLU unit stored [row][channel], first operand channel-major
         if (!d->a_chanmajor || args.plan.max_slots > 2 || mask_tile >= 0 || d->a2_si % 8 || d->a2_so % 8) return 0;
-        for (int i = 0; i < d->n_tiles; ++i)
-            if (!d->tiles[i].glu || !ws_by_rows(d->tiles[i])) return 0;
+        for (int i = 0; i < d->n_tiles; ++i) {
+            const ffk_tile& t = d->tiles[i];
+            if (!t.glu || !ws_by_rows(t)) return 0;
+            // plain residual GLU tiles of 64 channels only
+            if (t.kind != FFK_TILE_STRIDED || t.gate || t.rowmask || t.scale != 1.0f || t.ncols != 64) return 0;
+        }
         *status = ws_launch<2, 128, true, true>(args, st);
     } else if (d->a_chanmajor) {
         if (args.plan.max_slots > 2 || mask_tile >= 0) return 0;

@@ -280,16 +280,27 @@ def pack_trimul(proj_w, proj_b, gate_w, gate_b, og_w, og_b, c, dtype, device):
     return torch.cat([w, wg], 0).contiguous(), torch.cat([b, bg], 0).contiguous(), n_glu
 
 
-def pack_trimul_out(out_w, out_b, og_w, og_b, C, dtype, device):
+def pack_trimul_out(out_w, out_b, og_w, og_b, C, dtype, device, ln_p, ln_z):
     """Output stage with the gate computed in the same launch: GLU tiles of 64 channels,
-    [Wout c0..c0+31 | Wog c0..c0+31 | Wout c0+32..c0+63 | Wog c0+32..c0+63] (biases alike)."""
-    ws, bs = [], []
+    [Wout c0..c0+31 | Wog c0..c0+31 | Wout c0+32..c0+63 | Wog c0+32..c0+63] (biases alike), with both
+    LayerNorms folded in: ``ln_p = (gamma, beta)`` of the contraction result into the value rows, ``ln_z`` of the
+    pair tensor into the gate rows (W' = W * gamma rounded to the kernel dtype, b' = W beta + b).  Returns
+    (weights, biases, fp32 row sums of W' in the same packed order)."""
+    def fold(w, b, ln):
+        w, b = w.detach().float(), b.detach().float()
+        gam, bet = ln[0].detach().float(), ln[1].detach().float()
+        wf = (w * gam[None, :]).to(dtype).float()
+        return wf, w @ bet + b, wf.sum(1)
+    out_w, out_b, out_rs = fold(out_w, out_b, ln_p)
+    og_w, og_b, og_rs = fold(og_w, og_b, ln_z)
+    ws, bs, cs = [], [], []
     for t in range(C // 64):
         for q in range(2):
             sl = slice(t * 64 + q * 32, t * 64 + q * 32 + 32)
             ws += [out_w[sl], og_w[sl]]
             bs += [out_b[sl], og_b[sl]]
-    return pack_rows(ws, dtype, device), pack_vec(bs, dtype, device)
+            cs += [out_rs[sl], og_rs[sl]]
+    return pack_rows(ws, dtype, device), pack_vec(bs, dtype, device), pack_vec(cs, torch.float32, device)
 
 
 def trimul_gate_in_output_stage(dtype, r, C, c):
@@ -334,11 +345,12 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
                   o_bs=r * kpad, s_i=kpad)
     del lr
     if dual:
-        wd, bd = dual_pk
+        wd, bd, rowsums = dual_pk
         tiles = [make_tile(out.data_ptr() + t * 64 * es, bias=bd.data_ptr() + t * 128 * es, glu=1, ncols=64,
                            resid=z.data_ptr() + t * 64 * es, inner=M, s_i=C) for t in range(C // 64)]
+        # both LayerNorms (of p and of z) are folded into the packed weights: no normalisation pass over either
         _lib.fused_linear(p, wd, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
-                          ln=ln2, a2=z, ln2=ln1, a2_inner=M, a2_si=C)
+                          ln_rowsums=rowsums, a2=z, a2_inner=M, a2_si=C)
         return out
     tiles = []
     for t in range((C + 127) // 128):

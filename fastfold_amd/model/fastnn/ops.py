@@ -8,6 +8,7 @@ lowers the scratch-memory budget of the launches, since attention logits and tra
 outer-product intermediates are already streamed.
 """
 import math
+import os
 
 import torch
 import torch.nn as nn
@@ -426,7 +427,8 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
             raise RuntimeError("TriangleMultiplication: unsupported widths %d / %d" % (C, self.c))
         ps = [self.left_right_projection.weight, self.left_right_projection.bias, self.left_right_gate.weight,
               self.left_right_gate.bias, self.output_gate.weight, self.output_gate.bias,
-              self.output_projection.weight, self.output_bias]
+              self.output_projection.weight, self.output_bias, self.layernorm2.weight, self.layernorm2.bias,
+              self.layernorm1.weight, self.layernorm1.bias]
 
         def build():
             w, b, n_glu = F_.pack_trimul(self.left_right_projection.weight, self.left_right_projection.bias,
@@ -435,7 +437,9 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
             dual = None
             if F_.trimul_gate_in_output_stage(dt, r, C, self.c):
                 dual = F_.pack_trimul_out(self.output_projection.weight, self.output_bias, self.output_gate.weight,
-                                          self.output_gate.bias, C, dt, dev)
+                                          self.output_gate.bias, C, dt, dev,
+                                          ln_p=(self.layernorm2.weight, self.layernorm2.bias),
+                                          ln_z=(self.layernorm1.weight, self.layernorm1.bias))
             return (w, b, n_glu, F_.pack_rows([self.output_projection.weight], dt, dev),
                     F_.pack_vec([self.output_bias], dt, dev), dual)
         w, b, n_glu, wout, bout, dual = self._packed(("tm", dt, dev, r % 8 == 0), ps, build)

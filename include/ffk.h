@@ -170,13 +170,22 @@ typedef struct ffk_linear_desc {
     float ln_eps;
     int32_t dtype;
     const void* w;         /* [n_tiles * 128, K] row-major, zero-padded rows */
-    int32_t M, K, n_tiles, reserved;
+    int32_t M, K, n_tiles;
+    /* ln_folded: 0, or 1 together with a second operand (a2, below): LayerNorms are then not applied to the
+       rows but folded into the weights.  For a row x of either operand with statistics (mean, rstd),
+           W LN(x) + b = rstd * (W' x - mean * rowsum(W')) + b',   W' = W * gamma,  b' = W beta + b,
+       so w holds W' (value rows: the first operand's gamma, gate rows: the second operand's), the tile
+       biases hold b', ln_gamma points to an fp32 table [n_tiles * 128] of the row sums of W' in packed tile
+       order and ln_beta / ln2_gamma / ln2_beta are ignored; the kernel takes mean and rstd of a row from the
+       operand fragments it multiplies anyway.  Tiles must be plain residual GLU tiles of 64 channels (no
+       gate pointer, no row mask, scale 1). */
+    int32_t ln_folded;
     /* Optional second operand (NULL = none): the gate halves of the GLU tiles are then computed from
-       LayerNorm(a2) with ln2_gamma / ln2_beta instead of from the first operand.  a2 is K-contiguous,
-       logical row m at  a2 + (m / a2_inner) * a2_so + (m % a2_inner) * a2_si.  Built for bf16, K = 128
-       and a channel-major first operand (the output stage of the triangle multiplication, whose gate
-       comes from the pair tensor and whose value from the contraction result); other combinations
-       return FFK_ERR_UNSUPPORTED. */
+       LayerNorm(a2) instead of from the first operand, both LayerNorms folded into the weights (ln_folded must
+       be 1).  a2 is K-contiguous, logical row m at  a2 + (m / a2_inner) * a2_so + (m % a2_inner) * a2_si.
+       Built for bf16, K = 128 and a channel-major first operand (the output stage of the triangle
+       multiplication, whose gate comes from the pair tensor and whose value from the contraction result);
+       other combinations return FFK_ERR_UNSUPPORTED. */
     const void* a2;
     const void* ln2_gamma;
     const void* ln2_beta;

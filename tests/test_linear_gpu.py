@@ -397,9 +397,11 @@ def test_transition_fused_kernel(dev, M):
 
 @pytest.mark.parametrize("r", [64, 104])
 def test_fused_linear_second_operand(dev, r):
-    """GLU tiles whose gate halves come from a second operand with its own LayerNorm (the output stage of the
-    triangle multiplication): out = resid + (W_p LN2(p) + b_p) * sigmoid(W_g LN1(z) + b_g), p channel-major."""
+    """GLU tiles whose gate halves come from a second operand (the output stage of the triangle multiplication):
+    out = resid + (W_p LN2(p) + b_p) * sigmoid(W_g LN1(z) + b_g), p channel-major, both LayerNorms folded into
+    the packed weights (statistics taken from the operand fragments inside the kernel)."""
     from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn import _fused as F_
     dtype = torch.bfloat16
     C, M = 128, r * r
     g = torch.Generator().manual_seed(r)
@@ -409,32 +411,37 @@ def test_fused_linear_second_operand(dev, r):
     bet1, bet2 = ((0.1 * torch.randn(C, generator=g)).to(dev, dtype) for _ in range(2))
     wp, wg = ((torch.randn(C, C, generator=g) / C ** 0.5).to(dev, dtype) for _ in range(2))
     bp, bg = (torch.randn(C, generator=g).to(dev, dtype) for _ in range(2))
-    ws, bs = [], []
-    for t in range(2):
-        for q in range(2):
-            sl = slice(t * 64 + q * 32, t * 64 + q * 32 + 32)
-            ws += [wp[sl], wg[sl]]
-            bs += [bp[sl], bg[sl]]
-    w_pk, b_pk = torch.cat(ws, 0).contiguous(), torch.cat(bs, 0).contiguous()
+    w_pk, b_pk, rowsums = F_.pack_trimul_out(wp, bp, wg, bg, C, dtype, dev, ln_p=(gam2, bet2), ln_z=(gam1, bet1))
     out = torch.empty(M, C, device=dev, dtype=dtype)
     tiles = [_lib.make_tile(out.data_ptr() + t * 64 * 2, bias=b_pk.data_ptr() + t * 128 * 2, glu=1, ncols=64,
                             resid=z.data_ptr() + t * 64 * 2, inner=M, s_i=C) for t in range(2)]
-    _lib.fused_linear(p_cm, w_pk, tiles, M=M, K=C, a_inner=r, a_so=r, a_si=1, a_chanmajor=True, a_cs=r * r,
-                      ln=(gam2, bet2), a2=z, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
-    pn = _np(torch.from_numpy(ops_np.layer_norm(_np(p_cm).reshape(C, M).T, _np(gam2), _np(bet2))).to(dtype))
-    zn = _np(torch.from_numpy(ops_np.layer_norm(_np(z), _np(gam1), _np(bet1))).to(dtype))
+    kw = dict(M=M, K=C, a_inner=r, a_so=r, a_si=1, a_chanmajor=True, a_cs=r * r, ln_rowsums=rowsums, a2_inner=M, a2_si=C)
+    _lib.fused_linear(p_cm, w_pk, tiles, a2=z, **kw)
+    pn = ops_np.layer_norm(_np(p_cm).reshape(C, M).T, _np(gam2), _np(bet2))
+    zn = ops_np.layer_norm(_np(z), _np(gam1), _np(bet1))
     upd = ops_np.linear(pn, _np(wp), _np(bp)) / (1 + np.exp(-ops_np.linear(zn, _np(wg), _np(bg))))
     assert _rel(_np(out) - _np(z), upd) < TOL[dtype]
     # in place on the second operand / residual
     z2 = z.clone()
     tiles = [_lib.make_tile(z2.data_ptr() + t * 64 * 2, bias=b_pk.data_ptr() + t * 128 * 2, glu=1, ncols=64,
                             resid=z2.data_ptr() + t * 64 * 2, inner=M, s_i=C) for t in range(2)]
-    _lib.fused_linear(p_cm, w_pk, tiles, M=M, K=C, a_inner=r, a_so=r, a_si=1, a_chanmajor=True, a_cs=r * r,
-                      ln=(gam2, bet2), a2=z2, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
+    _lib.fused_linear(p_cm, w_pk, tiles, a2=z2, **kw)
     assert torch.equal(z2, out)
-    # a second operand without the shapes it is built for is refused, not ignored
+    # rows with a large common offset: the folded form subtracts mean * rowsum after the product
+    p_off = (p_cm.float() + 40.0).to(dtype)
+    out3 = torch.empty_like(out)
+    tiles3 = [_lib.make_tile(out3.data_ptr() + t * 64 * 2, bias=b_pk.data_ptr() + t * 128 * 2, glu=1, ncols=64,
+                             resid=z.data_ptr() + t * 64 * 2, inner=M, s_i=C) for t in range(2)]
+    _lib.fused_linear(p_off, w_pk, tiles3, a2=z, **kw)
+    pn = ops_np.layer_norm(_np(p_off).reshape(C, M).T, _np(gam2), _np(bet2))
+    upd = ops_np.linear(pn, _np(wp), _np(bp)) / (1 + np.exp(-ops_np.linear(zn, _np(wg), _np(bg))))
+    assert _rel(_np(out3) - _np(z), upd) < TOL[dtype]
+    # a second operand without the shapes it is built for, or without folded LayerNorms, is refused, not ignored
     with pytest.raises(RuntimeError):
-        _lib.fused_linear(z, w_pk, tiles, M=M, K=C, ln=(gam2, bet2), a2=z, ln2=(gam1, bet1), a2_inner=M, a2_si=C)
+        _lib.fused_linear(z, w_pk, tiles, M=M, K=C, ln_rowsums=rowsums, a2=z, a2_inner=M, a2_si=C)
+    with pytest.raises(RuntimeError):
+        _lib.fused_linear(p_cm, w_pk, tiles, M=M, K=C, a_inner=r, a_so=r, a_si=1, a_chanmajor=True, a_cs=r * r,
+                          ln=(gam2, bet2), a2=z, a2_inner=M, a2_si=C)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
