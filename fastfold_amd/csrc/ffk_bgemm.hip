@@ -159,7 +159,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float x = acc[ni][mi][4 * g + e] + bv[ni][g][e];
-                    if (d.act == FFK_ACT_RELU) x = fmaxf(x, 0.0f);
+                    if (d.act == FFK_ACT_RELU) x = relu_f(x);
                     else if (d.act == FFK_ACT_SIGMOID) x = sigmoid_f(x);
                     dst[e] = DT<OT>::from_f(x * d.scale * rdiv);
                 }

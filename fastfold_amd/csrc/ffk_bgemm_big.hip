@@ -210,7 +210,7 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             for (int v = 0; v < 16; ++v) {
                 float x = acc[ni][mi][v];
                 if (bias) x += (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7];
-                if (d.act == FFK_ACT_RELU) x = fmaxf(x, 0.0f);
+                if (d.act == FFK_ACT_RELU) x = relu_f(x);
                 else if (d.act == FFK_ACT_SIGMOID) x = sigmoid_f(x);
                 x *= mul;
                 if (resid) x = (float)(T)x + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7];

@@ -146,6 +146,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // ------------------------------------------------------------ fast math ----
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// max(x, 0) in one instruction: fmaxf first canonicalises its argument (a second v_max) under IEEE rules
+__device__ __forceinline__ float relu_f(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, 3.0e38f); }
 __device__ __forceinline__ float sigmoid_f(float x) {
     // 1 / (1 + 2^(-x*log2e))
     return fast_rcp(1.0f + fast_exp2(-1.4426950408889634f * x));

@@ -79,7 +79,7 @@ __device__ __forceinline__ void stage_tile(const f32x16 (&acc)[CT], const T (&bv
                     const float gv = acc[ct | 1][4 * g + e] + DT<T>::to_f(bv[ct | 1][g][e]);
                     x = x * sigmoid_f(gv);
                 } else if (ACT == FFK_ACT_RELU) {
-                    x = fmaxf(x, 0.0f);
+                    x = relu_f(x);
                 } else if (ACT == FFK_ACT_SIGMOID) {
                     x = sigmoid_f(x);
                 }

@@ -77,9 +77,6 @@ __device__ __forceinline__ float ws_sigmoid_pre(float acc, float bs) {
     return fast_rcp(1.0f + fast_exp2(__builtin_fmaf(acc, -1.4426950408889634f, bs)));
 }
 
-// max(x, 0) as one instruction (fmaxf also canonicalises its argument first)
-__device__ __forceinline__ float ws_relu(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, 3.0e38f); }
-
 // tiles stored with channels contiguous (lane = row) vs rows contiguous (lane = channel)
 __host__ __device__ __forceinline__ bool ws_by_rows(const ffk_tile& t) {
     return t.kind == FFK_TILE_QK || t.kind == FFK_TILE_ACC || (t.kind == FFK_TILE_STRIDED && t.s_d == 1);
@@ -144,7 +141,7 @@ __device__ __forceinline__ void ws_store_rows_compact(const WsSlot& t, const f32
     }
     if (!GLU && t.act == FFK_ACT_RELU) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = fmaxf(x[v], 0.0f);
+        for (int v = 0; v < 16; ++v) x[v] = relu_f(x[v]);
     }
     T y[16];
     if (t.masked || t.scale != 1.0f) {
@@ -224,7 +221,7 @@ __device__ __forceinline__ void ws_store_cols_compact(const WsSlot& t, const f32
         for (int v = 0; v < 16; ++v) x[v] = acc[v] + bv;
         if (t.act == FFK_ACT_RELU) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) x[v] = fmaxf(x[v], 0.0f);
+            for (int v = 0; v < 16; ++v) x[v] = relu_f(x[v]);
         }
     }
 
@@ -304,12 +301,12 @@ __device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc
         } else if (t.act == FFK_ACT_SIGMOID) {
             emit([&](int v) { return ws_sigmoid_pre(acc[v], bv[v >> 2][v & 3]); });
         } else if (t.act == FFK_ACT_RELU) {
-            emit([&](int v) { return ws_relu(acc[v] + bv[v >> 2][v & 3]); });
+            emit([&](int v) { return relu_f(acc[v] + bv[v >> 2][v & 3]); });
         } else {
             emit([&](int v) { return acc[v] + bv[v >> 2][v & 3]; });
         }
     } else if (t.act == FFK_ACT_RELU) {
-        emit([&](int v) { return ws_relu(acc[v]); });
+        emit([&](int v) { return relu_f(acc[v]); });
     } else {
         emit([&](int v) { return acc[v]; });
     }
@@ -379,7 +376,7 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
         for (int v = 0; v < 16; ++v) x[v] = ws_sigmoid_pre(acc[v], bv);
     } else if (t.act == FFK_ACT_RELU) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = ws_relu(acc[v] + bv);
+        for (int v = 0; v < 16; ++v) x[v] = relu_f(acc[v] + bv);
     } else if (t.has_bias) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) x[v] = acc[v] + bv;
@@ -576,6 +573,8 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const T* rm = mt >= 0 ? (const T*)d.tiles[mt].rowmask : nullptr;
     const unsigned m_inner = mt >= 0 ? (unsigned)d.tiles[mt].inner : 1u;
     const long m_so = mt >= 0 ? d.tiles[mt].m_so : 0, m_si = mt >= 0 ? d.tiles[mt].m_si : 0;
+    // plain row-major operands (inner >= M) need no division per fetched vector
+    const bool a_flat = d.a_inner >= M, a2_flat = DUAL && d.a2_inner >= M, m_flat = m_inner >= (unsigned)M;
     Vec16<T> pre[4];
     T pm[4];
     // Channel-major A (element (m, k) at a + k * a_cs + rowoffset(m), K = 128): a thread fetches eight
@@ -593,7 +592,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             for (int i = 0; i < 4; ++i) {
                 long m = (long)slab * WS_BM + i * 32 + (tid >> 4);
                 m = m < M ? m : M - 1;
-                const unsigned hi = (unsigned)m / (unsigned)d.a2_inner, lo = (unsigned)m - hi * (unsigned)d.a2_inner;
+                const unsigned hi = a2_flat ? 0u : (unsigned)m / (unsigned)d.a2_inner, lo = (unsigned)m - hi * (unsigned)d.a2_inner;
                 const T* gp = (const T*)d.a2 + (long)hi * d.a2_so + (long)lo * d.a2_si + a2_col * 8;
                 const unsigned dst = lds_a2 + tobuf * (WS_BM * 256) + (i * WS_THREADS + wave * 64) * 16;
 #pragma clang diagnostic push
@@ -605,7 +604,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         if (CM) {
             long m = (long)slab * WS_BM + cm_mg * 8;
             m = m < M ? m : M - 8;                       // M % 8 == 0; clamped groups are never stored
-            const unsigned hi = (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
+            const unsigned hi = a_flat ? 0u : (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
             const T* base = A + (long)hi * d.a_so + lo;  // a_si == 1
 #pragma unroll
             for (int i = 0; i < 4; ++i) pre[i] = ld16(base + (long)(cm_k + 32 * i) * d.a_cs);
@@ -615,10 +614,10 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         for (int i = 0; i < 4; ++i) {
             long m = (long)slab * WS_BM + r0 + RPP * i;
             m = m < M ? m : M - 1;                       // clamped: rows past the end are never stored
-            const unsigned hi = (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
+            const unsigned hi = a_flat ? 0u : (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
             pre[i] = ld16(A + (long)hi * d.a_so + (long)lo * d.a_si + c8 * 8);
             if (rm) {
-                const unsigned mh = (unsigned)m / m_inner, ml = (unsigned)m - mh * m_inner;
+                const unsigned mh = m_flat ? 0u : (unsigned)m / m_inner, ml = (unsigned)m - mh * m_inner;
                 pm[i] = rm[(long)mh * m_so + (long)ml * m_si];
             }
         }

@@ -159,7 +159,7 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int t = 0; t < 8; ++t) hf[ht][j][t] = (T)fmaxf(h[8 * j + t], 0.0f);
+                for (int t = 0; t < 8; ++t) hf[ht][j][t] = (T)relu_f(h[8 * j + t]);
         }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
