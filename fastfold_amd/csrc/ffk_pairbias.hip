@@ -2,7 +2,7 @@
 //     bias_t[h][q/32][k/32][tile(k, q)] = scale * ( LayerNorm(z[q, k, :]) . w[h, :] )
 // written directly in the keys x queries operand tiles the attention kernel consumes.
 //
-// The op is a skinny projection (C = 128 channels -> H <= 8 heads) and purely HBM-bound (one read of
+// The op is a skinny projection (C = 128 or 64 channels -> H <= 8 heads) and purely HBM-bound (one read of
 // z).  One workgroup owns a 32 x 32 block of (q, k) and walks it in four 16 x 16 quarter blocks: the
 // 256 rows of a quarter are fetched with 16 lanes per row (coalesced 256-byte rows, 16 loads in
 // flight per thread, the next quarter's loads issued before this one is finished) into LDS.  The
@@ -147,7 +147,7 @@ extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, con
                              float eps, int dtype, void* stream) {
     FFK_REQUIRE(bias_t && z && scratch && (!w || (gamma && beta)), FFK_ERR_NULL, "ffk_pair_bias: null pointer");
     FFK_REQUIRE(dtype == FFK_BF16, FFK_ERR_DTYPE, "ffk_pair_bias: bf16 only (dtype tag %d)", dtype);
-    FFK_REQUIRE(C == 128, FFK_ERR_UNSUPPORTED, "ffk_pair_bias: built for 128 pair channels, got %ld", (long)C);
+    FFK_REQUIRE(C == 128 || C == 64, FFK_ERR_UNSUPPORTED, "ffk_pair_bias: built for 64 or 128 pair channels, got %ld", (long)C);
     FFK_REQUIRE(N > 0 && N <= 46340 && H > 0 && H <= PB_MAXH && a_inner > 0, FFK_ERR_SHAPE,
                 "ffk_pair_bias: bad shape N=%ld H=%ld a_inner=%ld", (long)N, (long)H, (long)a_inner);
     FFK_REQUIRE(ffk_aligned16(z) && ffk_aligned16(scratch) && a_so % 8 == 0 && a_si % 8 == 0, FFK_ERR_ALIGN,
@@ -161,16 +161,21 @@ extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, con
         int rc = ffk_check_launch("ffk_pair_bias");
         if (rc != FFK_OK) return rc;
     }
-    const size_t smem = 256 * (128 * 2 + 16) + 256 * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)pair_bias_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_pair_bias: cannot reserve LDS: %s", hipGetErrorString(e));
-        configured = true;
-    }
     const unsigned T = (unsigned)((N + 31) / 32);
-    pair_bias_kernel<128><<<dim3(T, T), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wop, c01, (int)N, (int)H,
-                                                                (int)a_inner, a_so, a_si, scale, eps);
+#define PB_LAUNCH(CC)                                                                                                   \
+    {                                                                                                                   \
+        const size_t smem = 256 * (CC * 2 + 16) + 256 * sizeof(float);                                                  \
+        static bool configured = false;                                                                                 \
+        if (!configured) {                                                                                              \
+            hipError_t e = hipFuncSetAttribute((const void*)pair_bias_kernel<CC>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                               (int)smem);                                                              \
+            if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_pair_bias: cannot reserve LDS: %s", hipGetErrorString(e)); \
+            configured = true;                                                                                          \
+        }                                                                                                               \
+        pair_bias_kernel<CC><<<dim3(T, T), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wop, c01, (int)N, \
+                                                                   (int)H, (int)a_inner, a_so, a_si, scale, eps);       \
+    }
+    if (C == 128) PB_LAUNCH(128) else PB_LAUNCH(64)
+#undef PB_LAUNCH
     return ffk_check_launch("ffk_pair_bias");
 }

@@ -222,7 +222,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     for t0 in range(0, len(tiles), per):
         _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
                           w_row_off=t0 * 128)
-    if bias_tile is not None and C == 128:      # the skinny bias projection has its own pass over x
+    if bias_tile is not None and C in (64, 128):      # the skinny bias projection has its own pass over x
         _pair_bias_launch(bias_t, x, ln, w_pk[4 * tpg * 128:], pb_scratch, N=N, C=C, H=H, a_inner=a_inner,
                           a_so=a_so, a_si=a_si, scale=LOG2E)
     elif bias_tile is not None:
@@ -251,7 +251,7 @@ def pair_bias(z, *, r, C, H, ln, wb_pk, pb_scratch=None):
     """bias_t[h][q/32][k/32][tile] = log2e * (LN(z)[q, k, :] . Wb[h, :]) in score-accumulator tiles."""
     NT = (r + 31) // 32
     bias_t = alloc((H, NT, NT, 1024), z.dtype, z.device, zero=(r % 32) != 0)
-    if z.dtype == torch.bfloat16 and C == 128 and H <= 8:
+    if z.dtype == torch.bfloat16 and C in (64, 128) and H <= 8:
         _pair_bias_launch(bias_t, z, ln, wb_pk, pb_scratch, N=r, C=C, H=H, a_inner=r * r, a_so=0, a_si=C, scale=LOG2E)
         return bias_t
     tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=r, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H, scale=LOG2E)

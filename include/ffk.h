@@ -265,7 +265,7 @@ int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v
  * zero-filled by the caller when N is not a multiple of 32; scratch is caller-owned device memory of
  * at least 16*C + 16 floats (the kernel builds its weight operand there; with w == NULL it uses the
  * operand a previous call with the same w, gamma, beta and scratch left there, gamma / beta may then be
- * NULL too).  bf16, C = 128.
+ * NULL too).  bf16, C = 128 or 64.
  * Replaces: F.linear(LayerNorm(Z), linear_b_weights) and its permute / unsqueeze
  * (fastfold/model/fastnn/msa.py:61-66, ops.py:659-664,890-896). */
 int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w,

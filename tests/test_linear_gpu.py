@@ -307,13 +307,13 @@ def test_weights_stationary_matches_other_variant(dev, monkeypatch):
         assert _rel(_np(a), _np(b)) < 1e-2
 
 
-@pytest.mark.parametrize("r,H", [(45, 4), (64, 8), (96, 4)])
-def test_pair_bias_kernel(dev, r, H):
+@pytest.mark.parametrize("r,H,C", [(45, 4, 128), (64, 8, 128), (96, 4, 128), (45, 4, 64), (64, 4, 64)])
+def test_pair_bias_kernel(dev, r, H, C):
     """ffk_pair_bias (bf16): LayerNorm + H-row projection written as attention bias tiles, in both
     traversal orders, against float64 numpy."""
     from fastfold_amd import _lib
     from fastfold_amd.model.fastnn.kernel import layouts
-    dtype, C = torch.bfloat16, 128
+    dtype = torch.bfloat16
     g = torch.Generator().manual_seed(r + H)
     z = (torch.randn(r, r, C, generator=g) * 1.5 + 0.4).to(dev, dtype)
     wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dev, dtype)
