@@ -172,6 +172,36 @@ def feeder_stacks(dev, r):
     return res
 
 
+def long_sequence(dev):
+    """BASELINE configs[4]: one block at N_seq = 64, N_res = 4096 (z = 4.3 GB), chunk size 64, in place; latency
+    and peak device memory."""
+    import torch
+    from fastfold_amd.model.fastnn import set_chunk_size
+    s, r = 64, 4096
+    stack = build_stack(1, dev, torch.bfloat16)
+    g = torch.Generator().manual_seed(2)
+    m = [torch.randn(s, r, 256, generator=g).to(dev, torch.bfloat16)]
+    z = [torch.randn(r, r, 128, generator=g).to(dev, torch.bfloat16)]
+    mm = torch.ones(s, r, device=dev, dtype=torch.bfloat16)
+    pm = torch.ones(r, r, device=dev, dtype=torch.bfloat16)
+    set_chunk_size(64)
+    try:
+        torch.cuda.reset_peak_memory_stats()
+        with torch.no_grad():
+            stack.inplace(m, z, mm, pm, chunk_size=64)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            stack.inplace(m, z, mm, pm, chunk_size=64)
+            torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3
+    finally:
+        set_chunk_size(None)
+    assert bool(torch.isfinite(z[0].float()).all())
+    return {"workload": "configs[4]: 1 block bf16 N_seq=64 N_res=4096, chunk_size=64, in place",
+            "ms_per_block": round(ms, 2), "block_tflop": round(block_gflop(s, r) / 1e3, 1),
+            "tflops": round(block_gflop(s, r) / ms, 1), "peak_device_GB": round(torch.cuda.max_memory_allocated() / 1e9, 1)}
+
+
 def cpu_baseline(threads):
     """The CPU oracle timed on the host cores: one fp32 block at N_seq=128, N_res=256."""
     import numpy as np
@@ -207,6 +237,8 @@ def main():
     ap.add_argument("--no-micro", action="store_true")
     ap.add_argument("--only-feeders", action="store_true",
                     help="time only the extra-MSA and template pair stacks (for profiling them on their own)")
+    ap.add_argument("--long-sequence", action="store_true",
+                    help="also time one block at N_res = 4096 (a few seconds and 26 GB of device memory more)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the Evoformer on ONE GPU (DAP size 1, no collectives); "
@@ -288,6 +320,9 @@ def main():
         del m3, z3, mm3, pm3
     del stack, out
     torch.cuda.empty_cache()
+    if args.long_sequence:
+        line["long_sequence"] = long_sequence(dev)
+        torch.cuda.empty_cache()
     if not args.no_micro:
         line["feeders"] = feeder_stacks(dev, r)
         line["ops"] = micro_ops(dev)
