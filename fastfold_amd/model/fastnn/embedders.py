@@ -1,5 +1,6 @@
 """Input and recycling embedders with the reference's interface (fastfold/model/fastnn/ops.py:1046-1145,
-1238-1334; the reference's ``inject_embedder`` swaps exactly these two, utils/inject_fastnn.py:376-416).
+1238-1334; the reference's ``inject_embedder`` swaps exactly these two, utils/inject_fastnn.py:376-416), and
+the three Linear-only feature embedders of fastnn/embedders.py:257-372 (template angle / pair, extra MSA).
 
 The r x r x c_z parts run in one launch of ``ffk_pair_embed`` each: a Linear on a one-hot vector is a pick of
 one weight column, so neither the [r, r, 65] relative-position one-hot nor the [r, r, 15] distogram one-hot
@@ -122,3 +123,46 @@ class RecyclingEmbedder(nn.Module, _PackMixin):
                         pos=x.to(torch.float32).contiguous(), edges=edges, inf=float(self.inf), r=z.shape[0],
                         C=self.c_z, nb=self.no_bins, ln_eps=self.layer_norm_z.eps)
         return m_update, out
+
+
+class TemplateAngleEmbedder(nn.Module):
+    """Embeds the "template_angle_feat" feature: Algorithm 2, line 7 (fastnn/embedders.py:257-297)."""
+
+    def __init__(self, c_in: int, c_out: int, **kwargs):
+        super(TemplateAngleEmbedder, self).__init__()
+        self.c_out = c_out
+        self.c_in = c_in
+        self.linear_1 = Linear(self.c_in, self.c_out, initializer="relu")
+        self.relu = nn.ReLU()
+        self.linear_2 = Linear(self.c_out, self.c_out, initializer="relu")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [*, N_templ, N_res, c_in] -> [*, N_templ, N_res, c_out]; the relu runs in the first launch's epilogue."""
+        return self.linear_2(self.linear_1(x, act=_lib.FFK_ACT_RELU))
+
+
+class TemplatePairEmbedder(nn.Module):
+    """Embeds "template_pair_feat" features: Algorithm 2, line 9 (fastnn/embedders.py:300-341)."""
+
+    def __init__(self, c_in: int, c_out: int, **kwargs):
+        super(TemplatePairEmbedder, self).__init__()
+        self.c_in = c_in
+        self.c_out = c_out
+        self.linear = Linear(self.c_in, self.c_out, initializer="relu")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.linear(x)
+
+
+class ExtraMSAEmbedder(nn.Module):
+    """Embeds unclustered MSA sequences: Algorithm 2, line 15 (fastnn/embedders.py:344-372)."""
+
+    def __init__(self, c_in: int, c_out: int, **kwargs):
+        super(ExtraMSAEmbedder, self).__init__()
+        self.c_in = c_in
+        self.c_out = c_out
+        self.linear = Linear(self.c_in, self.c_out)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [*, N_extra_seq, N_res, c_in] -> [*, N_extra_seq, N_res, c_out]."""
+        return self.linear(x)

@@ -116,18 +116,26 @@ class Linear(nn.Linear, _PackMixin):
             with torch.no_grad():
                 self.bias.fill_(bias_init)
 
+    def _kpad(self):
+        # ragged input widths (feature embedders: 22, 25, 49, 57, 88 ...) are zero-padded to the kernels' K step
+        return self.in_features if self.in_features % 32 == 0 else F_.round_up(self.in_features, 32)
+
     def _pk(self, dtype, device):
         params = [self.weight] + ([self.bias] if self.use_bias else [])
+        kp = self._kpad()
         return self._packed(("lin", dtype, device), params, lambda: (
-            F_.pack_rows([self.weight], dtype, device),
+            F_.pack_rows([torch.nn.functional.pad(self.weight.detach(), (0, kp - self.in_features))], dtype, device),
             F_.pack_vec([self.bias], dtype, device) if self.use_bias else None))
 
-    def forward(self, input):
+    def forward(self, input, act=_lib.FFK_ACT_NONE):
         F_.check_cuda(input)
         _no_grad_guard(self, input)
         w, b = self._pk(input.dtype, input.device)
-        x2 = input.reshape(-1, self.in_features).contiguous()
-        out = F_.linear(x2, w, b, self.out_features)
+        x2 = input.reshape(-1, self.in_features)
+        kp = self._kpad()
+        if kp != self.in_features:
+            x2 = torch.nn.functional.pad(x2, (0, kp - self.in_features))
+        out = F_.linear(x2.contiguous(), w, b, self.out_features, act=act)
         return out.view(*input.shape[:-1], self.out_features)
 
 
@@ -535,7 +543,8 @@ def __getattr__(name):
     if name == "ChunkMSARowAttentionWithPairBias":
         from .msa import ChunkMSARowAttentionWithPairBias
         return ChunkMSARowAttentionWithPairBias
-    if name in ("InputEmbedder", "RecyclingEmbedder"):      # ops.py:1046-1145,1238-1334
+    if name in ("InputEmbedder", "RecyclingEmbedder", "TemplateAngleEmbedder", "TemplatePairEmbedder",
+                "ExtraMSAEmbedder"):      # ops.py:1046-1145,1238-1334; embedders.py:257-372
         from . import embedders
         return getattr(embedders, name)
     raise AttributeError("module %r has no attribute %r" % (__name__, name))

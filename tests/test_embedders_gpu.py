@@ -118,3 +118,26 @@ def test_pair_embed_rejects_bad_arguments(dev):
     with pytest.raises(RuntimeError, match="C must be"):
         _lib.pair_embed(torch.zeros(4, 4, 96, device=dev), None, None, None, torch.zeros(3, 96, device=dev), None, None, None,
                         mode=_lib.FFK_EMBED_RELPOS, pos=pos, r=4, C=96, nb=3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_only_embedders(dev, dtype):
+    """Template angle / pair and extra-MSA embedders (ragged input widths 57 / 88 / 25) against F.linear."""
+    import torch.nn.functional as F
+    from fastfold_amd.model.fastnn.ops import ExtraMSAEmbedder, TemplateAngleEmbedder, TemplatePairEmbedder
+    torch.manual_seed(3)
+    ang = TemplateAngleEmbedder(57, 256).to(dev, dtype).eval()
+    pair = TemplatePairEmbedder(88, 64).to(dev, dtype).eval()
+    extra = ExtraMSAEmbedder(25, 64).to(dev, dtype).eval()
+    with torch.no_grad():
+        for mod in (ang, pair, extra):
+            for p in mod.parameters():
+                p.copy_(torch.randn_like(p.float()) * 0.2)
+        x = torch.randn(2, 33, 57, device=dev).to(dtype)
+        want = F.linear(F.relu(F.linear(x.float(), ang.linear_1.weight.float(), ang.linear_1.bias.float())),
+                        ang.linear_2.weight.float(), ang.linear_2.bias.float())
+        _check(_f(ang(x)), want.cpu().numpy(), dtype)
+        x = torch.randn(1, 21, 21, 88, device=dev).to(dtype)
+        _check(_f(pair(x)), F.linear(x.float(), pair.linear.weight.float(), pair.linear.bias.float()).cpu().numpy(), dtype)
+        x = torch.randn(40, 17, 25, device=dev).to(dtype)
+        _check(_f(extra(x)), F.linear(x.float(), extra.linear.weight.float(), extra.linear.bias.float()).cpu().numpy(), dtype)
