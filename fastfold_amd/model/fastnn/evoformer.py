@@ -35,15 +35,13 @@ class Evoformer(nn.Module):
     # -- un-padded core on [1, s, r, c_m] / [1, r, r, c_z] / [1, s, r] / [1, r, r] ----------
     def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
         if self.is_multimer:
-            # multimer order (evoformer.py:70-76): OPM and pair stack first, MSA stack on the old z
-            z_ori = z
-            z_new = self.communication.forward(m, msa_mask, z)
+            # multimer order (evoformer.py:70-76, 133-137): outer product mean first, the MSA stack reads the
+            # pair tensor it leaves, the pair stack runs last
+            z_new = z if inplace else torch.empty_like(z)
+            self.communication._run(m, msa_mask, z, z_new)
+            m = self.msa.inplace(m, z_new, msa_mask) if inplace else self.msa.forward(m, z_new, msa_mask)
             self.pair.inplace([z_new], pair_mask)
-            m_new = self.msa.inplace(m, z_ori, msa_mask) if inplace else self.msa.forward(m, z_ori, msa_mask)
-            if inplace:
-                z.copy_(z_new)
-                return m_new, z
-            return m_new, z_new
+            return m, z_new
         if inplace:
             m = self.msa.inplace(m, z, msa_mask)
             self.communication._run(m, msa_mask, z, z)

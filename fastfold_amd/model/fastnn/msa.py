@@ -177,12 +177,12 @@ class ExtraMSABlock(nn.Module):
     def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
         """m [1, s, r, c_m], z [1, r, r, c_z] contiguous, masks [1, s, r] / [1, r, r]."""
         if self.is_multimer:
-            # msa.py:264-270: outer product mean and pair stack first, MSA stack on the z in between
+            # msa.py:252-258, 321-332: outer product mean first, the MSA stack reads the pair tensor it leaves,
+            # the pair stack runs last
             z_new = z if inplace else torch.empty_like(z)
             self.communication._run(m, msa_mask, z, z_new)
-            z_ori = z_new.clone()
+            m = self.msa_stack.inplace([m], z_new, msa_mask)[0] if inplace else self.msa_stack.forward(m, z_new, msa_mask)
             self.pair_stack.inplace([z_new], pair_mask)
-            m = self.msa_stack.inplace([m], z_ori, msa_mask)[0] if inplace else self.msa_stack.forward(m, z_ori, msa_mask)
             return m, z_new
         if inplace:
             m = self.msa_stack.inplace([m], z, msa_mask)[0]

@@ -280,3 +280,33 @@ def test_inject_fastnn_swaps_both_stacks_and_keys(dev):
               "blocks.0.pair_stack.TriangleAttentionEndingNode.out_bias"):
         assert k in keys, k
     assert model.extra_msa_stack.blocks[0].msa_stack.MSARowAttentionWithPairBias.attention.to_qkv.weight.shape == (192, 64)
+
+
+@pytest.mark.parametrize("inplace", [False, True])
+def test_multimer_block_order(dev, inplace):
+    """is_multimer blocks run outer product mean and pair stack first and the MSA stack on the pair tensor in
+    between (fastnn/evoformer.py:70-76, fastnn/msa.py:264-270): checked against the same modules called in
+    that order by hand."""
+    from fastfold_amd.model.fastnn import Evoformer, ExtraMSABlock
+    torch.manual_seed(11)
+    for cls, c_m in ((Evoformer, 256), (ExtraMSABlock, 64)):
+        blk = cls(c_m, 128, first_block=True, last_block=True, is_multimer=True)
+        with torch.no_grad():
+            for n, p in blk.named_parameters():
+                p.copy_((1.0 if ("norm" in n and n.endswith("weight")) else 0.0) + 0.05 * torch.randn_like(p))
+        blk = blk.to(dev).eval()
+        s, r = 9, 20
+        m, z, mm, pm = (_t(x, dev, torch.float32) for x in synth_inputs(12, s, r, c_m=c_m, mask_tail_frac=0.1))
+        msa = blk.msa if cls is Evoformer else blk.msa_stack
+        pair = blk.pair if cls is Evoformer else blk.pair_stack
+        with torch.no_grad():
+            z1 = blk.communication(m[None], mm[None], z[None])
+            z2 = pair(z1, pm[None])
+            m2 = msa(m[None], z1, mm[None])
+            if inplace:
+                ml, zl = [m.clone()], [z.clone()]
+                ml, zl = blk.inplace(ml, zl, mm, pm)
+                gm, gz = ml[0], zl[0]
+            else:
+                gm, gz = blk(m, z, mm, pm)
+        assert torch.equal(gm, m2[0]) and torch.equal(gz, z2[0]), cls.__name__
