@@ -176,6 +176,8 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
     T* out = (T*)d.out + (long)bz * d.o_bs;
     const T* resid = d.resid ? (const T*)d.resid + (long)bz * d.o_bs : nullptr;
     const T* bias = (const T*)d.bias;
+    const bool plain = !bias && !resid && d.act == FFK_ACT_NONE;
+    const bool bias_resid = bias && resid && d.act == FFK_ACT_NONE;
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
         const long m = m0 + wm * 64 + mi * 32 + l32;
@@ -196,25 +198,43 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             const long nc = n + 16 <= N ? n : (N >= 16 ? N - 16 : 0);   // clamped for loads
             const long o = roff + (n >> 5) * d.s_h + (n & 31);
             const long oc = roff + (nc >> 5) * d.s_h + (nc & 31);
-            u32x4 bv[2], rv[2];
-            if (bias) {
+            // The three uniform switches (bias, residual, activation) are resolved once per block of 16 columns:
+            // the two common combinations get straight-line code, anything else the general loop.
+            T y[16];
+            if (plain) {                                     // contraction: scale only
+#pragma unroll
+                for (int v = 0; v < 16; ++v) y[v] = (T)(acc[ni][mi][v] * mul);
+            } else if (bias_resid) {                         // projection back onto the residual stream
+                u32x4 bv[2], rv[2];
                 bv[0] = *reinterpret_cast<const u32x4*>(bias + nc);
                 bv[1] = *reinterpret_cast<const u32x4*>(bias + nc + 8);
-            }
-            if (resid) {
                 rv[0] = *reinterpret_cast<const u32x4*>(resid + oc);
                 rv[1] = *reinterpret_cast<const u32x4*>(resid + oc + 8);
-            }
-            T y[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float x = acc[ni][mi][v];
-                if (bias) x += (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7];
-                if (d.act == FFK_ACT_RELU) x = relu_f(x);
-                else if (d.act == FFK_ACT_SIGMOID) x = sigmoid_f(x);
-                x *= mul;
-                if (resid) x = (float)(T)x + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7];
-                y[v] = (T)x;
+                for (int v = 0; v < 16; ++v) {
+                    const float x = (acc[ni][mi][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7]) * mul;
+                    y[v] = (T)((float)(T)x + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7]);
+                }
+            } else {
+                u32x4 bv[2], rv[2];
+                if (bias) {
+                    bv[0] = *reinterpret_cast<const u32x4*>(bias + nc);
+                    bv[1] = *reinterpret_cast<const u32x4*>(bias + nc + 8);
+                }
+                if (resid) {
+                    rv[0] = *reinterpret_cast<const u32x4*>(resid + oc);
+                    rv[1] = *reinterpret_cast<const u32x4*>(resid + oc + 8);
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    float x = acc[ni][mi][v];
+                    if (bias) x += (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7];
+                    if (d.act == FFK_ACT_RELU) x = relu_f(x);
+                    else if (d.act == FFK_ACT_SIGMOID) x = sigmoid_f(x);
+                    x *= mul;
+                    if (resid) x = (float)(T)x + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7];
+                    y[v] = (T)x;
+                }
             }
             if (ok0) *reinterpret_cast<u32x4*>(out + o) = *reinterpret_cast<const u32x4*>(&y[0]);
             if (ok1) *reinterpret_cast<u32x4*>(out + o + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
