@@ -51,7 +51,7 @@ def _check(got, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("s,r", [(5, 37), (16, 64)])
+@pytest.mark.parametrize("s,r", [(1, 1), (5, 37), (16, 64), (2, 129)])
 def test_input_embedder(dev, dtype, s, r):
     from fastfold_amd.model.fastnn.embedders import InputEmbedder
     ref, fast = _models(dev, dtype)
@@ -71,7 +71,7 @@ def test_input_embedder(dev, dtype, s, r):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("r", [23, 64])
+@pytest.mark.parametrize("r", [5, 23, 64])
 def test_recycling_embedder(dev, dtype, r):
     from fastfold_amd.model.fastnn import set_chunk_size
     ref, fast = _models(dev, dtype, seed=1)

@@ -228,3 +228,25 @@ def test_state_dict_keys_and_cpu_error(dev):
     with pytest.raises(RuntimeError):
         with torch.no_grad():
             st(torch.zeros(4, 8, 256), torch.zeros(8, 8, 128), torch.ones(4, 8), torch.ones(8, 8), chunk_size=None)
+
+
+@pytest.mark.parametrize("s,r,tail", [(1, 1, 0.0), (2, 1, 0.0), (1, 17, 0.0), (5, 8, 0.25), (129, 33, 0.1), (7, 130, 0.3)])
+def test_stack_extreme_shapes(dev, s, r, tail):
+    """Degenerate and ragged sizes (a single sequence, a single residue, sizes just past a tile edge) through a
+    two-block stack, both precisions, against the oracle."""
+    model = _oracle(5, 2)
+    m, z, mm, pm = synth_inputs(3, s, r, mask_tail_frac=tail)
+    with torch.no_grad():
+        rm, rz, rs = model.evoformer(*(torch.from_numpy(x) for x in (m, z, mm, pm)), chunk_size=None, _mask_trans=False)
+    nv = r - int(round(tail * r))
+    rm, rz, rs = rm.numpy()[:, :nv], rz.numpy()[:nv, :nv], rs.numpy()[:nv]
+    for dtype in (torch.float32, torch.bfloat16):
+        fast = _fast(model, dev, dtype)
+        with torch.no_grad():
+            gm, gz, gs = fast(*(_t(x, dev, dtype) for x in (m, z, mm, pm)), chunk_size=None, _mask_trans=False)
+        gm, gz, gs = _f(gm)[:, :nv], _f(gz)[:nv, :nv], _f(gs)[:nv]
+        if dtype == torch.float32:
+            for g, ref in ((gm, rm), (gz, rz), (gs, rs)):
+                assert np.abs(g - ref).max() <= 1e-4 * max(1.0, float(np.abs(ref).max()))
+        else:
+            assert _rel_l2(gm, rm) <= 2e-2 and _rel_l2(gz, rz) <= 2e-2 and _rel_l2(gs, rs) <= 2e-2

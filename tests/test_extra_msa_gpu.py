@@ -310,3 +310,23 @@ def test_multimer_block_order(dev, inplace):
             else:
                 gm, gz = blk(m, z, mm, pm)
         assert torch.equal(gm, m2[0]) and torch.equal(gz, z2[0]), cls.__name__
+
+
+@pytest.mark.parametrize("s,r,tail", [(1, 1, 0.0), (3, 1, 0.0), (2, 17, 0.1), (1025, 33, 0.1)])
+def test_extra_stack_extreme_shapes(dev, s, r, tail):
+    """A single extra sequence, a single residue, N_extra just past a 1024 boundary: two blocks, both precisions."""
+    model = _oracle(44, 2)
+    m, z, mm, pm = synth_inputs(4, s, r, c_m=64, mask_tail_frac=tail)
+    with torch.no_grad():
+        rz = model.extra_msa_stack(torch.from_numpy(m), torch.from_numpy(z), msa_mask=torch.from_numpy(mm),
+                                   pair_mask=torch.from_numpy(pm), _mask_trans=False).numpy()
+    nv = r - int(round(tail * r))
+    for dtype in (torch.float32, torch.bfloat16):
+        fast = _fast(model, dev, dtype)
+        with torch.no_grad():
+            gz = _f(fast(*(_t(x, dev, dtype) for x in (m, z)), chunk_size=None, msa_mask=_t(mm, dev, dtype),
+                         pair_mask=_t(pm, dev, dtype)))
+        if dtype == torch.float32:
+            assert np.abs(gz[:nv, :nv] - rz[:nv, :nv]).max() <= 1e-4 * max(1.0, float(np.abs(rz).max()))
+        else:
+            assert _rel_l2(gz[:nv, :nv], rz[:nv, :nv]) <= 2e-2

@@ -157,3 +157,21 @@ def test_template_stack_bf16_rel_l2(dev):
         got = _f(fast(_t(tb, dev, torch.bfloat16), _t(pm[None], dev, torch.bfloat16), chunk_size=None))
     nv = r - int(round(tail * r))
     assert _rel_l2(got[:, :nv, :nv], ref[:, :nv, :nv]) <= 2e-2
+
+
+@pytest.mark.parametrize("nt,r,tail", [(1, 1, 0.0), (4, 2, 0.0), (1, 17, 0.1), (2, 130, 0.2)])
+def test_template_stack_extreme_shapes(dev, nt, r, tail):
+    """One residue, two residues with four templates, sizes just past a tile edge: two blocks, both precisions."""
+    oracle = _oracle(54, 2)
+    t, pm = synth_template_inputs(5, nt, r, mask_tail_frac=tail)
+    with torch.no_grad():
+        ref = oracle(torch.from_numpy(t), torch.from_numpy(pm)[None], _mask_trans=False).numpy()
+    nv = r - int(round(tail * r))
+    for dtype in (torch.float32, torch.bfloat16):
+        fast = _fast(oracle, dev, dtype)
+        with torch.no_grad():
+            got = _f(fast(_t(t, dev, dtype), _t(pm[None], dev, dtype), chunk_size=None))
+        if dtype == torch.float32:
+            assert np.abs(got[:, :nv, :nv] - ref[:, :nv, :nv]).max() <= 1e-4 * max(1.0, float(np.abs(ref).max()))
+        else:
+            assert _rel_l2(got[:, :nv, :nv], ref[:, :nv, :nv]) <= 2e-2
