@@ -33,7 +33,8 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
         if len(procs) >= jobs:
             _drain(procs, verbose)
     _drain(procs, verbose)
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--version-script=" + os.path.join(HERE, "ffk.map"),
+           "-o", LIB] + objs
     out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if out.returncode != 0:
         raise RuntimeError("link failed:\n" + out.stdout)
