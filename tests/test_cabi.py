@@ -47,3 +47,15 @@ def test_argument_validation_without_gpu():
     assert lib.ffk_bias_sigmoid_mul(p, p, None, p, 2, 4, _lib.FFK_F32, None) == 3
     with pytest.raises(RuntimeError):
         _lib.call("ffk_softmax_bwd", None, None, None, 1, 1, 0, None)
+
+
+def test_library_exports_nothing_else():
+    """The dynamic symbol table holds the declared entry points and no internal (C++-mangled) helpers."""
+    import shutil
+    import subprocess
+    nm = shutil.which("nm")
+    if nm is None:
+        pytest.skip("binutils nm not available")
+    out = subprocess.run([nm, "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == _declared(), sorted(set(exported) ^ set(_declared()))
