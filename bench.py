@@ -9,7 +9,7 @@ the Evoformer-block latency (ms per block = step time / 48).  The same JSON line
                 algorithmic FLOPs / HIP-event time of its launches inside the timed region,
   cpu_baseline  the CPU oracle (plain-PyTorch restatement of the reference's nn Evoformer block)
                 timed on this box's host cores on a bounded sample,
-and the op micro-benchmarks of BASELINE config 2 (fused softmax, LayerNorm: HBM GB/s).
+and the op micro-benchmarks of benchmark configuration 2 (fused softmax, LayerNorm: HBM GB/s).
 """
 import argparse
 import json
@@ -62,7 +62,7 @@ def build_stack(no_blocks, dev, dtype, seed=0):
 
 
 def micro_ops(dev):
-    """BASELINE config 2: fused softmax [1,128,8,256,256] bf16 with pair bias and 10% masked keys;
+    """benchmark configuration 2: fused softmax [1,128,8,256,256] bf16 with pair bias and 10% masked keys;
     LayerNorm over [65536,128] and [32768,256] bf16; plus a plain device copy of the softmax's
     bytes as the practical HBM ceiling of this box.  Each op runs over rotating buffers (> 512 MB in
     total, so nothing is served from cache) as N launches recorded into one HIP graph; the time is
@@ -173,7 +173,7 @@ def feeder_stacks(dev, r):
 
 
 def long_sequence(dev):
-    """BASELINE configs[4]: one block at N_seq = 64, N_res = 4096 (z = 4.3 GB), chunk size 64, in place; latency
+    """Benchmark configuration 5: one block at N_seq = 64, N_res = 4096 (z = 4.3 GB), chunk size 64, in place; latency
     and peak device memory."""
     import torch
     from fastfold_amd.model.fastnn import set_chunk_size
@@ -305,7 +305,7 @@ def main():
         "roofline": roofline,
     }
     if args.workload == "cfg4" and not args.no_micro:
-        # the same stack at BASELINE configs[2] (N_res = 256), reported beside the headline number
+        # the same stack at benchmark configuration 3 (N_res = 256), reported beside the headline number
         w3 = WORKLOADS["cfg3"]
         m3, z3, mm3, pm3 = (torch.from_numpy(t).to(dev, torch.bfloat16)
                             for t in synth_inputs(0, w3["n_seq"], w3["n_res"], mask_tail_frac=w3["tail"]))

@@ -156,7 +156,7 @@ def test_golden_vectors_fp32(dev):
 
 
 def test_config1_block_fp32(dev):
-    """BASELINE config 1: one block, fp32, s=32, r=64, weights N(0, 0.02^2): max-abs <= 1e-4."""
+    """Benchmark configuration 1: one block, fp32, s=32, r=64, weights N(0, 0.02^2): max-abs <= 1e-4."""
     model = _oracle(1, 1, fis=False)
     fast = _fast(model, dev, torch.float32)
     m, z, mm, pm = synth_inputs(1, 32, 64)

@@ -47,7 +47,7 @@ def _rel_l2(a, b):
 
 
 def test_cfg3_two_blocks_bf16_against_oracle(dev):
-    """BASELINE configs[2] shape (N_seq = 128, N_res = 256), two blocks, O(1) updates, padded tail."""
+    """benchmark configuration 3 shape (N_seq = 128, N_res = 256), two blocks, O(1) updates, padded tail."""
     s, r, tail = 128, 256, 0.05
     model, fast = _models(61, 2, dev)
     m, z, mm, pm = synth_inputs(61, s, r, mask_tail_frac=tail)
