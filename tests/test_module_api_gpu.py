@@ -249,3 +249,47 @@ def test_dropout_modules_are_identity_in_eval(dev):
         # the mask is shared along rows (dim 1) or columns (dim 2)
         dim = 1 if cls is DropoutRowwise else 2
         assert torch.equal(keep, keep.narrow(dim, 0, 1).expand_as(keep))
+
+
+def test_side_stream_matches_default_stream(dev):
+    """Launches go to the caller's current stream: a block run on a side stream gives the bits of the default stream."""
+    blk = _block(dev, torch.bfloat16, "Evoformer")
+    m, z, mm, pm = (torch.from_numpy(np.ascontiguousarray(t)).to(dev, torch.bfloat16)
+                    for t in synth_inputs(8, 12, 72, mask_tail_frac=0.1))
+    with torch.no_grad():
+        rm, rz = blk(m, z, mm, pm)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            gm, gz = blk(m, z, mm, pm)
+        side.synchronize()
+    assert torch.equal(gm, rm) and torch.equal(gz, rz)
+
+
+def test_block_forward_replays_from_a_captured_graph(dev):
+    """One block forward captured in a HIP graph and replayed with new input contents, with eager work and
+    synchronisations between the replays: every replay equals the eager result on the same inputs."""
+    blk = _block(dev, torch.bfloat16, "Evoformer")
+    ins = [[torch.from_numpy(np.ascontiguousarray(t)).to(dev, torch.bfloat16)
+            for t in synth_inputs(20 + i, 16, 64, mask_tail_frac=0.1)] for i in range(3)]
+    static = [t.clone() for t in ins[0]]
+    with torch.no_grad():
+        eager = [blk(*x) for x in ins]                      # also warms the weight packs and launch attributes
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            blk(*static)                                    # warm-up on the capture stream
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            gm, gz = blk(*static)
+        for i in (1, 2, 0, 1):
+            for dst, src in zip(static, ins[i]):
+                dst.copy_(src)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(gm, eager[i][0]) and torch.equal(gz, eager[i][1]), "replay with input set %d" % i
+            blk(*ins[(i + 1) % 3])                          # eager work between replays
+            torch.cuda.synchronize()
