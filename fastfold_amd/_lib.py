@@ -303,3 +303,15 @@ SIGNATURES["ffk_pair_embed"] = [_P, _P, _P, _P, _F, _P, _P, _P, _P, _I, _P, _P, 
 def pair_embed(out, z, gamma, beta, table, bias, row, col, *, mode, pos, edges=None, inf=1e8, r, C, nb, ln_eps=1e-5):
     call("ffk_pair_embed", ptr(out), ptr(z), ptr(gamma), ptr(beta), ln_eps, ptr(table), ptr(bias), ptr(row), ptr(col),
          mode, ptr(pos), ptr(edges), inf, r, C, nb, dtype_tag(out.dtype), stream_ptr())
+
+
+SIGNATURES["ffk_pointwise_attention_core"] = [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]
+
+
+def pointwise_attention_core(o, q, kv, bias, *, P, H, D, NT, kv_st, kv_sp, v_off):
+    """o[p, h] = softmax_t(q[p, h] . k[t, p, h] + bias[t]) v[t, p, h]; strides in elements (see include/ffk.h)."""
+    check_device(o, q, kv, bias)
+    if bias.dtype != torch.float32 or bias.numel() != NT:
+        raise RuntimeError("pointwise_attention_core: bias must be fp32 [NT]")
+    call("ffk_pointwise_attention_core", ptr(o), ptr(q), ptr(kv), ptr(bias), P, H, D, NT, kv_st, kv_sp, v_off,
+         dtype_tag(q.dtype), stream_ptr())

@@ -4,7 +4,7 @@ from .msa import MSACore, ExtraMSACore, ExtraMSABlock, ExtraMSAStack
 from .ops import OutProductMean, set_chunk_size, get_chunk_size
 from .triangle import PairCore
 from .evoformer import Evoformer, EvoformerStack
-from .template import TemplatePairBlock, TemplatePairStack
+from .template import TemplatePairBlock, TemplatePairStack, TemplatePointwiseAttention
 
 __all__ = ['MSACore', 'OutProductMean', 'PairCore', 'set_chunk_size', 'get_chunk_size', 'Evoformer', 'EvoformerStack',
-           'ExtraMSACore', 'ExtraMSABlock', 'ExtraMSAStack', 'TemplatePairBlock', 'TemplatePairStack']
+           'ExtraMSACore', 'ExtraMSABlock', 'ExtraMSAStack', 'TemplatePairBlock', 'TemplatePairStack', 'TemplatePointwiseAttention']

@@ -14,9 +14,85 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from fastfold_amd.model.fastnn.kernel import LayerNorm
+from fastfold_amd import _lib
 from . import _fused as F_
 from .ops import (AsyncChunkTriangleMultiplicationIncoming, AsyncChunkTriangleMultiplicationOutgoing,
-                  ChunkTransition, ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode)
+                  ChunkTransition, ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode, Linear,
+                  _PackMixin, _no_grad_guard)
+
+
+class _PointwiseProjections(nn.Module):
+    """Parameter holder with the names of the reference's generic ``Attention`` (nn/primitives.py:333-338),
+    gating off: ``linear_q`` / ``linear_k`` / ``linear_v`` without bias, ``linear_o`` with bias."""
+
+    def __init__(self, c_q, c_kv, c_hidden, no_heads):
+        super(_PointwiseProjections, self).__init__()
+        hc = c_hidden * no_heads
+        self.linear_q = Linear(c_q, hc, use_bias=False)
+        self.linear_k = Linear(c_kv, hc, use_bias=False)
+        self.linear_v = Linear(c_kv, hc, use_bias=False)
+        self.linear_o = Linear(hc, c_q, initializer='zeros')
+
+
+class TemplatePointwiseAttention(nn.Module, _PackMixin):
+    """Algorithm 17 (fastfold/model/fastnn/template.py:33-182): every pair position attends over the
+    templates' embeddings at that position.  Two projection launches (q from z, k and v from t), one
+    streaming kernel for the softmax over at most 8 templates, one output projection; the update is zero
+    when no template is valid, as in the reference."""
+
+    def __init__(self, c_t, c_z, c_hidden, no_heads, inf, **kwargs):
+        super(TemplatePointwiseAttention, self).__init__()
+        self.c_t, self.c_z, self.c_hidden, self.no_heads, self.inf = c_t, c_z, c_hidden, no_heads, inf
+        self.mha = _PointwiseProjections(c_z, c_t, c_hidden, no_heads)
+
+    def _run(self, t, z, template_mask, resid):
+        F_.check_cuda(t, z, template_mask)
+        _no_grad_guard(self, t, z)
+        if t.dim() != 4 or z.dim() != 3 or t.shape[1:3] != z.shape[:2] or t.shape[-1] != self.c_t or z.shape[-1] != self.c_z:
+            raise RuntimeError("TemplatePointwiseAttention: expected t [N_templ, r, r, %d] and z [r, r, %d], got %s / %s"
+                               % (self.c_t, self.c_z, tuple(t.shape), tuple(z.shape)))
+        NT, r = t.shape[0], t.shape[1]
+        if NT > 8:
+            raise RuntimeError("TemplatePointwiseAttention: at most 8 templates per launch, got %d" % NT)
+        dt, dev = z.dtype, z.device
+        H, D = self.no_heads, self.c_hidden
+        hc = H * D
+        P = r * r
+        m = self.mha
+        wq, wkv, wo, bo = self._packed(("pw", dt, dev), [m.linear_q.weight, m.linear_k.weight, m.linear_v.weight,
+                                                          m.linear_o.weight, m.linear_o.bias], lambda: (
+            F_.pack_rows([m.linear_q.weight.detach() * (float(D) ** -0.5)], dt, dev),
+            F_.pack_rows([m.linear_k.weight, m.linear_v.weight], dt, dev),
+            F_.pack_rows([m.linear_o.weight], dt, dev), F_.pack_vec([m.linear_o.bias], dt, dev)))
+        if template_mask is None:
+            template_mask = t.new_ones(NT)
+        tm = template_mask.to(device=dev, dtype=torch.float32).reshape(NT)
+        bias = (self.inf * (tm - 1.0)).contiguous()
+        any_valid = (tm.sum() > 0).to(dt)                                  # stays on the device: no host round trip
+        q = F_.linear(z.contiguous().view(P, self.c_z), wq, None, hc)
+        kv = F_.linear(t.contiguous().view(NT * P, self.c_t), wkv, None, 2 * hc)
+        o = torch.empty(P, hc, dtype=dt, device=dev)
+        _lib.pointwise_attention_core(o, q, kv, bias, P=P, H=H, D=D, NT=NT, kv_st=P * 2 * hc, kv_sp=2 * hc, v_off=hc)
+        del q, kv
+        o.mul_(any_valid)
+        out = F_.linear(o, wo, bo * any_valid, self.c_z, out=resid, resid=resid)     # in place when a residual is given
+        return out.view(r, r, self.c_z)
+
+    def forward(self, t: torch.Tensor, z: torch.Tensor, template_mask: Optional[torch.Tensor] = None,
+                chunk_size: Optional[int] = None) -> torch.Tensor:
+        """t [N_templ, N_res, N_res, C_t], z [N_res, N_res, C_z], template_mask [N_templ]
+        -> the pair update [N_res, N_res, C_z] (not yet added to z)."""
+        return self._run(t, z, template_mask, None)
+
+    def inplace(self, t: torch.Tensor, z: torch.Tensor, template_mask: Optional[torch.Tensor] = None,
+                chunk_size: Optional[int] = None) -> torch.Tensor:
+        """Same, with the update added to z in place; returns z."""
+        zc = z.contiguous()
+        out = self._run(t, zc, template_mask, zc.view(-1, self.c_z))
+        if zc.data_ptr() != z.data_ptr():
+            z.copy_(out)
+            return z
+        return out
 
 
 class TemplatePairBlock(nn.Module):

@@ -155,6 +155,28 @@ def synth_template_nn_state(seed=0, no_blocks=2, std=0.02, fan_in_scaled=False, 
     return sd
 
 
+def synth_pointwise_nn_state(seed=0, c_t=64, c_z=128, c_hidden=16, no_heads=4):
+    """nn-layout state of a ``TemplatePointwiseAttention`` (``mha.linear_{q,k,v,o}``), fan-in scaled weights so
+    that the logits over the templates are O(1)."""
+    rng = np.random.RandomState(seed)
+    hc = c_hidden * no_heads
+    sd = OrderedDict()
+    for name, shape in (("mha.linear_q.weight", (hc, c_z)), ("mha.linear_k.weight", (hc, c_t)),
+                        ("mha.linear_v.weight", (hc, c_t)), ("mha.linear_o.weight", (c_z, hc))):
+        sd[name] = (rng.standard_normal(shape) * (2.0 if name.endswith("q.weight") else 1.0)
+                    / np.sqrt(shape[1])).astype(np.float32)
+    sd["mha.linear_o.bias"] = (0.1 * rng.standard_normal((c_z,))).astype(np.float32)
+    return sd
+
+
+def synth_pointwise_inputs(seed, n_templ, n_res, c_t=64, c_z=128):
+    """t [n_templ, r, r, c_t], z [r, r, c_z] ~ N(0, 1) fp32."""
+    rng = np.random.RandomState(seed + 7)
+    t = rng.standard_normal((n_templ, n_res, n_res, c_t)).astype(np.float32)
+    z = rng.standard_normal((n_res, n_res, c_z)).astype(np.float32)
+    return t, z
+
+
 def synth_nn_state(seed=0, no_blocks=1, std=0.02, c_m=256, c_z=128, c_s=384, fan_in_scaled=False, **dims):
     """OrderedDict name -> float32 numpy array, nn layout, for an ``EvoformerStack``.
 

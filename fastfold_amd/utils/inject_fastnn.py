@@ -21,7 +21,7 @@ import torch
 
 from fastfold_amd.model.fastnn import EvoformerStack, ExtraMSAStack
 from fastfold_amd.model.fastnn.embedders import InputEmbedder, RecyclingEmbedder
-from fastfold_amd.model.fastnn.template import TemplatePairStack
+from fastfold_amd.model.fastnn.template import TemplatePairStack, TemplatePointwiseAttention
 
 
 def copy_layernorm(model_fast, model_ori):
@@ -180,7 +180,7 @@ def copy_template_pair_block_para(fast_module, target_module):
 def inject_template_pair_stack(template_embedder):
     """Swaps ``template_embedder.template_pair_stack`` (nn layout) for the HIP-backed stack.  The
     reference's ``inject_template`` (inject_fastnn.py:358-374) replaces the whole template embedder;
-    its embedders and point-wise attention are outside this build and stay as they are."""
+    the point-wise attention is swapped too when the embedder has one; its feature embedders stay as they are."""
     with torch.no_grad():
         target = template_embedder.template_pair_stack
         blk = target.blocks[0]
@@ -196,6 +196,31 @@ def inject_template_pair_stack(template_embedder):
         if target.training is False:
             fast.eval()
         template_embedder.template_pair_stack = fast
+        if getattr(template_embedder, "template_pointwise_att", None) is not None:
+            inject_template_pointwise_att(template_embedder)
+    return template_embedder
+
+
+def copy_native_att(model_fast, model_ori):
+    """linear_q / linear_k / linear_v / linear_o of an un-gated ``Attention`` (inject_fastnn.py:98-104)."""
+    for name in ("linear_q", "linear_k", "linear_v"):
+        getattr(model_fast, name).weight.copy_(getattr(model_ori, name).weight)
+    copy_linear(model_fast.linear_o, model_ori.linear_o)
+
+
+def inject_template_pointwise_att(template_embedder):
+    """Swaps ``template_embedder.template_pointwise_att`` for the HIP-backed module (the reference copies its
+    parameters with ``copy_native_att``, inject_fastnn.py:278-279)."""
+    with torch.no_grad():
+        target = template_embedder.template_pointwise_att
+        ref_param = next(target.parameters())
+        fast = TemplatePointwiseAttention(c_t=target.c_t, c_z=target.c_z, c_hidden=target.c_hidden,
+                                          no_heads=target.no_heads, inf=target.inf).to(device=ref_param.device,
+                                                                                       dtype=ref_param.dtype)
+        copy_native_att(fast.mha, target.mha)
+        if target.training is False:
+            fast.eval()
+        template_embedder.template_pointwise_att = fast
     return template_embedder
 
 

@@ -518,6 +518,27 @@ class TemplatePairStack(nn.Module):
         return self.layer_norm(t)
 
 
+class TemplatePointwiseAttention(nn.Module):
+    """Algorithm 17 (nn/template.py:45-133): every pair position attends over the templates' embeddings at
+    that position.  q = W_q z[i, j], keys / values from t[n, i, j], additive bias inf * (template_mask - 1)
+    over the template axis, no gating.  The caller zeroes the update when no template is valid
+    (nn/embedders.py:316); the fastnn module does that inside (fastnn/template.py:117-119)."""
+
+    def __init__(self, c_t=64, c_z=128, c_hidden=16, no_heads=4, inf=1e5, **kwargs):
+        super().__init__()
+        self.c_t, self.c_z, self.c_hidden, self.no_heads, self.inf = c_t, c_z, c_hidden, no_heads, inf
+        self.mha = Attention(c_z, c_t, c_t, c_hidden, no_heads, gating=False)
+
+    def forward(self, t, z, template_mask=None, chunk_size=None):
+        """t [N_templ, N_res, N_res, C_t], z [N_res, N_res, C_z], template_mask [N_templ] -> [N_res, N_res, C_z]."""
+        if template_mask is None:
+            template_mask = t.new_ones(t.shape[:-3])
+        bias = self.inf * (template_mask[..., None, None, None, None, :] - 1)     # [1, 1, 1, 1, N_templ]
+        q_x = z.unsqueeze(-2)                                                    # [r, r, 1, C_z]
+        kv_x = t.permute(1, 2, 0, 3)                                             # [r, r, N_templ, C_t]
+        return self.mha(q_x, kv_x, biases=[bias]).squeeze(-2)
+
+
 # --------------------------------------------------------------------------
 # input and recycling embedders  (reference: fastfold/model/nn/embedders.py:35-232,
 # one_hot: fastfold/utils/tensor_utils.py:63-67)

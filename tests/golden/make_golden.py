@@ -6,6 +6,7 @@ and inputs.  Run only in the build container, where /root/reference is mounted:
     python tests/golden/make_golden.py            # Evoformer stack
     python tests/golden/make_golden.py extra      # extra-MSA stack
     python tests/golden/make_golden.py template   # template pair stack
+    python tests/golden/make_golden.py pointwise  # template point-wise attention
 
 The fixture pins what closed forms cannot: the composition of a block (order of the
 sub-updates, residual placement, OPM reading the updated MSA), the q/k/v and left/right
@@ -121,8 +122,39 @@ def main_template():
     print("wrote", os.path.join(HERE, "template_pair_nn_golden.npz"))
 
 
+POINTWISE_CASES = [
+    # name, seed, n_templ, n_res, template_mask
+    ("pw_all", 61, 4, 12, (1.0, 1.0, 1.0, 1.0)),
+    ("pw_masked", 62, 4, 9, (1.0, 0.0, 1.0, 0.0)),
+    ("pw_one", 63, 1, 7, (1.0,)),
+    ("pw_none", 64, 2, 5, (0.0, 0.0)),
+]
+
+
+def main_pointwise():
+    from fastfold.model.nn.template import TemplatePointwiseAttention  # the reference
+    from fastfold_amd.synthetic import synth_pointwise_inputs, synth_pointwise_nn_state
+
+    out = {}
+    for name, seed, nt, r, tmask in POINTWISE_CASES:
+        mod = TemplatePointwiseAttention(c_t=64, c_z=128, c_hidden=16, no_heads=4, inf=1e5).eval()
+        sd = synth_pointwise_nn_state(seed=seed)
+        missing, unexpected = mod.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        assert not missing and not unexpected
+        t, z = synth_pointwise_inputs(seed, nt, r)
+        with torch.no_grad():
+            upd = mod(torch.from_numpy(t), torch.from_numpy(z), template_mask=torch.tensor(tmask), chunk_size=None)
+        out[name + ".out"] = upd.numpy()
+        out[name + ".cfg"] = np.array([seed, nt, r] + [int(x) for x in tmask], dtype=np.int64)
+        print(name, "mean |update|", float(np.abs(upd.numpy()).mean()))
+    np.savez_compressed(os.path.join(HERE, "template_pointwise_nn_golden.npz"), **out)
+    print("wrote", os.path.join(HERE, "template_pointwise_nn_golden.npz"))
+
+
 if __name__ == "__main__":
-    if "template" in sys.argv[1:]:
+    if "pointwise" in sys.argv[1:]:
+        main_pointwise()
+    elif "template" in sys.argv[1:]:
         main_template()
     elif "extra" in sys.argv[1:]:
         main_extra()

@@ -311,3 +311,41 @@ def test_embedders_brute_force():
                 want = want + P["linear.weight"][:, hit[0]]
             assert np.abs(zu[i, j] - want).max() < 1e-10
     assert none_hit >= r + 2        # the diagonal and the pair on the edge
+
+
+def test_template_pointwise_golden_and_brute_force():
+    """The point-wise template attention against the reference's vectors (tests/golden/make_golden.py pointwise)
+    and against float64 loops over positions, heads and templates."""
+    from fastfold_amd.synthetic import synth_pointwise_inputs, synth_pointwise_nn_state
+    from oracle.evoformer_ref import TemplatePointwiseAttention
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "template_pointwise_nn_golden.npz"))
+    names = sorted(k[:-4] for k in g.files if k.endswith(".cfg"))
+    assert len(names) == 4
+    for name in names:
+        cfg = g[name + ".cfg"]
+        seed, nt, r, tmask = int(cfg[0]), int(cfg[1]), int(cfg[2]), [float(x) for x in cfg[3:]]
+        mod = TemplatePointwiseAttention().eval()
+        sd = synth_pointwise_nn_state(seed=seed)
+        mod.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        t, z = synth_pointwise_inputs(seed, nt, r)
+        with torch.no_grad():
+            out = mod(torch.from_numpy(t), torch.from_numpy(z), template_mask=torch.tensor(tmask)).numpy()
+        assert np.abs(out - g[name + ".out"]).max() <= 2e-5, name
+        # brute force on a few positions (not when every template is masked: the reference adds -1e5 to the fp32
+        # logits there, which rounds them to multiples of 2^-7; that case is pinned by the vectors alone)
+        if sum(tmask) == 0:
+            continue
+        W = {k: v.astype(np.float64) for k, v in sd.items()}
+        H, D = 4, 16
+        for (i, j) in ((0, 0), (r - 1, 2), (3, r - 1)):
+            q = (W["mha.linear_q.weight"] @ z[i, j].astype(np.float64)) / np.sqrt(D)
+            o = np.zeros(H * D)
+            for h in range(H):
+                logit = np.array([q[h * D:(h + 1) * D] @ (W["mha.linear_k.weight"] @ t[n, i, j].astype(np.float64))[h * D:(h + 1) * D]
+                                  + 1e5 * (tmask[n] - 1) for n in range(nt)])
+                w = np.exp(logit - logit.max())
+                w /= w.sum()
+                for n in range(nt):
+                    o[h * D:(h + 1) * D] += w[n] * (W["mha.linear_v.weight"] @ t[n, i, j].astype(np.float64))[h * D:(h + 1) * D]
+            ref = W["mha.linear_o.weight"] @ o + W["mha.linear_o.bias"]
+            assert np.abs(out[i, j] - ref).max() <= 1e-4, (name, i, j)

@@ -175,3 +175,99 @@ def test_template_stack_extreme_shapes(dev, nt, r, tail):
             assert np.abs(got[:, :nv, :nv] - ref[:, :nv, :nv]).max() <= 1e-4 * max(1.0, float(np.abs(ref).max()))
         else:
             assert _rel_l2(got[:, :nv, :nv], ref[:, :nv, :nv]) <= 2e-2
+
+
+# ---------------------------------------------------------------- template point-wise attention ----
+def _pointwise(seed, dev, dtype):
+    from fastfold_amd.model.fastnn import TemplatePointwiseAttention
+    from fastfold_amd.synthetic import synth_pointwise_nn_state
+    from oracle.evoformer_ref import TemplatePointwiseAttention as OraclePW
+    sd = {k: torch.from_numpy(v) for k, v in synth_pointwise_nn_state(seed=seed).items()}
+    ref = OraclePW().eval()
+    ref.load_state_dict(sd, strict=True)
+    fast = TemplatePointwiseAttention(c_t=64, c_z=128, c_hidden=16, no_heads=4, inf=1e5)
+    missing, unexpected = fast.load_state_dict(sd, strict=True)       # same keys as the reference's module
+    assert not missing and not unexpected
+    return ref, fast.to(dev, dtype).eval()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nt,r,tmask", [(4, 12, (1, 1, 1, 1)), (4, 9, (1, 0, 1, 0)), (1, 7, (1,)), (2, 5, (0, 0)),
+                                        (8, 33, (1, 1, 0, 1, 1, 0, 1, 1)), (3, 1, (0, 1, 1))])
+def test_template_pointwise_attention(dev, dtype, nt, r, tmask):
+    """fastnn/template.py:83-131 against the oracle (pinned by the reference's vectors); the fastnn module zeroes
+    the update itself when no template is valid (template.py:117-119)."""
+    from fastfold_amd.synthetic import synth_pointwise_inputs
+    ref, fast = _pointwise(70 + nt, dev, dtype)
+    t, z = synth_pointwise_inputs(70 + r, nt, r)
+    tm = torch.tensor([float(x) for x in tmask])
+    tb, zb = (torch.from_numpy(x).to(dtype).float() for x in (t, z))
+    with torch.no_grad():
+        want = ref(tb, zb, template_mask=tm).numpy() * float(tm.sum() > 0)
+        got = fast(tb.to(dev, dtype), zb.to(dev, dtype), template_mask=tm.to(dev, dtype))
+        zin = zb.to(dev, dtype)
+        zres = fast.inplace(tb.to(dev, dtype), zin, template_mask=tm.to(dev, dtype))
+    assert got.shape == (r, r, 128) and got.dtype == dtype
+    assert zres.data_ptr() == zin.data_ptr()
+    got, zres = _f(got), _f(zres)
+    if dtype == torch.float32:
+        assert np.abs(got - want).max() <= 1e-4 * max(1.0, float(np.abs(want).max()))
+        assert np.abs(zres - (zb.numpy() + want)).max() <= 1e-4 * max(1.0, float(np.abs(want).max()))
+    else:
+        if tm.sum() > 0:
+            assert _rel_l2(got, want) <= 2e-2
+        else:
+            assert np.abs(got).max() == 0.0
+        assert _rel_l2(zres, zb.numpy() + want) <= 2e-2
+
+
+def test_template_pointwise_golden_vectors(dev):
+    """The reference's own outputs (tests/golden/make_golden.py pointwise), fp32."""
+    from fastfold_amd.synthetic import synth_pointwise_inputs
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "template_pointwise_nn_golden.npz"))
+    for name in sorted(k[:-4] for k in g.files if k.endswith(".cfg")):
+        cfg = g[name + ".cfg"]
+        seed, nt, r, tmask = int(cfg[0]), int(cfg[1]), int(cfg[2]), [float(x) for x in cfg[3:]]
+        if sum(tmask) == 0:
+            continue          # the fastnn module returns zeros there; the reference's nn module leaves that to its caller
+        _, fast = _pointwise(seed, dev, torch.float32)
+        t, z = synth_pointwise_inputs(seed, nt, r)
+        with torch.no_grad():
+            got = _f(fast(_t(t, dev, torch.float32), _t(z, dev, torch.float32), template_mask=torch.tensor(tmask, device=dev)))
+        assert np.abs(got - g[name + ".out"]).max() <= 1e-4, name
+
+
+def test_pointwise_core_rejects_bad_arguments(dev):
+    from fastfold_amd import _lib
+    q = torch.zeros(4, 64, device=dev)
+    kv = torch.zeros(2, 4, 128, device=dev)
+    o = torch.empty(4, 64, device=dev)
+    b = torch.zeros(2, device=dev)
+    with pytest.raises(RuntimeError, match="head width"):
+        _lib.pointwise_attention_core(o, q, kv, b, P=4, H=4, D=12, NT=2, kv_st=512, kv_sp=128, v_off=64)
+    with pytest.raises(RuntimeError, match="NT"):
+        _lib.pointwise_attention_core(o, q, kv, torch.zeros(9, device=dev), P=4, H=4, D=16, NT=9, kv_st=512, kv_sp=128, v_off=64)
+    with pytest.raises(RuntimeError, match="v_off"):
+        _lib.pointwise_attention_core(o, q, kv, b, P=4, H=4, D=16, NT=2, kv_st=512, kv_sp=128, v_off=32)
+
+
+def test_inject_swaps_the_pointwise_attention_too(dev):
+    """An embedder that carries both the pair stack and the point-wise attention gets both swapped, parameters
+    copied (inject_fastnn.py:271-279)."""
+    from fastfold_amd.model.fastnn import TemplatePairStack, TemplatePointwiseAttention
+    from fastfold_amd.synthetic import synth_pointwise_inputs, synth_pointwise_nn_state
+    from fastfold_amd.utils.inject_fastnn import inject_template_pair_stack
+    from oracle.evoformer_ref import TemplatePointwiseAttention as OraclePW
+    e = _Embedder(copy.deepcopy(_oracle(54, 1)))
+    e.template_pointwise_att = OraclePW().eval()
+    e.template_pointwise_att.load_state_dict({k: torch.from_numpy(v) for k, v in synth_pointwise_nn_state(seed=5).items()})
+    ref = copy.deepcopy(e.template_pointwise_att)
+    inject_template_pair_stack(e)
+    assert isinstance(e.template_pair_stack, TemplatePairStack)
+    assert isinstance(e.template_pointwise_att, TemplatePointwiseAttention) and not e.template_pointwise_att.training
+    t, z = synth_pointwise_inputs(5, 2, 6)
+    e = e.to(dev)
+    with torch.no_grad():
+        got = _f(e.template_pointwise_att(_t(t, dev, torch.float32), _t(z, dev, torch.float32)))
+        want = ref(torch.from_numpy(t), torch.from_numpy(z)).numpy()
+    assert np.abs(got - want).max() <= 1e-4
