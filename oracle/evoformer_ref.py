@@ -16,6 +16,8 @@ Pinning (what each part is checked against, see tests/test_oracle.py):
                                                reference's fastfold.model.nn in the
                                                build container (tests/golden/)
   * global attention                           float64 loops over the published formula
+  * template point-wise attention              golden vectors from the reference's module and
+                                               float64 loops over positions / heads / templates
   * input / recycling embedders                float64 loops (a Linear on a one-hot vector is a
                                                column pick); no golden vectors: the reference's
                                                nn/embedders.py needs dm-tree, absent here
