@@ -59,6 +59,13 @@ def check_cuda(*ts):
                                "(got a %s tensor); there is no CPU fallback" % t.device)
 
 
+def check_nonempty(who, *ts):
+    """The kernels take at least one sequence and one residue; an empty tensor is an error of the caller."""
+    for t in ts:
+        if t is not None and t.numel() == 0:
+            raise RuntimeError("%s: empty input tensor of shape %s" % (who, tuple(t.shape)))
+
+
 # ---- values derived from a mask only (key bias + tile flags of an attention, the normaliser of the outer
 # product mean) are the same in every block of a stack: inside `mask_cache()` they are computed once ----
 _MASK_CACHE = None

@@ -34,6 +34,7 @@ class Evoformer(nn.Module):
 
     # -- un-padded core on [1, s, r, c_m] / [1, r, r, c_z] / [1, s, r] / [1, r, r] ----------
     def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
+        F_.check_nonempty("Evoformer", m, z)
         if self.is_multimer:
             # multimer order (evoformer.py:70-76, 133-137): outer product mean first, the MSA stack reads the
             # pair tensor it leaves, the pair stack runs last

@@ -176,6 +176,7 @@ class ExtraMSABlock(nn.Module):
 
     def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
         """m [1, s, r, c_m], z [1, r, r, c_z] contiguous, masks [1, s, r] / [1, r, r]."""
+        F_.check_nonempty("ExtraMSABlock", m, z)
         if self.is_multimer:
             # msa.py:252-258, 321-332: outer product mean first, the MSA stack reads the pair tensor it leaves,
             # the pair stack runs last

@@ -121,6 +121,7 @@ class TemplatePairBlock(nn.Module):
 
     def _core(self, z, mask, inplace: bool):
         """z [1, r, r, c_t] contiguous, mask [1, r, r]; order as template.py:248-256."""
+        F_.check_nonempty("TemplatePairBlock", z)
         out = z if inplace else torch.empty_like(z)
         self.TriangleAttentionStartingNode._run(z, mask, out)
         self.TriangleAttentionEndingNode._run(out, mask, out)

@@ -293,3 +293,12 @@ def test_block_forward_replays_from_a_captured_graph(dev):
             assert torch.equal(gm, eager[i][0]) and torch.equal(gz, eager[i][1]), "replay with input set %d" % i
             blk(*ins[(i + 1) % 3])                          # eager work between replays
             torch.cuda.synchronize()
+
+
+def test_empty_inputs_raise(dev):
+    """No sequence or no residue is an error of the caller, reported before any launch."""
+    blk = _block(dev, torch.float32, "Evoformer")
+    for s, r in ((0, 8), (4, 0)):
+        m, z = torch.zeros(s, r, 256, device=dev), torch.zeros(r, r, 128, device=dev)
+        with torch.no_grad(), pytest.raises(RuntimeError, match="empty input"):
+            blk(m, z, torch.ones(s, r, device=dev), torch.ones(r, r, device=dev))
