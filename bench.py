@@ -130,7 +130,7 @@ def micro_ops(dev):
 def feeder_stacks(dev, r):
     """The two stacks that run before the Evoformer (hub/alphafold.py:262-362) at their own widths, random
     weights: the 4-block extra-MSA stack on 1024 extra sequences and the 2-block template pair stack on one
-    template; milliseconds per block."""
+    template, milliseconds per block; and the point-wise attention over four templates, milliseconds."""
     import torch
     from fastfold_amd.model.fastnn import ExtraMSAStack, TemplatePairStack
 
@@ -142,8 +142,11 @@ def feeder_stacks(dev, r):
                 p.copy_((1.0 if ln_w else 0.0) + 0.02 * torch.randn(p.shape, generator=g))
         return mod.to(dev, torch.bfloat16).eval()
 
-    def timed(fn, blocks, reps=2):
+    def timed(fn, blocks, reps=3):
+        # two untimed passes: the first packs the weights, the second lets the caching allocator settle on the
+        # multi-GB intermediates (a pass that still has to ask the driver for memory is host-bound)
         with torch.no_grad():
+            fn()
             fn()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -169,6 +172,14 @@ def feeder_stacks(dev, r):
     t = torch.randn(1, r, r, 64, generator=g).to(dev, torch.bfloat16)
     res["template_pair_stack"] = {"workload": "2 blocks, 1 template, N_res=%d, c_t=64" % r,
                                   "ms_per_block": timed(lambda: tp(t, pm[None], chunk_size=None), 2)}
+    del tp, t
+    from fastfold_amd.model.fastnn import TemplatePointwiseAttention
+    pw = init(TemplatePointwiseAttention(c_t=64, c_z=128, c_hidden=16, no_heads=4, inf=1e5))
+    t4 = torch.randn(4, r, r, 64, generator=g).to(dev, torch.bfloat16)
+    z = torch.randn(r, r, 128, generator=g).to(dev, torch.bfloat16)
+    tm = torch.ones(4, device=dev, dtype=torch.bfloat16)
+    res["template_pointwise_attention"] = {"workload": "4 templates, N_res=%d" % r,
+                                           "ms": timed(lambda: pw(t4, z, template_mask=tm), 1)}
     return res
 
 
