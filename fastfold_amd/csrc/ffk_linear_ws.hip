@@ -562,9 +562,9 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             s_ln1[tid] = ((const T*)d.ln_gamma)[tid];
             s_ln1[WS_K + tid] = ((const T*)d.ln_beta)[tid];
         }
-        if (ln && CM && tid < 128) {
+        if (ln && CM && tid < WS_K) {
             s_cmln[tid] = (float)((const T*)d.ln_gamma)[tid];
-            s_cmln[128 + tid] = (float)((const T*)d.ln_beta)[tid];
+            s_cmln[WS_K + tid] = (float)((const T*)d.ln_beta)[tid];
         }
         lds_barrier();
     }
@@ -577,10 +577,13 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const bool a_flat = d.a_inner >= M, a2_flat = DUAL && d.a2_inner >= M, m_flat = m_inner >= (unsigned)M;
     Vec16<T> pre[4];
     T pm[4];
-    // Channel-major A (element (m, k) at a + k * a_cs + rowoffset(m), K = 128): a thread fetches eight
-    // consecutive rows of channel k = lane % 32 + 32 i; the two half-waves of wave w own the row groups
-    // 2w and 2w + 1 of the slab, so the LayerNorm reduction over k stays inside 32 lanes.  The slab is
-    // transposed on its way into LDS (2-byte stores, consecutive lanes -> consecutive k of one row).
+    // Channel-major A (element (m, k) at a + k * a_cs + rowoffset(m), K = 128 or 64): a thread fetches eight
+    // consecutive rows of channel k = lane % 32 + 32 cb (cb < K / 32); the two half-waves of wave w own the row
+    // groups 2w and 2w + 1 of each 128-row pass of the slab (one pass at K = 128, two at K = 64), so the LayerNorm
+    // reduction over k stays inside 32 lanes.  The slab is transposed on its way into LDS (2-byte stores,
+    // consecutive lanes -> consecutive k of one row).
+    constexpr int CMI = CM ? WS_K / 32 : 4;              // channel blocks per thread
+    static_assert(!CM || WS_K == 128 || WS_K == 64, "channel-major operands are built for K = 128 and 64");
     const int cm_k = lane & 31, cm_mg = 2 * wave + (lane >> 5);
     // second operand: vector v = i * 512 + tid of a slab is row v / 16, LDS column v % 16, which holds
     // global column (v % 16) ^ (row % 16); the 16 lanes of a row are adjacent, as the LayerNorm wants them
@@ -602,12 +605,15 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             }
         }
         if (CM) {
-            long m = (long)slab * WS_BM + cm_mg * 8;
-            m = m < M ? m : M - 8;                       // M % 8 == 0; clamped groups are never stored
-            const unsigned hi = a_flat ? 0u : (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
-            const T* base = A + (long)hi * d.a_so + lo;  // a_si == 1
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pre[i] = ld16(base + (long)(cm_k + 32 * i) * d.a_cs);
+            for (int rp = 0; rp < 4 / CMI; ++rp) {
+                long m = (long)slab * WS_BM + (cm_mg + 16 * rp) * 8;
+                m = m < M ? m : M - 8;                   // M % 8 == 0; clamped groups are never stored
+                const unsigned hi = a_flat ? 0u : (unsigned)m / (unsigned)d.a_inner, lo = (unsigned)m - hi * (unsigned)d.a_inner;
+                const T* base = A + (long)hi * d.a_so + lo;  // a_si == 1
+#pragma unroll
+                for (int cb = 0; cb < CMI; ++cb) pre[rp * CMI + cb] = ld16(base + (long)(cm_k + 32 * cb) * d.a_cs);
+            }
             return;
         }
 #pragma unroll
@@ -631,7 +637,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
-                        *reinterpret_cast<T*>(sa + (cm_mg * 8 + j) * WS_AP + (cm_k + 32 * i) * 2) = pre[i].e[j];
+                        *reinterpret_cast<T*>(sa + ((cm_mg + 16 * (i / CMI)) * 8 + j) * WS_AP + (cm_k + 32 * (i % CMI)) * 2) = pre[i].e[j];
                 return;
             }
             float f[4][8];
@@ -640,31 +646,41 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 #pragma unroll
                 for (int j = 0; j < 8; ++j) f[i][j] = (float)pre[i].e[j];
             if (ln) {
-                float cm_g[4], cm_b[4];                  // gamma / beta of this lane's four channels
+                float cm_g[CMI], cm_b[CMI];              // gamma / beta of this lane's channels
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    cm_g[i] = s_cmln[(lane & 31) + 32 * i];
-                    cm_b[i] = s_cmln[128 + (lane & 31) + 32 * i];
+                for (int cb = 0; cb < CMI; ++cb) {
+                    cm_g[cb] = s_cmln[(lane & 31) + 32 * cb];
+                    cm_b[cb] = s_cmln[WS_K + (lane & 31) + 32 * cb];
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float mu = group_sum((f[0][j] + f[1][j]) + (f[2][j] + f[3][j]), 32) * (1.0f / WS_K);
-                    float q = 0.0f;
+                for (int rp = 0; rp < 4 / CMI; ++rp)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        f[i][j] -= mu;
-                        q += f[i][j] * f[i][j];
+                    for (int j = 0; j < 8; ++j) {
+                        float su = 0.0f;
+                        if (CMI == 4) {
+                            su = (f[0][j] + f[1][j]) + (f[2][j] + f[3][j]);
+                        } else {
+#pragma unroll
+                            for (int cb = 0; cb < CMI; ++cb) su += f[rp * CMI + cb][j];
+                        }
+                        const float mu = group_sum(su, 32) * (1.0f / WS_K);
+                        float q = 0.0f;
+#pragma unroll
+                        for (int cb = 0; cb < CMI; ++cb) {
+                            f[rp * CMI + cb][j] -= mu;
+                            q += f[rp * CMI + cb][j] * f[rp * CMI + cb][j];
+                        }
+                        const float rs = rsqrtf(group_sum(q, 32) * (1.0f / WS_K) + d.ln_eps);
+#pragma unroll
+                        for (int cb = 0; cb < CMI; ++cb)
+                            f[rp * CMI + cb][j] = f[rp * CMI + cb][j] * rs * cm_g[cb] + cm_b[cb];
                     }
-                    const float rs = rsqrtf(group_sum(q, 32) * (1.0f / WS_K) + d.ln_eps);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) f[i][j] = f[i][j] * rs * cm_g[i] + cm_b[i];
-                }
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    *reinterpret_cast<T*>(sa + (cm_mg * 8 + j) * WS_AP + (cm_k + 32 * i) * 2) = (T)f[i][j];
+                    *reinterpret_cast<T*>(sa + ((cm_mg + 16 * (i / CMI)) * 8 + j) * WS_AP + (cm_k + 32 * (i % CMI)) * 2) = (T)f[i][j];
             return;
         }
 #pragma unroll
@@ -1029,7 +1045,8 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->dtype != FFK_BF16 || (d->K != 64 && d->K != 128 && d->K != 256)) return 0;
     if ((d->ln_folded != 0) != (d->a2 != nullptr)) return 0;    // folded LayerNorms and the second operand go together
-    if (d->a_chanmajor && (d->K != 128 || d->a_si != 1 || d->a_inner % 8 || d->a_so % 8 || d->a_cs % 8 || d->M % 8)) return 0;
+    if (d->a_chanmajor && ((d->K != 128 && d->K != 64) || d->a_si != 1 || d->a_inner % 8 || d->a_so % 8 || d->a_cs % 8 || d->M % 8)) return 0;
+    if (d->a2 && d->K != 128) return 0;                          // the second operand is built for K = 128
     const bool k256 = d->K == 256;
     if (getenv("FFK_NO_WS")) return 0;
     bool chan_major = false, v_tiles = false;
@@ -1073,7 +1090,7 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
         *status = ws_launch<2, 128, true, true>(args, st);
     } else if (d->a_chanmajor) {
         if (args.plan.max_slots > 2 || mask_tile >= 0) return 0;
-        *status = ws_launch<2, 128, true>(args, st);
+        *status = k64 ? ws_launch<2, 64, true>(args, st) : ws_launch<2, 128, true>(args, st);
     } else if (k256) {
         *status = ws_launch<2, 256, false>(args, st);
     } else if (k64) {

@@ -184,13 +184,14 @@ def test_bias_tiles(dev, dtype, r, H):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C,with_ln", [(128, True), (64, True), (64, False)])
 @pytest.mark.parametrize("r", [40, 27, 104])
-def test_channel_major_a_with_layernorm(dev, dtype, r):
-    """Triangle-multiplication output stage: A[(i,j), c] = P[c][i][jpad]."""
+def test_channel_major_a_with_layernorm(dev, dtype, r, C, with_ln):
+    """Triangle-multiplication output stage: A[(i,j), c] = P[c][i][jpad], at the Evoformer's 128 channels and the
+    template stack's 64."""
     from fastfold_amd import _lib
-    C = 128
     jpad = (r + 7) // 8 * 8
-    g = torch.Generator().manual_seed(r)
+    g = torch.Generator().manual_seed(r + C)
     P = torch.randn(C, r, jpad, generator=g).to(dev, dtype)
     w = (torch.randn(C, C, generator=g) / C ** 0.5).to(dev, dtype)
     gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
@@ -199,12 +200,14 @@ def test_channel_major_a_with_layernorm(dev, dtype, r):
     gate = torch.rand(r * r, C, generator=g).to(dev, dtype)
     z = torch.randn(r, r, C, generator=g).to(dev, dtype)
     z0 = z.clone()
-    tiles = [_lib.make_tile(z, bias=b, resid=z, gate=gate, gate_ld=C, inner=r * r, s_i=C)]
+    tiles = [_lib.make_tile(z, bias=b, resid=z, gate=gate, gate_ld=C, inner=r * r, s_i=C, ncols=C)]
     _lib.fused_linear(P, _pack(w, 1), tiles, M=r * r, K=C, a_inner=r, a_so=jpad, a_si=1, a_chanmajor=True,
-                      a_cs=r * jpad, ln=(gam, bet))
-    x = ops_np.layer_norm(_np(P)[:, :, :r].transpose(1, 2, 0), _np(gam), _np(bet))
-    if dtype == torch.bfloat16:
-        x = _np(torch.from_numpy(x).to(torch.bfloat16))
+                      a_cs=r * jpad, ln=(gam, bet) if with_ln else None)
+    x = _np(P)[:, :, :r].transpose(1, 2, 0)
+    if with_ln:
+        x = ops_np.layer_norm(x, _np(gam), _np(bet))
+        if dtype == torch.bfloat16:
+            x = _np(torch.from_numpy(x).to(torch.bfloat16))
     ref = _np(z0) + _np(gate).reshape(r, r, C) * ops_np.linear(x, _np(w), _np(b))
     assert _rel(_np(z), ref) < TOL[dtype]
 
