@@ -271,3 +271,29 @@ def test_inject_swaps_the_pointwise_attention_too(dev):
         got = _f(e.template_pointwise_att(_t(t, dev, torch.float32), _t(z, dev, torch.float32)))
         want = ref(torch.from_numpy(t), torch.from_numpy(z)).numpy()
     assert np.abs(got - want).max() <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("P,H,D,NT", [(37, 4, 16, 4), (130, 8, 8, 3), (65, 2, 32, 8), (1, 1, 8, 1)])
+def test_pointwise_core_widths(dev, dtype, P, H, D, NT):
+    """The core at every supported head width, with strided key / value rows, against float64 torch."""
+    from fastfold_amd import _lib
+    g = torch.Generator().manual_seed(P + D)
+    hc = H * D
+    pitch = 2 * hc + 16                                   # rows padded: strides are arguments
+    q = torch.randn(P, hc, generator=g).to(dev, dtype)
+    kv = torch.randn(NT, P, pitch, generator=g).to(dev, dtype)
+    bias = torch.where(torch.rand(NT, generator=g) < 0.3, torch.tensor(-1e5), torch.tensor(0.0))
+    bias[0] = 0.0
+    o = torch.empty(P, hc, device=dev, dtype=dtype)
+    _lib.pointwise_attention_core(o, q, kv, bias.to(dev), P=P, H=H, D=D, NT=NT, kv_st=P * pitch, kv_sp=pitch, v_off=hc + 16)
+    qd = q.double().cpu().view(P, H, D)
+    kd = kv.double().cpu()[..., :hc].reshape(NT, P, H, D)
+    vd = kv.double().cpu()[..., hc + 16:2 * hc + 16].reshape(NT, P, H, D)
+    logits = torch.einsum("phd,tphd->pht", qd, kd) + bias.double()
+    want = torch.einsum("pht,tphd->phd", torch.softmax(logits, -1), vd).reshape(P, hc).numpy()
+    got = _f(o)
+    if dtype == torch.float32:
+        assert np.abs(got - want).max() <= 1e-4 * max(1.0, float(np.abs(want).max()))
+    else:
+        assert _rel_l2(got, want) <= 2e-2
