@@ -305,13 +305,15 @@ def pair_embed(out, z, gamma, beta, table, bias, row, col, *, mode, pos, edges=N
          mode, ptr(pos), ptr(edges), inf, r, C, nb, dtype_tag(out.dtype), stream_ptr())
 
 
-SIGNATURES["ffk_pointwise_attention_core"] = [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]
+SIGNATURES["ffk_pointwise_attention_core"] = [_P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]
 
 
-def pointwise_attention_core(o, q, kv, bias, *, P, H, D, NT, kv_st, kv_sp, v_off):
+def pointwise_attention_core(o, q, kv, bias, *, P, H, D, NT, kv_st, kv_sp, v_off, out_scale=None):
     """o[p, h] = softmax_t(q[p, h] . k[t, p, h] + bias[t]) v[t, p, h]; strides in elements (see include/ffk.h)."""
     check_device(o, q, kv, bias)
     if bias.dtype != torch.float32 or bias.numel() != NT:
         raise RuntimeError("pointwise_attention_core: bias must be fp32 [NT]")
-    call("ffk_pointwise_attention_core", ptr(o), ptr(q), ptr(kv), ptr(bias), P, H, D, NT, kv_st, kv_sp, v_off,
+    if out_scale is not None and (out_scale.dtype != torch.float32 or out_scale.numel() != 1 or not out_scale.is_cuda):
+        raise RuntimeError("pointwise_attention_core: out_scale must be one fp32 value on the device")
+    call("ffk_pointwise_attention_core", ptr(o), ptr(q), ptr(kv), ptr(bias), ptr(out_scale), P, H, D, NT, kv_st, kv_sp, v_off,
          dtype_tag(q.dtype), stream_ptr())

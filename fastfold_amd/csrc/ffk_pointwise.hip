@@ -1,6 +1,6 @@
 // Point-wise attention over a short axis (see ffk_pointwise_attention_core in include/ffk.h):
 // every one of P positions has its own query q[p, h, :] and T (<= 8) key / value rows kv[t, p, ...];
-//     w[p, h, t] = softmax_t( q[p, h, :] . k[t, p, h, :] + bias[t] ),   o[p, h, :] = sum_t w[p, h, t] v[t, p, h, :].
+//     w[p, h, t] = softmax_t( q[p, h, :] . k[t, p, h, :] + bias[t] ),   o[p, h, :] = scale * sum_t w[p, h, t] v[t, p, h, :].
 // The op is a stream: each element is read once, so one thread owns one (position, head) pair, keeps its
 // D-element query and the T logits in registers and walks the T key and value rows with 16-byte loads;
 // neighbouring threads read neighbouring 2 D-byte pieces of a row.
@@ -14,7 +14,8 @@ constexpr int PW_MAXT = 8;
 template <typename T, int D>
 __global__ __launch_bounds__(PW_THREADS) void pointwise_attention_kernel(T* __restrict__ o, const T* __restrict__ q,
                                                                          const T* __restrict__ kv,
-                                                                         const float* __restrict__ bias, long P, int H,
+                                                                         const float* __restrict__ bias,
+                                                                         const float* __restrict__ out_scale, long P, int H,
                                                                          int NT, long kv_st, long kv_sp, int v_off) {
     constexpr int VEC = DT<T>::VEC;
     constexpr int NV = D / VEC;                       // 16-byte vectors per head slice
@@ -53,7 +54,7 @@ __global__ __launch_bounds__(PW_THREADS) void pointwise_attention_kernel(T* __re
         logit[t] = t < NT ? __expf(logit[t] - mx) : 0.0f;
         sum += logit[t];
     }
-    const float inv = 1.0f / sum;
+    const float inv = (out_scale ? *out_scale : 1.0f) / sum;      // the optional device scalar rides on the normaliser
     float acc[D];
 #pragma unroll
     for (int j = 0; j < D; ++j) acc[j] = 0.0f;
@@ -80,14 +81,14 @@ __global__ __launch_bounds__(PW_THREADS) void pointwise_attention_kernel(T* __re
 }
 
 template <typename T>
-int pw_launch(void* o, const void* q, const void* kv, const float* bias, long P, int H, int D, int NT, long kv_st,
-              long kv_sp, int v_off, hipStream_t st) {
+int pw_launch(void* o, const void* q, const void* kv, const float* bias, const float* out_scale, long P, int H, int D,
+              int NT, long kv_st, long kv_sp, int v_off, hipStream_t st) {
     const long total = P * H;
     const unsigned grid = (unsigned)ffk_cdiv(total, PW_THREADS);
 #define PW_CASE(DD)                                                                                                    \
     case DD:                                                                                                           \
-        pointwise_attention_kernel<T, DD><<<grid, PW_THREADS, 0, st>>>((T*)o, (const T*)q, (const T*)kv, bias, P, H, NT, \
-                                                                       kv_st, kv_sp, v_off);                           \
+        pointwise_attention_kernel<T, DD><<<grid, PW_THREADS, 0, st>>>((T*)o, (const T*)q, (const T*)kv, bias, out_scale, P, \
+                                                                       H, NT, kv_st, kv_sp, v_off);                           \
         break;
     switch (D) {
         PW_CASE(8)
@@ -101,9 +102,9 @@ int pw_launch(void* o, const void* q, const void* kv, const float* bias, long P,
 
 }  // namespace
 
-extern "C" int ffk_pointwise_attention_core(void* o, const void* q, const void* kv, const float* bias, int64_t P, int64_t H,
-                                            int64_t D, int64_t NT, int64_t kv_st, int64_t kv_sp, int64_t v_off, int dtype,
-                                            void* stream) {
+extern "C" int ffk_pointwise_attention_core(void* o, const void* q, const void* kv, const float* bias, const float* out_scale,
+                                            int64_t P, int64_t H, int64_t D, int64_t NT, int64_t kv_st, int64_t kv_sp,
+                                            int64_t v_off, int dtype, void* stream) {
     FFK_REQUIRE(o && q && kv && bias, FFK_ERR_NULL, "ffk_pointwise_attention_core: null pointer");
     FFK_REQUIRE(P > 0 && H > 0 && H <= 64 && NT > 0 && NT <= PW_MAXT && P * H < (1L << 31) * (long)PW_THREADS, FFK_ERR_SHAPE,
                 "ffk_pointwise_attention_core: bad shape P=%ld H=%ld NT=%ld (1 <= NT <= %d)", (long)P, (long)H, (long)NT,
@@ -120,6 +121,6 @@ extern "C" int ffk_pointwise_attention_core(void* o, const void* q, const void* 
                 "ffk_pointwise_attention_core: a key / value row needs v_off >= H*D and kv_sp >= v_off + H*D");
     hipStream_t st = (hipStream_t)stream;
     if (dtype == FFK_BF16)
-        return pw_launch<bf16_t>(o, q, kv, bias, (long)P, (int)H, (int)D, (int)NT, (long)kv_st, (long)kv_sp, (int)v_off, st);
-    return pw_launch<float>(o, q, kv, bias, (long)P, (int)H, (int)D, (int)NT, (long)kv_st, (long)kv_sp, (int)v_off, st);
+        return pw_launch<bf16_t>(o, q, kv, bias, out_scale, (long)P, (int)H, (int)D, (int)NT, (long)kv_st, (long)kv_sp, (int)v_off, st);
+    return pw_launch<float>(o, q, kv, bias, out_scale, (long)P, (int)H, (int)D, (int)NT, (long)kv_st, (long)kv_sp, (int)v_off, st);
 }

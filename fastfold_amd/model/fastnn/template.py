@@ -68,14 +68,14 @@ class TemplatePointwiseAttention(nn.Module, _PackMixin):
             template_mask = t.new_ones(NT)
         tm = template_mask.to(device=dev, dtype=torch.float32).reshape(NT)
         bias = (self.inf * (tm - 1.0)).contiguous()
-        any_valid = (tm.sum() > 0).to(dt)                                  # stays on the device: no host round trip
+        any_valid = (tm.sum() > 0).to(torch.float32).reshape(1)            # stays on the device: no host round trip
         q = F_.linear(z.contiguous().view(P, self.c_z), wq, None, hc)
         kv = F_.linear(t.contiguous().view(NT * P, self.c_t), wkv, None, 2 * hc)
         o = torch.empty(P, hc, dtype=dt, device=dev)
-        _lib.pointwise_attention_core(o, q, kv, bias, P=P, H=H, D=D, NT=NT, kv_st=P * 2 * hc, kv_sp=2 * hc, v_off=hc)
+        _lib.pointwise_attention_core(o, q, kv, bias, P=P, H=H, D=D, NT=NT, kv_st=P * 2 * hc, kv_sp=2 * hc, v_off=hc,
+                                      out_scale=any_valid)
         del q, kv
-        o.mul_(any_valid)
-        out = F_.linear(o, wo, bo * any_valid, self.c_z, out=resid, resid=resid)     # in place when a residual is given
+        out = F_.linear(o, wo, (bo * any_valid).to(dt), self.c_z, out=resid, resid=resid)   # in place with a residual
         return out.view(r, r, self.c_z)
 
     def forward(self, t: torch.Tensor, z: torch.Tensor, template_mask: Optional[torch.Tensor] = None,

@@ -336,13 +336,14 @@ int ffk_pair_embed(void* out, const void* z, const void* ln_gamma, const void* l
  *     w[p, h, t] = softmax_t( q[p, h, :] . k[t, p, h, :] + bias[t] ),   o[p, h, :] = sum_t w[p, h, t] v[t, p, h, :]
  * q, o : [P, H * D] (q already scaled by 1 / sqrt(D)); kv : row (t, p) starts at kv + t * kv_st + p * kv_sp
  * (elements) and holds the H * D key channels at offset 0 and the H * D value channels at offset v_off;
- * bias : [NT] fp32 (inf * (template_mask - 1)); 1 <= NT <= 8; D in {8, 16, 32}; fp32 or bf16.
+ * bias : [NT] fp32 (inf * (template_mask - 1)); out_scale : NULL or one fp32 value on the device that multiplies
+ * o (0 when no template is valid: the reference zeroes the update then); 1 <= NT <= 8; D in {8, 16, 32}; fp32 or bf16.
  * Replaces: the softmax(q k^T + bias) v core of TemplatePointwiseAttention.forward, where the reference calls
  * its generic Attention module on a [N_res, N_res, 1, C_z] query and [N_res, N_res, N_templ, C_t] keys
  * (fastfold/model/fastnn/template.py:83-131; nn/template.py:95-133; nn/primitives.py:344-419). */
-int ffk_pointwise_attention_core(void* o, const void* q, const void* kv, const float* bias, int64_t P, int64_t H,
-                                 int64_t D, int64_t NT, int64_t kv_st, int64_t kv_sp, int64_t v_off, int dtype,
-                                 void* stream);
+int ffk_pointwise_attention_core(void* o, const void* q, const void* kv, const float* bias, const float* out_scale,
+                                 int64_t P, int64_t H, int64_t D, int64_t NT, int64_t kv_st, int64_t kv_sp, int64_t v_off,
+                                 int dtype, void* stream);
 
 /* keybias[b, k] = mask[b, k] != 0 ? 0 : -1e9*log2(e) for k < N, and -3e38 for N <= k < Npad
  * (Npad = ceil(N/32)*32).  mask is [B, N] with strides (mask_sb, mask_sn) in elements of the

@@ -286,12 +286,13 @@ def test_pointwise_core_widths(dev, dtype, P, H, D, NT):
     bias = torch.where(torch.rand(NT, generator=g) < 0.3, torch.tensor(-1e5), torch.tensor(0.0))
     bias[0] = 0.0
     o = torch.empty(P, hc, device=dev, dtype=dtype)
-    _lib.pointwise_attention_core(o, q, kv, bias.to(dev), P=P, H=H, D=D, NT=NT, kv_st=P * pitch, kv_sp=pitch, v_off=hc + 16)
+    _lib.pointwise_attention_core(o, q, kv, bias.to(dev), P=P, H=H, D=D, NT=NT, kv_st=P * pitch, kv_sp=pitch, v_off=hc + 16,
+                                  out_scale=torch.full((1,), 0.5, device=dev))
     qd = q.double().cpu().view(P, H, D)
     kd = kv.double().cpu()[..., :hc].reshape(NT, P, H, D)
     vd = kv.double().cpu()[..., hc + 16:2 * hc + 16].reshape(NT, P, H, D)
     logits = torch.einsum("phd,tphd->pht", qd, kd) + bias.double()
-    want = torch.einsum("pht,tphd->phd", torch.softmax(logits, -1), vd).reshape(P, hc).numpy()
+    want = 0.5 * torch.einsum("pht,tphd->phd", torch.softmax(logits, -1), vd).reshape(P, hc).numpy()
     got = _f(o)
     if dtype == torch.float32:
         assert np.abs(got - want).max() <= 1e-4 * max(1.0, float(np.abs(want).max()))
