@@ -147,7 +147,7 @@ class LinearDesc(ctypes.Structure):
         ("w", c_void_p),
         ("M", c_int), ("K", c_int), ("n_tiles", c_int), ("ln_folded", c_int),
         ("a2", c_void_p), ("ln2_gamma", c_void_p), ("ln2_beta", c_void_p),
-        ("a2_so", c_int64), ("a2_si", c_int64), ("a2_inner", c_int), ("reserved2", c_int),
+        ("a2_so", c_int64), ("a2_si", c_int64), ("a2_inner", c_int), ("variant", c_int),
         ("tiles", Tile * FFK_MAX_TILES),
     ]
 
@@ -172,7 +172,7 @@ def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, g
 
 def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanmajor=False, a_cs=0,
                  ln=None, eps=1e-5, a_off=0, w_row_off=0, a2=None, ln2=None, a2_inner=None, a2_so=0, a2_si=None,
-                 ln_rowsums=None):
+                 ln_rowsums=None, staged=False):
     """Launches ``ffk_fused_linear``.  ``a`` / ``w`` are tensors (``w`` packed [>= n_tiles*128, K]);
     ``ln`` is ``(gamma, beta)`` or None; ``a_off`` (elements) / ``w_row_off`` (rows) offset the bases.
     ``a2`` is the second operand the gate halves of GLU tiles are computed from; it goes with ``ln_rowsums``
@@ -195,6 +195,7 @@ def fused_linear(a, w, tiles, *, M, K, a_inner=None, a_so=0, a_si=None, a_chanma
     d.dtype = dtype_tag(a.dtype)
     d.w = w.data_ptr() + w_row_off * K * w.element_size()
     d.M, d.K, d.n_tiles = M, K, len(tiles)
+    d.variant = 1 if staged else 0      # FFK_LINEAR_STAGED: the LDS-staged kernels even where the weights-stationary one applies
     if a2 is not None:
         if ln_rowsums is None:
             raise RuntimeError("fused_linear: a second operand needs folded LayerNorms (ln_rowsums)")

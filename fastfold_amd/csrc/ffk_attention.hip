@@ -396,13 +396,10 @@ template <typename T, bool HAS_BIAS>
 int launch_attention_b(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
                        const int* flags, const void* gate, long B2, long H, long Nq, long Nk, int aflags, hipStream_t st) {
     const size_t smem = (3 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 + ATT_THREADS * 16) * sizeof(T);   // operand ring + gate
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)attention_kernel<T, HAS_BIAS>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_attention_fwd: cannot reserve %zu B of LDS: %s", smem,
-                                             hipGetErrorString(e));
-        configured = true;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)attention_kernel<T, HAS_BIAS>, smem, "ffk_attention_fwd");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     const long items = (long)ffk_cdiv((Nq + 31) / 32, 4) * H * ffk_cdiv(B2, 2);
     FFK_REQUIRE(items < (1L << 31) - 8, FFK_ERR_SHAPE, "ffk_attention_fwd: %ld workgroups exceed the grid limit", items);

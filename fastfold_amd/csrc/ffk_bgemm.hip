@@ -235,13 +235,10 @@ int launch_bgemm(const ffk_bgemm_desc& d, hipStream_t st) {
     size_t ring = 4 * (size_t)BT * (128 + 16);
     size_t ct = (size_t)BT * (BT * sizeof(OT) + 16);
     const size_t smem = ring > ct ? ring : ct;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)bgemm_nt_kernel<T, OT>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_bgemm_nt: cannot reserve %zu B of LDS: %s", smem,
-                                             hipGetErrorString(e));
-        configured = true;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)bgemm_nt_kernel<T, OT>, smem, "ffk_bgemm_nt");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     const long tiles = (long)ffk_cdiv(d.M, BT) * ffk_cdiv(d.N, BT) * d.batch;
     FFK_REQUIRE(tiles < (1L << 31) - 8, FFK_ERR_SHAPE, "ffk_bgemm_nt: %ld output tiles exceed the grid limit", tiles);

@@ -249,11 +249,10 @@ template <int WTN>
 int bg_launch(const ffk_bgemm_desc& d, hipStream_t st) {
     constexpr int BM = 256, BN = 2 * WTN;
     const size_t smem = (size_t)BG_SLOTS * (BM + BN) * 64;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)bgemm_big_kernel<WTN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_bgemm_nt: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
-        configured = true;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)bgemm_big_kernel<WTN>, smem, "ffk_bgemm_nt");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     const long tiles = (long)ffk_cdiv(d.M, BM) * ffk_cdiv(d.N, BN) * d.batch;
     if (tiles >= (1L << 31) - 8) return ffk_fail(FFK_ERR_SHAPE, "ffk_bgemm_nt: %ld output tiles exceed the grid limit", tiles);
@@ -267,7 +266,6 @@ int bg_launch(const ffk_bgemm_desc& d, hipStream_t st) {
 // Launches the large-tile kernel if it can take this (already validated) descriptor and returns 1 with
 // the launch status in *status; returns 0 if the caller has to use the small-tile kernel.
 int ffk_bgemm_big_try(const ffk_bgemm_desc* d, hipStream_t st, int* status) {
-    if (getenv("FFK_NO_BIG")) return 0;
     if (d->dtype != FFK_BF16 || d->out_f32 || d->K % BG_BK != 0 || d->K < 3 * BG_BK || d->s_d != 1) return 0;
     if (d->M < 256 || d->N < 64 || d->N % 16 != 0) return 0;
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };

@@ -8,6 +8,8 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <atomic>
+#include <mutex>
 
 #include "../../include/ffk.h"
 
@@ -23,6 +25,29 @@ int ffk_fail(int code, const char* fmt, ...);
 int ffk_linear_slab_launch(const ffk_linear_desc* d, hipStream_t st);   // ffk_linear_slab.hip
 int ffk_bgemm_big_try(const ffk_bgemm_desc* d, hipStream_t st, int* status);    // ffk_bgemm_big.hip
 int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status);   // ffk_linear_ws.hip
+
+// Dynamic-LDS reservation of one kernel: hipFuncSetAttribute is needed once per device (again only if a
+// later launch asks for more).  A function-scope `static FfkLdsReservation` (zero-initialised) remembers, per
+// device, what has been reserved; the slow path is serialised so that concurrent first calls from several host
+// threads cannot leave a smaller reservation behind than the one recorded.
+constexpr int FFK_MAX_DEVICES = 64;
+struct FfkLdsReservation {
+    std::atomic<size_t> bytes[FFK_MAX_DEVICES];
+};
+std::mutex& ffk_config_mutex();    // ffk_rowops.hip
+static inline int ffk_reserve_lds(FfkLdsReservation& r, const void* func, size_t smem, const char* what) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+    if (dev < 0 || dev >= FFK_MAX_DEVICES) return ffk_fail(FFK_ERR_UNSUPPORTED, "%s: device ordinal %d not supported", what, dev);
+    if (smem <= r.bytes[dev].load(std::memory_order_acquire)) return FFK_OK;
+    std::lock_guard<std::mutex> lock(ffk_config_mutex());
+    if (smem <= r.bytes[dev].load(std::memory_order_relaxed)) return FFK_OK;
+    e = hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "%s: cannot reserve %zu B of LDS: %s", what, smem, hipGetErrorString(e));
+    r.bytes[dev].store(smem, std::memory_order_release);
+    return FFK_OK;
+}
 
 static inline bool ffk_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

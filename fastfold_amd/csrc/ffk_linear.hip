@@ -445,13 +445,10 @@ int launch_linear(const ffk_linear_desc& d, hipStream_t st) {
     size_t ct = (size_t)NT * (Cfg::BM * ES + 16);
     if (ct > ring) ring = ct;
     const size_t smem = (size_t)Cfg::BM * (d.K * ES + 16) + ring;
-    static size_t configured = 0;
-    if (smem > configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<T>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem,
-                                             hipGetErrorString(e));
-        configured = smem;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)fused_linear_kernel<T>, smem, "ffk_fused_linear");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     LinArgs a;
     a.d = d;

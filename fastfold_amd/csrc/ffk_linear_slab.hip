@@ -494,13 +494,10 @@ __global__ __launch_bounds__(THREADS, 2) void fused_linear_slab_kernel(const Lin
 
 template <typename T, int NA>
 int launch_linear_na(const ffk_linear_desc& d, size_t smem, hipStream_t st) {
-    static size_t configured = 0;
-    if (smem > configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)fused_linear_slab_kernel<T, NA>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem,
-                                             hipGetErrorString(e));
-        configured = smem;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)fused_linear_slab_kernel<T, NA>, smem, "ffk_fused_linear");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     LinArgs a;
     a.d = d;

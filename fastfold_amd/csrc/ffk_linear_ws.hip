@@ -1025,12 +1025,10 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
     const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float) +
                         (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) + FFK_MAX_TILES * 128 * sizeof(float) : 0) +
                         (CM ? 256 * sizeof(float) : 2 * K * sizeof(T));
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)linear_ws_kernel<NS, K, CM, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess)
-            return ffk_fail(FFK_ERR_LAUNCH, "ffk_fused_linear: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
-        configured = true;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)linear_ws_kernel<NS, K, CM, DUAL>, smem, "ffk_fused_linear");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     const int nslabs = ffk_cdiv(args.d.M, WS_BM);
     const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
@@ -1048,7 +1046,7 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->a_chanmajor && ((d->K != 128 && d->K != 64) || d->a_si != 1 || d->a_inner % 8 || d->a_so % 8 || d->a_cs % 8 || d->M % 8)) return 0;
     if (d->a2 && d->K != 128) return 0;                          // the second operand is built for K = 128
     const bool k256 = d->K == 256;
-    if (getenv("FFK_NO_WS")) return 0;
+    if (d->variant == FFK_LINEAR_STAGED) return 0;
     bool chan_major = false, v_tiles = false;
     int mask_tile = -1;
     for (int i = 0; i < d->n_tiles; ++i) {

@@ -190,11 +190,10 @@ template <int KS1>
 int opm_launch(T* out, const T* resid, const T* at, const T* bt, const T* w2p, const T* bias, const float* norm, int r,
                float eps, hipStream_t st) {
     const size_t smem = 2 * (size_t)OP_A2 + 3 * OP_W2SLOT + 2 * (size_t)(OP_TJ * OP_EC * KS1 * 32);
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)opm_fused_kernel<KS1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_opm_fused: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
-        configured = true;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)opm_fused_kernel<KS1>, smem, "ffk_opm_fused");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     const unsigned grid = (unsigned)((r / OP_TI) * (r / OP_TJ));
     opm_fused_kernel<KS1><<<grid, OP_THREADS, smem, st>>>(out, resid, at, bt, w2p, bias, norm, r, eps);

@@ -140,42 +140,45 @@ __global__ void pair_bias_prep_kernel(bf16_t* wop, float* c01, const bf16_t* w, 
     }
 }
 
-}  // namespace
-
-extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w, float* scratch,
-                             int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so, int64_t a_si, float scale,
-                             float eps, int dtype, void* stream) {
-    FFK_REQUIRE(bias_t && z && scratch && (!w || (gamma && beta)), FFK_ERR_NULL, "ffk_pair_bias: null pointer");
-    FFK_REQUIRE(dtype == FFK_BF16, FFK_ERR_DTYPE, "ffk_pair_bias: bf16 only (dtype tag %d)", dtype);
-    FFK_REQUIRE(C == 128 || C == 64, FFK_ERR_UNSUPPORTED, "ffk_pair_bias: built for 64 or 128 pair channels, got %ld", (long)C);
+// Validates, builds the weight operand in `scratch` (unless w == NULL) and launches.  Shared by both entry points.
+int pair_bias_run(const char* who, void* bias_t, const void* z, const void* gamma, const void* beta, const void* w,
+                  float* scratch, int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so, int64_t a_si, float scale,
+                  float eps, int dtype, hipStream_t st) {
+    FFK_REQUIRE(bias_t && z && scratch && (!w || (gamma && beta)), FFK_ERR_NULL, "%s: null pointer", who);
+    FFK_REQUIRE(dtype == FFK_BF16, FFK_ERR_DTYPE, "%s: bf16 only (dtype tag %d)", who, dtype);
+    FFK_REQUIRE(C == 128 || C == 64, FFK_ERR_UNSUPPORTED, "%s: built for 64 or 128 pair channels, got %ld", who, (long)C);
     FFK_REQUIRE(N > 0 && N <= 46340 && H > 0 && H <= PB_MAXH && a_inner > 0, FFK_ERR_SHAPE,
-                "ffk_pair_bias: bad shape N=%ld H=%ld a_inner=%ld", (long)N, (long)H, (long)a_inner);
+                "%s: bad shape N=%ld H=%ld a_inner=%ld (at most %d heads)", who, (long)N, (long)H, (long)a_inner, PB_MAXH);
     FFK_REQUIRE(ffk_aligned16(z) && ffk_aligned16(scratch) && a_so % 8 == 0 && a_si % 8 == 0, FFK_ERR_ALIGN,
-                "ffk_pair_bias: rows of z must be 16-byte aligned");
-    hipStream_t st = (hipStream_t)stream;
+                "%s: rows of z must be 16-byte aligned", who);
     bf16_t* wop = reinterpret_cast<bf16_t*>(scratch);     // [32][C] bf16 = 16 * C floats
     float* c01 = scratch + 16 * C;                       // [H][2]
     if (w) {       // w == NULL: scratch still holds the operand an earlier call built from the same w, gamma, beta
         pair_bias_prep_kernel<<<32, 64, 0, st>>>(wop, c01, (const bf16_t*)w, (const bf16_t*)gamma, (const bf16_t*)beta,
                                                  (int)H, (int)C);
-        int rc = ffk_check_launch("ffk_pair_bias");
+        int rc = ffk_check_launch(who);
         if (rc != FFK_OK) return rc;
     }
     const unsigned T = (unsigned)((N + 31) / 32);
 #define PB_LAUNCH(CC)                                                                                                   \
     {                                                                                                                   \
         const size_t smem = 256 * (CC * 2 + 16) + 256 * sizeof(float);                                                  \
-        static bool configured = false;                                                                                 \
-        if (!configured) {                                                                                              \
-            hipError_t e = hipFuncSetAttribute((const void*)pair_bias_kernel<CC>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                               (int)smem);                                                              \
-            if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_pair_bias: cannot reserve LDS: %s", hipGetErrorString(e)); \
-            configured = true;                                                                                          \
-        }                                                                                                               \
+        static FfkLdsReservation lds_reserved;                                                                          \
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)pair_bias_kernel<CC>, smem, who);                 \
+        if (rc_lds != FFK_OK) return rc_lds;                                                                            \
         pair_bias_kernel<CC><<<dim3(T, T), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wop, c01, (int)N, \
                                                                    (int)H, (int)a_inner, a_so, a_si, scale, eps);       \
     }
     if (C == 128) PB_LAUNCH(128) else PB_LAUNCH(64)
 #undef PB_LAUNCH
-    return ffk_check_launch("ffk_pair_bias");
+    return ffk_check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w, float* scratch,
+                             int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so, int64_t a_si, float scale,
+                             float eps, int dtype, void* stream) {
+    return pair_bias_run("ffk_pair_bias", bias_t, z, gamma, beta, w, scratch, N, C, H, a_inner, a_so, a_si, scale, eps, dtype,
+                         (hipStream_t)stream);
 }

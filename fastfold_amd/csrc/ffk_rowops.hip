@@ -17,7 +17,12 @@ int ffk_fail(int code, const char* fmt, ...) {
     return code;
 }
 
-extern "C" int ffk_version(void) { return 100; }
+std::mutex& ffk_config_mutex() {
+    static std::mutex m;
+    return m;
+}
+
+extern "C" int ffk_version(void) { return 110; }
 extern "C" const char* ffk_last_error_string(void) { return ffk_err_buf; }
 
 namespace {
@@ -31,13 +36,9 @@ constexpr float MASK_FILL = -1e9f;
 struct RowGeom {
     int lpr, vpl;
 };
-static int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : dflt;
-}
 static bool row_geom(long nvec, RowGeom* g) {
-    static const int min_lpr = env_int("FFK_ROW_LPR", 8);
-    static const int tgt_vpl = env_int("FFK_ROW_VPL", 4);
+    constexpr int min_lpr = 8;
+    constexpr int tgt_vpl = 4;
     int lpr = min_lpr;   // >= 8 lanes x 16 B: every wave-level access covers whole 128-byte lines
     while (lpr < 64 && (long)lpr * tgt_vpl < nvec) lpr <<= 1;
     long vpl = (nvec + lpr - 1) / lpr;
@@ -52,7 +53,7 @@ static bool row_geom(long nvec, RowGeom* g) {
 static int row_grid(long rows, int lpr) {
     long rows_per_block = (long)WAVES_PER_BLOCK * (64 / lpr);
     long blocks = (rows + rows_per_block - 1) / rows_per_block;
-    static const long cap = 256L * env_int("FFK_ROW_CAP", 16);   // 256 CUs x resident blocks; grid-stride beyond
+    constexpr long cap = 256L * 16;   // 256 CUs x resident blocks; grid-stride beyond
     return (int)(blocks < cap ? blocks : cap);
 }
 
@@ -187,7 +188,7 @@ int softmax_launch(T* out, const T* x, const T* mask, const T* bias, long rows, 
                         (!mask || ffk_aligned16(mask)) && (!bias || ffk_aligned16(bias)) &&
                         row_geom(cols / VEC, &g);
     if (vec_ok) {
-        static const bool nts = env_int("FFK_ROW_NT", 1) != 0;
+        constexpr bool nts = true;
         dim3 grid(row_grid(rows, g.lpr));
         switch (g.vpl) {
             case 1: (nts ? softmax_vec_kernel<T, 1, true><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq) : softmax_vec_kernel<T, 1, false><<<grid, BLOCK, 0, st>>>(out, x, mask, bias, rows, (int)cols, g.lpr, hq)); break;
@@ -383,7 +384,7 @@ int layernorm_launch(T* out, float* mean, float* rstd, const T* x, const T* gamm
     const bool vec_ok = cols % VEC == 0 && ffk_aligned16(out) && ffk_aligned16(x) && ffk_aligned16(gamma) &&
                         ffk_aligned16(beta) && row_geom(cols / VEC, &g);
     if (vec_ok) {
-        static const bool nts = env_int("FFK_ROW_NT", 1) != 0;
+        constexpr bool nts = true;
         dim3 grid(row_grid(rows, g.lpr));
         switch (g.vpl) {
             case 1: (nts ? layernorm_vec_kernel<T, 1, true><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps) : layernorm_vec_kernel<T, 1, false><<<grid, BLOCK, 0, st>>>(out, mean, rstd, x, gamma, beta, rows, (int)cols, g.lpr, eps)); break;

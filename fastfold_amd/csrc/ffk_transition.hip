@@ -208,11 +208,10 @@ extern "C" int ffk_transition_fused(void* out, const void* x, const void* gamma,
                     ffk_aligned16(w2) && ffk_aligned16(b2),
                 FFK_ERR_ALIGN, "ffk_transition_fused: buffers must be 16-byte aligned");
     const size_t smem = 2 * (size_t)TR_W1SLOT + 2 * TR_W2SLOT + TR_H * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)transition_fused_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_transition_fused: cannot reserve %zu B of LDS: %s", smem, hipGetErrorString(e));
-        configured = true;
+    static FfkLdsReservation lds_reserved;
+    {
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel, smem, "ffk_transition_fused");
+        if (rc_lds != FFK_OK) return rc_lds;
     }
     const unsigned grid = (unsigned)ffk_cdiv(M, TR_BM);
     transition_fused_kernel<<<grid, TR_THREADS, smem, (hipStream_t)stream>>>((T*)out, (const T*)x, (const T*)gamma, (const T*)beta,

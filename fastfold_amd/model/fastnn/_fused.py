@@ -77,7 +77,7 @@ def mask_cache():
     (storage, view geometry, version) and reused.  Entries keep their mask alive, so its memory cannot be
     handed to another tensor while the entry exists; the cache dies with the context."""
     global _MASK_CACHE
-    prev, _MASK_CACHE = _MASK_CACHE, (None if os.environ.get("FFK_NO_MASK_CACHE") else [])
+    prev, _MASK_CACHE = _MASK_CACHE, []
     try:
         yield
     finally:
@@ -318,8 +318,6 @@ def pack_trimul_out(out_w, out_b, og_w, og_b, C, dtype, device, ln_p, ln_z):
 def trimul_gate_in_output_stage(dtype, r, C, c):
     """The output gate sigmoid(Wg LN(z) + bg) can be computed inside the output stage (second operand
     of the projection kernel) instead of being written by the first stage and read back."""
-    if os.environ.get("FFK_NO_WS") or os.environ.get("FFK_TRIMUL_GATE_FIRST"):    # debugging knobs: the two-pass form
-        return False
     return dtype == torch.bfloat16 and C == 128 and c == 128 and r % 8 == 0
 
 

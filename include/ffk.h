@@ -137,6 +137,7 @@ int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const 
  */
 enum { FFK_TILE_STRIDED = 0, FFK_TILE_QK = 1, FFK_TILE_V = 2, FFK_TILE_BIAS = 3, FFK_TILE_ACC = 4 };
 enum { FFK_ACT_NONE = 0, FFK_ACT_RELU = 1, FFK_ACT_SIGMOID = 2 };
+enum { FFK_LINEAR_AUTO = 0, FFK_LINEAR_STAGED = 1 };
 #define FFK_MAX_TILES 10
 
 typedef struct ffk_tile {
@@ -190,7 +191,9 @@ typedef struct ffk_linear_desc {
     const void* ln2_gamma;
     const void* ln2_beta;
     int64_t a2_so, a2_si;
-    int32_t a2_inner, reserved2;
+    int32_t a2_inner;
+    int32_t variant;       /* FFK_LINEAR_AUTO, or FFK_LINEAR_STAGED to force the LDS-staged kernels (used by tests that
+                              compare the kernel variants with each other) */
     ffk_tile tiles[FFK_MAX_TILES];
 } ffk_linear_desc;
 

@@ -272,7 +272,7 @@ def test_weights_stationary_many_slabs(dev):
     assert _rel(_np(plain).reshape(B2, N, C), np.maximum(lin[4] + _np(bias_r), 0)) < TOL[dtype]
 
 
-def test_weights_stationary_matches_other_variant(dev, monkeypatch):
+def test_weights_stationary_matches_other_variant(dev):
     """GLU + row mask, channel-major store, both traversal orders, at a multi-slab size: the
     weights-stationary kernel and the LDS-staged kernel must agree to bf16 rounding."""
     from fastfold_amd import _lib
@@ -287,8 +287,6 @@ def test_weights_stationary_matches_other_variant(dev, monkeypatch):
     mask = (torch.rand(r, r, generator=g) > 0.2).to(dev, dtype)
     outs = []
     for no_ws in (False, True):
-        if no_ws:
-            monkeypatch.setenv("FFK_NO_WS", "1")
         res = []
         for transposed in (False, True):
             out = torch.zeros(Ch, r, r, dtype=dtype, device=dev)
@@ -301,10 +299,9 @@ def test_weights_stationary_matches_other_variant(dev, monkeypatch):
             kw = dict(inner=r, s_o=C, s_i=r * C) if transposed else dict(inner=r * r, s_i=C)
             tiles.append(_lib.make_tile(gate, bias=bpk.data_ptr() + 2 * 128 * 2, act=_lib.FFK_ACT_SIGMOID, **kw))
             akw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else {}
-            _lib.fused_linear(z, wpk, tiles, M=r * r, K=C, ln=(gam, bet), **akw)
+            _lib.fused_linear(z, wpk, tiles, M=r * r, K=C, ln=(gam, bet), staged=no_ws, **akw)
             res += [out, gate]
         outs.append(res)
-    monkeypatch.delenv("FFK_NO_WS")
     for a, b in zip(*outs):
         assert float(a.float().abs().max()) > 0.1
         assert _rel(_np(a), _np(b)) < 1e-2
