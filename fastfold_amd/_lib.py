@@ -266,6 +266,15 @@ def pair_bias(bias_t, z, gamma, beta, w, scratch, *, N, C, H, a_inner, a_so, a_s
          scale, eps, dtype_tag(z.dtype), stream_ptr())
 
 
+SIGNATURES["ffk_pair_bias_static"] = [_P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _F, _F, _I, _P]
+
+
+def pair_bias_static(bias_t, z, gamma, beta, w, *, N, C, H, a_inner, a_so, a_si, scale, eps=1e-5):
+    """``ffk_pair_bias`` without a scratch tensor: the library's per-GPU static array holds the weight operand."""
+    call("ffk_pair_bias_static", ptr(bias_t), ptr(z), ptr(gamma), ptr(beta), ptr(w), N, C, H, a_inner, a_so, a_si,
+         scale, eps, dtype_tag(z.dtype), stream_ptr())
+
+
 SIGNATURES["ffk_opm_fused"] = [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _P]
 
 

@@ -174,6 +174,37 @@ int pair_bias_run(const char* who, void* bias_t, const void* z, const void* gamm
     return ffk_check_launch(who);
 }
 
+// ---- the scratch of ffk_pair_bias_static: the weight operand [32][C <= 128] bf16 + [8][2] fp32 constants ----
+constexpr int PB_STATIC_MAX_C = 128;
+constexpr int PB_STATIC_FLOATS = 16 * PB_STATIC_MAX_C + 2 * PB_MAXH;      // 8 256 bytes per device
+static __device__ __align__(256) float pb_static_scratch[PB_STATIC_FLOATS];
+
+// Device address of this device's copy of pb_static_scratch, looked up once per device (the array's name is only
+// a host-side handle: it must never be passed to a kernel or to a memory routine).
+int pb_static_ptr(float** out) {
+    static std::atomic<float*> ptrs[FFK_MAX_DEVICES];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return ffk_fail(FFK_ERR_LAUNCH, "ffk_pair_bias_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= FFK_MAX_DEVICES)
+        return ffk_fail(FFK_ERR_UNSUPPORTED, "ffk_pair_bias_static: device ordinal %d not supported", dev);
+    float* p = ptrs[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(ffk_config_mutex());
+        p = ptrs[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            void* sym = nullptr;
+            e = hipGetSymbolAddress(&sym, HIP_SYMBOL(pb_static_scratch));
+            if (e != hipSuccess || !sym)
+                return ffk_fail(FFK_ERR_LAUNCH, "ffk_pair_bias_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            p = static_cast<float*>(sym);
+            ptrs[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return FFK_OK;
+}
+
 }  // namespace
 
 extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w, float* scratch,
@@ -181,4 +212,19 @@ extern "C" int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, con
                              float eps, int dtype, void* stream) {
     return pair_bias_run("ffk_pair_bias", bias_t, z, gamma, beta, w, scratch, N, C, H, a_inner, a_so, a_si, scale, eps, dtype,
                          (hipStream_t)stream);
+}
+
+extern "C" int ffk_pair_bias_static(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w,
+                                    int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so, int64_t a_si,
+                                    float scale, float eps, int dtype, void* stream) {
+    FFK_REQUIRE(w && gamma && beta, FFK_ERR_NULL,
+                "ffk_pair_bias_static: w, gamma and beta are required (the shared scratch is rebuilt by every call)");
+    FFK_REQUIRE(C > 0 && C <= PB_STATIC_MAX_C && H > 0 && H <= PB_MAXH, FFK_ERR_SHAPE,
+                "ffk_pair_bias_static: C=%ld H=%ld exceed the static scratch (at most %d channels, %d heads)", (long)C, (long)H,
+                PB_STATIC_MAX_C, PB_MAXH);
+    float* scratch = nullptr;
+    int rc = pb_static_ptr(&scratch);
+    if (rc != FFK_OK) return rc;
+    return pair_bias_run("ffk_pair_bias_static", bias_t, z, gamma, beta, w, scratch, N, C, H, a_inner, a_so, a_si, scale, eps,
+                         dtype, (hipStream_t)stream);
 }

@@ -275,6 +275,17 @@ int ffk_pair_bias(void* bias_t, const void* z, const void* gamma, const void* be
                   float* scratch, int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so,
                   int64_t a_si, float scale, float eps, int dtype, void* stream);
 
+/* ffk_pair_bias for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments and results, without the scratch argument.  It has no
+ * counterpart in the reference.  The weight operand is built in a 8 256-byte array that the library holds in each
+ * GPU's memory for the life of the process (C <= 128 channels, H <= 8 heads; larger values are rejected with
+ * FFK_ERR_SHAPE).  The call allocates and frees nothing.  w, gamma and beta are required: every call rebuilds the
+ * operand, because all calls on one GPU share that GPU's array - calls that overlap on one GPU (different streams
+ * or host threads) race on it and must be serialised by the caller. */
+int ffk_pair_bias_static(void* bias_t, const void* z, const void* gamma, const void* beta, const void* w,
+                         int64_t N, int64_t C, int64_t H, int64_t a_inner, int64_t a_so, int64_t a_si,
+                         float scale, float eps, int dtype, void* stream);
+
 /* Fused core of the outer-product-mean (bf16, 32 projected channels, 128 pair channels):
  *     out[i, j, c] = resid[i, j, c] + ( sum_{d,e} (sum_s a[s,i,d] b[s,j,e]) * w[c, d, e] + bias[c] ) / (norm[i, j] + eps)
  * a_t, b_t : [r*32, spad] the masked projections, transposed (row i*32 + d, K = sequences, zero padded
