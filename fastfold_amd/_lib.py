@@ -135,6 +135,7 @@ class Tile(ctypes.Structure):
         ("gate_ld", c_int64), ("m_so", c_int64), ("m_si", c_int64),
         ("inner", c_int), ("kind", c_int), ("act", c_int), ("ncols", c_int), ("glu", c_int),
         ("scale", c_float), ("gate_rows", c_int), ("reserved", c_int),
+        ("xtail", c_void_p),
     ]
 
 
@@ -157,8 +158,9 @@ SIGNATURES["ffk_fused_linear"] = [ctypes.POINTER(LinearDesc), _P]
 
 def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, gate_ld=0, rowmask=None,
               m_so=0, m_si=0, s_o=0, s_i=0, s_h=32, s_d=1, inner=1, act=FFK_ACT_NONE, ncols=128, glu=0,
-              scale=1.0, gate_rows=0):
-    """Builds one epilogue descriptor; tensors may be passed directly (their data_ptr is taken)."""
+              scale=1.0, gate_rows=0, xtail=None):
+    """Builds one epilogue descriptor; tensors may be passed directly (their data_ptr is taken).  ``xtail`` is the
+    int8 tail tensor (or its address) of ``resid`` / ``out`` as an extended residual stream."""
     def p(t):
         return None if t is None else (t if isinstance(t, int) else t.data_ptr())
     t = Tile()
@@ -167,6 +169,7 @@ def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, g
     t.gate_ld, t.m_so, t.m_si = gate_ld, m_so, m_si
     t.inner, t.kind, t.act, t.ncols, t.glu, t.scale = inner, kind, act, ncols, glu, scale
     t.gate_rows = gate_rows
+    t.xtail = p(xtail)
     return t
 
 
@@ -218,7 +221,7 @@ class BgemmDesc(ctypes.Structure):
     """Mirror of ``ffk_bgemm_desc`` (include/ffk.h)."""
     _fields_ = [
         ("a", c_void_p), ("b", c_void_p), ("out", c_void_p), ("bias", c_void_p), ("resid", c_void_p),
-        ("rowdiv", c_void_p),
+        ("rowdiv", c_void_p), ("xtail", c_void_p),
         ("lda", c_int64), ("ldb", c_int64), ("a_bs", c_int64), ("b_bs", c_int64), ("o_bs", c_int64),
         ("s_o", c_int64), ("s_i", c_int64), ("s_h", c_int64), ("s_d", c_int64),
         ("inner", c_int), ("M", c_int), ("N", c_int), ("K", c_int), ("batch", c_int),
@@ -234,12 +237,14 @@ SIGNATURES["ffk_key_bias"] = [_P, _P, _P, _L, _L, _L, _L, _I, _P]
 
 def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, inner=None, s_o=0, s_i=None,
              s_h=32, s_d=1, bias=None, resid=None, rowdiv=None, div_eps=0.0, act=FFK_ACT_NONE, scale=1.0,
-             out_f32=False, dtype=None):
-    """Launches ``ffk_bgemm_nt``; default output addressing is row-major [M, N] (``s_i`` = N)."""
+             out_f32=False, dtype=None, xtail=None):
+    """Launches ``ffk_bgemm_nt``; default output addressing is row-major [M, N] (``s_i`` = N).  ``xtail``: int8 tail
+    of ``resid`` / ``out`` as an extended residual stream."""
     def p(t):
         return None if t is None else (t if isinstance(t, int) else t.data_ptr())
     d = BgemmDesc()
     d.a, d.b, d.out, d.bias, d.resid, d.rowdiv = p(a), p(b), p(out), p(bias), p(resid), p(rowdiv)
+    d.xtail = p(xtail)
     d.lda, d.ldb, d.a_bs, d.b_bs, d.o_bs = lda, ldb, a_bs, b_bs, o_bs
     d.inner = M if inner is None else inner
     d.s_o, d.s_i, d.s_h, d.s_d = s_o, (N if s_i is None else s_i), s_h, s_d
@@ -275,20 +280,20 @@ def pair_bias_static(bias_t, z, gamma, beta, w, *, N, C, H, a_inner, a_so, a_si,
          scale, eps, dtype_tag(z.dtype), stream_ptr())
 
 
-SIGNATURES["ffk_opm_fused"] = [_P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _P]
+SIGNATURES["ffk_opm_fused"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _F, _I, _P]
 
 
-def opm_fused(out, resid, a_t, b_t, w2p, bias, norm, *, r, spad, eps):
-    call("ffk_opm_fused", ptr(out), ptr(resid), ptr(a_t), ptr(b_t), ptr(w2p), ptr(bias), ptr(norm), r, spad, eps,
-         dtype_tag(a_t.dtype), stream_ptr())
+def opm_fused(out, resid, a_t, b_t, w2p, bias, norm, *, r, spad, eps, xtail=None):
+    call("ffk_opm_fused", ptr(out), ptr(resid), ptr(xtail), ptr(a_t), ptr(b_t), ptr(w2p), ptr(bias), ptr(norm), r, spad,
+         eps, dtype_tag(a_t.dtype), stream_ptr())
 
 
-SIGNATURES["ffk_transition_fused"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _P]
+SIGNATURES["ffk_transition_fused"] = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _F, _I, _P]
 
 
-def transition_fused(out, x, gamma, beta, w1, b1, w2, b2, *, M, C, hidden, eps=1e-5):
-    call("ffk_transition_fused", ptr(out), ptr(x), ptr(gamma), ptr(beta), ptr(w1), ptr(b1), ptr(w2), ptr(b2), M, C, hidden,
-         eps, dtype_tag(x.dtype), stream_ptr())
+def transition_fused(out, x, gamma, beta, w1, b1, w2, b2, *, M, C, hidden, eps=1e-5, xtail=None):
+    call("ffk_transition_fused", ptr(out), ptr(x), ptr(xtail), ptr(gamma), ptr(beta), ptr(w1), ptr(b1), ptr(w2), ptr(b2), M, C,
+         hidden, eps, dtype_tag(x.dtype), stream_ptr())
 
 
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):

@@ -6,6 +6,7 @@
 // computes C^T (rows of B are the M-operand) so that a lane holds 4 consecutive n of one
 // row m, and the tile is staged through LDS for 16-byte stores.
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -19,6 +20,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     constexpr int ES = sizeof(T);
     constexpr int OES = sizeof(OT);
     constexpr int OVEC = 16 / OES;
+    constexpr bool XS_OK = std::is_same<OT, bf16_t>::value;     // outputs that may carry a residual tail
     constexpr int BK = 128 / ES;                   // K elements per chunk (128 bytes per row)
     constexpr int P = 128 + 16;                    // ring row pitch (bytes)
     constexpr int SLOT = BT * P;
@@ -171,6 +173,9 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
     // ---- phase 2: staged tile -> global ----
     OT* out = (OT*)d.out + (long)bz * d.o_bs;
     const OT* resid = d.resid ? (const OT*)d.resid + (long)bz * d.o_bs : nullptr;
+    // extended residual stream (bf16 output with a residual, s_d == 1): the update is added at 24 bits
+    int8_t* xtail = nullptr;
+    if constexpr (XS_OK) xtail = d.xtail ? (int8_t*)d.xtail + (long)bz * d.o_bs : nullptr;
     if (d.s_d == 1) {
         constexpr int VPR = BT / OVEC;
         constexpr int N_IT = BT * VPR / THREADS;
@@ -183,6 +188,7 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
 #pragma unroll 1
             for (int i0 = 0; i0 < N_IT; i0 += 4) {
                 Vec16<OT> x[4], rv[4];
+                u32x2 tv[4];
                 long o[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -193,11 +199,28 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
                     o[j] = s_off[r] + (n >> 5) * d.s_h + (n & 31);
                     x[j] = *reinterpret_cast<const Vec16<OT>*>(sC + r * CP + c * OES);
                     if (resid) rv[j] = ld16(resid + o[j]);
+                    if (xtail) tv[j] = *reinterpret_cast<const u32x2*>(xtail + o[j]);
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int v = tid + THREADS * (i0 + j);
                     const int r = v / VPR, c = (v % VPR) * OVEC;
+                    if constexpr (XS_OK) {
+                        if (xtail) {
+                            float f[8];
+                            xs_decode8(*reinterpret_cast<const u32x4*>(&rv[j]), tv[j][0], tv[j][1], f);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) f[e] += (float)x[j].e[e];
+                            u32x4 hv;
+                            u32x2 tn;
+                            xs_encode8(f, hv, tn);
+                            if (m0 + r < M && n0 + c < N) {
+                                *reinterpret_cast<u32x4*>(out + o[j]) = hv;
+                                *reinterpret_cast<u32x2*>(xtail + o[j]) = tn;
+                            }
+                            continue;
+                        }
+                    }
                     if (resid) {
 #pragma unroll
                         for (int e = 0; e < OVEC; ++e)
@@ -213,6 +236,12 @@ __global__ __launch_bounds__(THREADS) void bgemm_nt_kernel(const ffk_bgemm_desc 
                 if (m >= M || n >= N) continue;
                 const long o = s_off[r] + (n >> 5) * d.s_h + (n & 31);
                 float y = DT<OT>::to_f(*reinterpret_cast<const OT*>(sC + r * CP + c * OES));
+                if constexpr (XS_OK) {
+                    if (xtail) {
+                        xs_round(y + xs_value(resid[o], xtail[o]), &out[o], &xtail[o]);
+                        continue;
+                    }
+                }
                 if (resid) y += DT<OT>::to_f(resid[o]);
                 out[o] = DT<OT>::from_f(y);
             }
@@ -252,6 +281,10 @@ int launch_bgemm(const ffk_bgemm_desc& d, hipStream_t st) {
 extern "C" int ffk_bgemm_nt(const ffk_bgemm_desc* d, void* stream) {
     FFK_REQUIRE(d, FFK_ERR_NULL, "ffk_bgemm_nt: null descriptor");
     FFK_REQUIRE(d->a && d->b && d->out, FFK_ERR_NULL, "ffk_bgemm_nt: null operand");
+    FFK_REQUIRE(!d->xtail || (d->dtype == FFK_BF16 && !d->out_f32 && d->resid && d->s_d == 1 && d->N % 16 == 0),
+                FFK_ERR_UNSUPPORTED, "ffk_bgemm_nt: a residual tail needs bf16 output, a residual, s_d == 1 and N %% 16 == 0");
+    FFK_REQUIRE(ffk_aligned16(d->xtail) && (!d->xtail || (d->o_bs % 16 == 0 && d->s_o % 8 == 0 && d->s_i % 8 == 0 && d->s_h % 8 == 0)),
+                FFK_ERR_ALIGN, "ffk_bgemm_nt: residual tail rows must be 16-byte aligned");
     const int es = d->dtype == FFK_F32 ? 4 : 2;
     const int vec = 16 / es;
     FFK_REQUIRE(d->M > 0 && d->N > 0 && d->K > 0 && d->batch > 0 && d->batch < 65536 && d->inner > 0, FFK_ERR_SHAPE,

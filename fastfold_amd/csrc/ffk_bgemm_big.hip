@@ -176,8 +176,9 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
     T* out = (T*)d.out + (long)bz * d.o_bs;
     const T* resid = d.resid ? (const T*)d.resid + (long)bz * d.o_bs : nullptr;
     const T* bias = (const T*)d.bias;
+    int8_t* xtail = d.xtail ? (int8_t*)d.xtail + (long)bz * d.o_bs : nullptr;   // extended residual stream (needs resid)
     const bool plain = !bias && !resid && d.act == FFK_ACT_NONE;
-    const bool bias_resid = bias && resid && d.act == FFK_ACT_NONE;
+    const bool bias_resid = bias && resid && d.act == FFK_ACT_NONE && !xtail;
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
         const long m = m0 + wm * 64 + mi * 32 + l32;
@@ -225,6 +226,7 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
                     rv[0] = *reinterpret_cast<const u32x4*>(resid + oc);
                     rv[1] = *reinterpret_cast<const u32x4*>(resid + oc + 8);
                 }
+                float upd[16];
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     float x = acc[ni][mi][v];
@@ -232,8 +234,20 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
                     if (d.act == FFK_ACT_RELU) x = relu_f(x);
                     else if (d.act == FFK_ACT_SIGMOID) x = sigmoid_f(x);
                     x *= mul;
+                    upd[v] = (float)(T)x;        // the update rounded to bf16, as every variant of this epilogue does
                     if (resid) x = (float)(T)x + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7];
                     y[v] = (T)x;
+                }
+                if (xtail) {       // the update is added to the 24-bit value instead (tails: 16 bytes at the element offset)
+                    const u32x4 tv = *reinterpret_cast<const u32x4*>(xtail + oc);
+                    u32x4 h0, h1, tn;
+                    xs_update16(upd, rv[0], rv[1], tv, h0, h1, tn);
+                    if (ok1) {     // all 16 columns or none (N % 16 == 0 is required with a tail)
+                        *reinterpret_cast<u32x4*>(out + o) = h0;
+                        *reinterpret_cast<u32x4*>(out + o + 8) = h1;
+                        *reinterpret_cast<u32x4*>(xtail + o) = tn;
+                    }
+                    continue;
                 }
             }
             if (ok0) *reinterpret_cast<u32x4*>(out + o) = *reinterpret_cast<const u32x4*>(&y[0]);
@@ -268,6 +282,7 @@ int bg_launch(const ffk_bgemm_desc& d, hipStream_t st) {
 int ffk_bgemm_big_try(const ffk_bgemm_desc* d, hipStream_t st, int* status) {
     if (d->dtype != FFK_BF16 || d->out_f32 || d->K % BG_BK != 0 || d->K < 3 * BG_BK || d->s_d != 1) return 0;
     if (d->M < 256 || d->N < 64 || d->N % 16 != 0) return 0;
+    if (d->xtail && (!d->resid || (reinterpret_cast<uintptr_t>(d->xtail) & 15) != 0)) return 0;
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al16(d->out) || (d->resid && !al16(d->resid)) || (d->bias && !al16(d->bias))) return 0;
     if (d->s_o % 8 || d->s_i % 8 || d->s_h % 8 || d->o_bs % 8) return 0;

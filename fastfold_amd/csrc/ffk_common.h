@@ -182,6 +182,71 @@ template <> __device__ __forceinline__ float exp_for<float>(float x) { return ex
 template <> __device__ __forceinline__ float exp_for<bf16_t>(float x) { return fast_exp2(1.4426950408889634f * x); }
 template <> __device__ __forceinline__ float exp_for<f16_t>(float x) { return fast_exp2(1.4426950408889634f * x); }
 
+// ------------------------------------------------- extended residual stream ----
+// A residual stream that is rounded to bf16 after every one of the ~300 updates of a 48-block stack drifts by
+// a random walk of half-ulp errors (about 2e-2 relative at the end).  The stream can therefore carry eight more
+// mantissa bits in a separate byte tensor ("tail", same element addressing as the bf16 tensor): the pair (h, t)
+// stands for the fp32 bit pattern (bits(h) << 16) + (t << 8), t a signed byte.  h is the value rounded to bf16
+// (half up, after rounding to 24 bits), so every reader that ignores the tail still sees a correctly rounded
+// bf16 tensor; only the kernels that add an update to the stream read and rewrite the tail.  Every such epilogue
+// rounds its update to bf16 first and then adds it at 24 bits, so that kernel variants (and chunked runs, which
+// may pick another variant for a ragged piece) agree bit for bit.
+__device__ __forceinline__ float xs_value(bf16_t h, int8_t t) {
+    const uint32_t hw = (uint32_t)__builtin_bit_cast(uint16_t, h) << 16;
+    return __builtin_bit_cast(float, hw + ((uint32_t)(int32_t)t << 8));
+}
+__device__ __forceinline__ void xs_round(float x, bf16_t* h, int8_t* t) {
+    const uint32_t w24 = __builtin_bit_cast(uint32_t, x) + 0x80u;
+    *h = __builtin_bit_cast(bf16_t, (uint16_t)((w24 + 0x8000u) >> 16));
+    *t = (int8_t)(uint8_t)(w24 >> 8);
+}
+// Eight consecutive elements: hv holds the bf16 values, (t0, t1) their tails.
+__device__ __forceinline__ void xs_decode8(const u32x4& hv, uint32_t t0, uint32_t t1, float* f) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t hw = (i & 1) ? (hv[i >> 1] & 0xFFFF0000u) : (hv[i >> 1] << 16);
+        const int32_t t = __builtin_amdgcn_sbfe((int32_t)(i < 4 ? t0 : t1), 8 * (i & 3), 8);
+        f[i] = __builtin_bit_cast(float, hw + ((uint32_t)t << 8));
+    }
+}
+__device__ __forceinline__ void xs_encode8(const float* f, u32x4& hv, uint32_t& t0, uint32_t& t1) {
+    uint32_t w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = __builtin_bit_cast(uint32_t, f[i]) + 0x80u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)      // high halves of (w + 0x8000) of two neighbours
+        hv[j] = __builtin_amdgcn_perm(w[2 * j + 1] + 0x8000u, w[2 * j] + 0x8000u, 0x07060302u);
+    // byte 1 of four neighbours
+    const uint32_t a = __builtin_amdgcn_perm(w[1], w[0], 0x0c0c0501u), b = __builtin_amdgcn_perm(w[3], w[2], 0x0c0c0501u);
+    const uint32_t c = __builtin_amdgcn_perm(w[5], w[4], 0x0c0c0501u), e = __builtin_amdgcn_perm(w[7], w[6], 0x0c0c0501u);
+    t0 = __builtin_amdgcn_perm(b, a, 0x05040100u);
+    t1 = __builtin_amdgcn_perm(e, c, 0x05040100u);
+}
+
+__device__ __forceinline__ void xs_encode8(const float* f, u32x4& hv, u32x2& tn) {
+    uint32_t a, b;
+    xs_encode8(f, hv, a, b);
+    tn[0] = a;
+    tn[1] = b;
+}
+// Sixteen consecutive elements of a lane: (r0, r1) the stream's bf16 values, tv their tail bytes; the update is
+// added to the 24-bit value and the result split again into (h0, h1) and tn.
+__device__ __forceinline__ void xs_update16(const float* upd, const u32x4& r0, const u32x4& r1, const u32x4& tv, u32x4& h0,
+                                            u32x4& h1, u32x4& tn) {
+    float f[16];
+    xs_decode8(r0, tv[0], tv[1], f);
+    xs_decode8(r1, tv[2], tv[3], f + 8);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) f[i] += upd[i];
+    uint32_t a, b, c, e;
+    xs_encode8(f, h0, a, b);
+    xs_encode8(f + 8, h1, c, e);
+    tn[0] = a;
+    tn[1] = b;
+    tn[2] = c;
+    tn[3] = e;
+}
+
 // ----------------------------------------------------------------- MFMA ----
 // A "fragment" is the 16 bytes one lane contributes to a 32x32 MFMA operand:
 // lane l supplies row (l & 31) of the operand and K-group (l >> 5).  For bf16 the

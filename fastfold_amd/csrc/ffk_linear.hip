@@ -11,6 +11,7 @@
 // (aliasing the weight ring) and written with 16-byte accesses in whichever direction the
 // destination layout is contiguous.
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -98,6 +99,7 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
     constexpr int CT = NT / (WN * 32);             // 32-channel MFMA tiles per wave
     constexpr int VEC = DT<T>::VEC;
     constexpr int ES = sizeof(T);
+    constexpr bool XS_OK = std::is_same<T, bf16_t>::value;     // outputs that may carry a residual tail
     constexpr int WP = BK * ES + 16;               // weight ring row pitch (bytes)
     constexpr int WBUF = NT * WP;                  // one ring slot
     constexpr int CP = NT * ES + 16;               // staged C pitch, [row][channel]
@@ -332,10 +334,13 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
             const bool qk = t.kind == FFK_TILE_QK;
             const T* gate = (const T*)t.gate;
             const T* resid = (const T*)t.resid;
+            int8_t* xtail = nullptr;                           // extended residual stream (bf16, with resid)
+            if constexpr (XS_OK) xtail = (int8_t*)t.xtail;
             const int c_last = ncols >= VEC ? ((ncols - VEC) / VEC) * VEC : 0;   // last full vector column
 #pragma unroll 1
             for (int i0 = 0; i0 < N_IT; i0 += 4) {
                 Vec16<T> x[4], gv[4], rv[4];
+                u32x2 tv[4];
                 long o[4];
                 // issue every load of the batch first (clamped, branch-free), then combine and store
 #pragma unroll
@@ -356,6 +361,7 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
                     mr = mr < M ? mr : M - 1;
                     if (gate) gv[j] = ld16(gate + (t.gate_rows > 0 ? mr % t.gate_rows : mr) * t.gate_ld + c);
                     if (resid) rv[j] = ld16(resid + o[j]);
+                    if (xtail) tv[j] = *reinterpret_cast<const u32x2*>(xtail + o[j]);
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -365,6 +371,22 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
 #pragma unroll
                         for (int e = 0; e < VEC; ++e)
                             x[j].e[e] = DT<T>::from_f(DT<T>::to_f(x[j].e[e]) * DT<T>::to_f(gv[j].e[e]));
+                    }
+                    if constexpr (XS_OK) {
+                        if (xtail) {
+                            float f[8];
+                            xs_decode8(*reinterpret_cast<const u32x4*>(&rv[j]), tv[j][0], tv[j][1], f);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) f[e] += (float)x[j].e[e];
+                            u32x4 hv;
+                            u32x2 tn;
+                            xs_encode8(f, hv, tn);
+                            if (m0 + r < M && c + VEC <= ncols) {
+                                *reinterpret_cast<u32x4*>(out + o[j]) = hv;
+                                *reinterpret_cast<u32x2*>(xtail + o[j]) = tn;
+                            }
+                            continue;
+                        }
                     }
                     if (resid) {
 #pragma unroll
@@ -389,6 +411,12 @@ __global__ __launch_bounds__(THREADS, 4) void fused_linear_kernel(const LinArgs 
                         oo = tab.off[r] + (long)(c >> 5) * t.s_h + (c & 31);
                     }
                     if (gate) y = DT<T>::to_f(DT<T>::from_f(y * DT<T>::to_f(gate[(t.gate_rows > 0 ? (m0 + r) % t.gate_rows : (m0 + r)) * t.gate_ld + c])));
+                    if constexpr (XS_OK) {
+                        if (xtail) {
+                            xs_round(y + xs_value(resid[oo], xtail[oo]), &out[oo], &xtail[oo]);
+                            continue;
+                        }
+                    }
                     if (resid) y += DT<T>::to_f(resid[oo]);
                     out[oo] = DT<T>::from_f(y);
                 }
@@ -499,6 +527,9 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
             FFK_REQUIRE(!t.gate || (ffk_aligned16(t.gate) && (t.gate_ld * es) % 16 == 0), FFK_ERR_ALIGN,
                         "ffk_fused_linear: tile %d: gate alignment", i);
         }
+        FFK_REQUIRE(!t.xtail || (d->dtype == FFK_BF16 && t.resid && t.kind == FFK_TILE_STRIDED && t.s_d == 1),
+                    FFK_ERR_UNSUPPORTED, "ffk_fused_linear: tile %d: a residual tail needs bf16, resid and a [row][channel] tile", i);
+        FFK_REQUIRE(ffk_aligned16(t.xtail), FFK_ERR_ALIGN, "ffk_fused_linear: tile %d: residual tail alignment", i);
     }
     // Two kernel variants.  Launches whose tiles are all stored channel-contiguous (plain, gated,
     // residual and q/k tiles) use the slab-persistent kernel (128-row slabs, register prefetch of the

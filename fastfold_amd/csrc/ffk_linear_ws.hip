@@ -62,6 +62,7 @@ struct WsSlot {
     T* out;
     const T* resid;
     const T* gate;
+    int8_t* xtail;           // tail bytes of resid / out as an extended residual stream, or nullptr
     long s_o, s_i, s_d, gate_ld;
     unsigned inner;
     unsigned gate_rows;      // 0, or the period of the gate's row index
@@ -112,7 +113,7 @@ __device__ __forceinline__ void unpack8(const T* p, float* f) {
 // STRIDED tiles: weight rows were loaded through tau, registers hold channels 16*half + v.
 // ACC / QK tiles: natural weight order, registers hold channels 8a + 4*half + b.
 // sb: this slot's 32 (GLU: 64) bias values in LDS (fp32); rmask: the row's mask value.
-template <bool GLU>
+template <bool GLU, bool XT>
 __device__ __forceinline__ void ws_store_rows_compact(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
                                               bool valid, unsigned mc, unsigned hi, unsigned lo, float rmask, int half) {
     const bool strided = t.kind == FFK_TILE_STRIDED;
@@ -181,6 +182,29 @@ __device__ __forceinline__ void ws_store_rows_compact(const WsSlot& t, const f32
                 const int cj = cl + 8 * j + 8 <= t.ncols_left ? 8 * j : (cl + 8 <= t.ncols_left ? 0 : -cl);
                 if (gate) gv[j] = *reinterpret_cast<const u32x4*>(gate + cj);
                 if (resid) rv[j] = *reinterpret_cast<const u32x4*>(resid + cj);
+            }
+            if (XT && t.xtail) {     // extended residual stream (whole 16-channel runs: ncols % 16 == 0 with a tail)
+                const u32x4 tv = *reinterpret_cast<const u32x4*>(t.xtail + (ok1 ? off : off - cl));
+                u32x4 tn;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {       // eight channels at a time (register budget)
+                    float f[8];
+                    xs_decode8(rv[j], tv[2 * j], tv[2 * j + 1], f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float u = (float)y[8 * j + e];
+                        if (gate) u = (float)(T)(u * (float)reinterpret_cast<const T*>(&gv[j])[e]);
+                        f[e] += u;
+                    }
+                    u32x4 hv;
+                    uint32_t ta, tb;
+                    xs_encode8(f, hv, ta, tb);
+                    tn[2 * j] = ta;
+                    tn[2 * j + 1] = tb;
+                    if (ok1) *reinterpret_cast<u32x4*>(out + off + 8 * j) = hv;
+                }
+                if (ok1) *reinterpret_cast<u32x4*>(t.xtail + off) = tn;
+                return;
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -269,7 +293,7 @@ __device__ __forceinline__ void ws_store_cols_compact(const WsSlot& t, const f32
 // STRIDED tiles: weight rows were loaded through tau, registers hold channels 16*half + v.
 // ACC / QK tiles: natural weight order, registers hold channels 8a + 4*half + b.
 // sb: this slot's 32 (GLU: 64) bias values in LDS (fp32); rmask: the row's mask value.
-template <bool GLU>
+template <bool GLU, bool XT>
 __device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
                                               bool valid, unsigned mc, unsigned hi, unsigned lo, float rmask, int half) {
     const bool strided = t.kind == FFK_TILE_STRIDED;
@@ -339,6 +363,29 @@ __device__ __forceinline__ void ws_store_rows(const WsSlot& t, const f32x16& acc
                 const int cj = cl + 8 * j + 8 <= t.ncols_left ? 8 * j : (cl + 8 <= t.ncols_left ? 0 : -cl);
                 if (gate) gv[j] = *reinterpret_cast<const u32x4*>(gate + cj);
                 if (resid) rv[j] = *reinterpret_cast<const u32x4*>(resid + cj);
+            }
+            if (XT && t.xtail) {     // extended residual stream (whole 16-channel runs: ncols % 16 == 0 with a tail)
+                const u32x4 tv = *reinterpret_cast<const u32x4*>(t.xtail + (ok1 ? off : off - cl));
+                u32x4 tn;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {       // eight channels at a time (register budget)
+                    float f[8];
+                    xs_decode8(rv[j], tv[2 * j], tv[2 * j + 1], f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float u = (float)y[8 * j + e];
+                        if (gate) u = (float)(T)(u * (float)reinterpret_cast<const T*>(&gv[j])[e]);
+                        f[e] += u;
+                    }
+                    u32x4 hv;
+                    uint32_t ta, tb;
+                    xs_encode8(f, hv, ta, tb);
+                    tn[2 * j] = ta;
+                    tn[2 * j + 1] = tb;
+                    if (ok1) *reinterpret_cast<u32x4*>(out + off + 8 * j) = hv;
+                }
+                if (ok1) *reinterpret_cast<u32x4*>(t.xtail + off) = tn;
+                return;
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -432,10 +479,51 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
 // products use, c2 sits in the bias table, c1 in a table of its own; the gate half does the same with the
 // second operand's row.  out = resid + value * sigmoid(gate), rounded once.  sb / sc1: this unit's 64 bias
 // values / 64 row sums in LDS (fp32), value half first.
+template <bool XT>
 __device__ __forceinline__ void ws_store_rows_folded(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
                                                      const float* sc1, float rstd, float nmr, float rstd_g, float nmr_g,
                                                      bool valid, unsigned hi, unsigned lo, int half) {
     // rstd_g / nmr_g (the second operand's statistics) arrive multiplied by -log2(e), as the gate's bias table is
+    const int cl = 16 * half;
+    const long off = (long)hi * t.s_o + (long)lo * t.s_i + cl;
+    u32x4 rv[2];
+    if (t.resid) {
+        rv[0] = *reinterpret_cast<const u32x4*>(t.resid + off);
+        rv[1] = *reinterpret_cast<const u32x4*>(t.resid + off + 8);
+    }
+    if (XT && t.xtail) {       // extended residual stream: the update is added at 24 bits, eight channels at a time
+        const u32x4 tv = *reinterpret_cast<const u32x4*>(t.xtail + off);
+        u32x4 tn;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            f32x4 bv[2], bg[2], cv[2], cg[2];      // the tables of these eight channels only (register budget)
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const int o = cl + 8 * j + 4 * a;
+                bv[a] = *reinterpret_cast<const f32x4*>(sb + o);
+                bg[a] = *reinterpret_cast<const f32x4*>(sb + 32 + o);
+                cv[a] = *reinterpret_cast<const f32x4*>(sc1 + o);
+                cg[a] = *reinterpret_cast<const f32x4*>(sc1 + 32 + o);
+            }
+            float f[8];
+            xs_decode8(rv[j], tv[2 * j], tv[2 * j + 1], f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int v = 8 * j + e;
+                const float val = __builtin_fmaf(acc[v], rstd, __builtin_fmaf(cv[e >> 2][e & 3], nmr, bv[e >> 2][e & 3]));
+                const float garg = __builtin_fmaf(accg[v], rstd_g, __builtin_fmaf(cg[e >> 2][e & 3], nmr_g, bg[e >> 2][e & 3]));
+                f[e] += (float)(T)(val * fast_rcp(1.0f + fast_exp2(garg)));
+            }
+            u32x4 hv;
+            uint32_t ta, tb;
+            xs_encode8(f, hv, ta, tb);
+            tn[2 * j] = ta;
+            tn[2 * j + 1] = tb;
+            if (valid) *reinterpret_cast<u32x4*>(t.out + off + 8 * j) = hv;
+        }
+        if (valid) *reinterpret_cast<u32x4*>(t.xtail + off) = tn;
+        return;
+    }
     f32x4 bv[4], bg[4], cv[4], cg[4];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
@@ -444,13 +532,6 @@ __device__ __forceinline__ void ws_store_rows_folded(const WsSlot& t, const f32x
         bg[a] = *reinterpret_cast<const f32x4*>(sb + 32 + o);
         cv[a] = *reinterpret_cast<const f32x4*>(sc1 + o);
         cg[a] = *reinterpret_cast<const f32x4*>(sc1 + 32 + o);
-    }
-    const int cl = 16 * half;
-    const long off = (long)hi * t.s_o + (long)lo * t.s_i + cl;
-    u32x4 rv[2];
-    if (t.resid) {
-        rv[0] = *reinterpret_cast<const u32x4*>(t.resid + off);
-        rv[1] = *reinterpret_cast<const u32x4*>(t.resid + off + 8);
     }
     T y[16];
     const T* rh = reinterpret_cast<const T*>(&rv[0]);
@@ -471,7 +552,8 @@ __device__ __forceinline__ void ws_store_rows_folded(const WsSlot& t, const f32x
 // DUAL: the gate halves of the GLU units multiply a second operand (row-major rows, own LayerNorm).  Its
 // slab goes from global memory straight into LDS (unpadded 256-byte rows, 16-byte columns XOR-swizzled
 // with the row index) one slab ahead and is normalised in place by the threads that requested it.
-template <int NS, int WS_K, bool CM, bool DUAL>
+// XT: the launch has tiles with a residual tail (extended residual stream); only those instantiations carry its code
+template <int NS, int WS_K, bool CM, bool DUAL, bool XT>
 __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs args) {
     typedef Mma<T> MM;
     typedef WsGeo<WS_K> G;
@@ -527,6 +609,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             sp[s].out = (T*)ts.out + coff;
             sp[s].resid = ts.resid ? (const T*)ts.resid + coff : nullptr;
             sp[s].gate = ts.gate ? (const T*)ts.gate + s_chan[s] : nullptr;
+            sp[s].xtail = XT && ts.xtail ? (int8_t*)ts.xtail + coff : nullptr;
             sp[s].s_o = ts.s_o;
             sp[s].s_i = ts.s_i;
             sp[s].s_d = ts.s_d;
@@ -803,7 +886,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                                 }
                             }
                             const float rmask = t.masked ? smk[n32] : 1.0f;
-                            ws_store_rows<G>(t, acc, G ? accg : acc, sb, valid, mc, c_hi, c_lo, rmask, half);
+                            ws_store_rows<G, XT>(t, acc, G ? accg : acc, sb, valid, mc, c_hi, c_lo, rmask, half);
                         } else {
                             const float* sm = t.masked ? smk : nullptr;
                             ws_store_cols<G>(t, acc, G ? accg : acc, sb, sm, m0g, M, l32, half);
@@ -904,10 +987,10 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                             su2 += lane_xor<32>(su2);
                             const float mean_g = su1 * (1.0f / WS_K);
                             const float rstd_g = -1.4426950408889634f * rsqrtf(fmaxf(su2 * (1.0f / WS_K) - mean_g * mean_g, 0.0f) + d.ln_eps);
-                            ws_store_rows_folded(t, acc, accg, sb, s_c1 + s_wrow[s], rstd, -rstd * mean, rstd_g, -rstd_g * mean_g,
+                            ws_store_rows_folded<XT>(t, acc, accg, sb, s_c1 + s_wrow[s], rstd, -rstd * mean, rstd_g, -rstd_g * mean_g,
                                                  valid, c_hi, c_lo, half);
-                        } else if (ALLOW_GLU && glu) ws_store_rows_compact<true>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
-                        else ws_store_rows_compact<false>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                        } else if (ALLOW_GLU && glu) ws_store_rows_compact<true, XT>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
+                        else ws_store_rows_compact<false, XT>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                     } else {
                         const float* sm = t.masked ? smk : nullptr;
                         if (ALLOW_GLU && glu) ws_store_cols_compact<true>(t, acc, accg, sb, sm, m0g, M, l32, half);
@@ -931,12 +1014,13 @@ bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
             if (t.ncols % 8 != 0 || t.s_o % 8 || t.s_i % 8 || t.s_h % 8) return false;
             if (t.resid && !al16(t.resid)) return false;
             if (t.gate && (!al16(t.gate) || t.gate_ld % 8)) return false;
+            if (t.xtail && (!t.resid || t.ncols % 16 != 0 || t.s_o % 16 || t.s_i % 16 || t.s_h % 16)) return false;
         } else {
-            if (t.ncols % 32 != 0 || t.resid || t.gate || t.s_o % 8 || t.s_h % 8) return false;
+            if (t.ncols % 32 != 0 || t.resid || t.gate || t.xtail || t.s_o % 8 || t.s_h % 8) return false;
         }
         return true;
     }
-    if (t.resid || t.gate) return false;
+    if (t.resid || t.gate || t.xtail) return false;
     if (t.kind == FFK_TILE_V) return t.inner % 32 == 0 && t.ncols % 32 == 0 && t.s_o % 8 == 0 && t.s_h % 8 == 0;
     if (t.kind != FFK_TILE_STRIDED) return false;
     return d.M % 16 == 0 && t.inner % 16 == 0 && t.s_i == 1 && t.s_o % 8 == 0 && t.s_h % 8 == 0 && t.s_d % 8 == 0;
@@ -1019,7 +1103,7 @@ bool ws_make_plan(const ffk_linear_desc& d, WsPlan& p, int rg_per_slab, int max_
     return true;
 }
 
-template <int NS, int K, bool CM, bool DUAL = false>
+template <int NS, int K, bool CM, bool DUAL = false, bool XT = false>
 int ws_launch(const WsArgs& args, hipStream_t st) {
     constexpr int WS_BM = WsGeo<K>::BM;
     const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float) +
@@ -1027,12 +1111,12 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
                         (CM ? 256 * sizeof(float) : 2 * K * sizeof(T));
     static FfkLdsReservation lds_reserved;
     {
-        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)linear_ws_kernel<NS, K, CM, DUAL>, smem, "ffk_fused_linear");
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)linear_ws_kernel<NS, K, CM, DUAL, XT>, smem, "ffk_fused_linear");
         if (rc_lds != FFK_OK) return rc_lds;
     }
     const int nslabs = ffk_cdiv(args.d.M, WS_BM);
     const int grid = nslabs < WS_MAX_GRID ? nslabs : WS_MAX_GRID;
-    linear_ws_kernel<NS, K, CM, DUAL><<<grid, WS_THREADS, smem, st>>>(args);
+    linear_ws_kernel<NS, K, CM, DUAL, XT><<<grid, WS_THREADS, smem, st>>>(args);
     return ffk_check_launch("ffk_fused_linear");
 }
 
@@ -1047,11 +1131,12 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->a2 && d->K != 128) return 0;                          // the second operand is built for K = 128
     const bool k256 = d->K == 256;
     if (d->variant == FFK_LINEAR_STAGED) return 0;
-    bool chan_major = false, v_tiles = false;
+    bool chan_major = false, v_tiles = false, tails = false;
     int mask_tile = -1;
     for (int i = 0; i < d->n_tiles; ++i) {
         const ffk_tile& t = d->tiles[i];
         if (!ws_tile_ok(*d, t)) return 0;
+        tails = tails || t.xtail != nullptr;
         chan_major = chan_major || (!ws_by_rows(t) && t.kind == FFK_TILE_STRIDED);
         v_tiles = v_tiles || t.kind == FFK_TILE_V;
         if (t.rowmask) {
@@ -1085,7 +1170,11 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
             // plain residual GLU tiles of 64 channels only
             if (t.kind != FFK_TILE_STRIDED || t.gate || t.rowmask || t.scale != 1.0f || t.ncols != 64) return 0;
         }
-        *status = ws_launch<2, 128, true, true>(args, st);
+        *status = tails ? ws_launch<2, 128, true, true, true>(args, st) : ws_launch<2, 128, true, true>(args, st);
+    } else if (tails) {
+        // residual tails: built for the output projections of the attentions (one plain tile group, two slots)
+        if (d->a_chanmajor || args.plan.max_slots > 2 || k64) return 0;
+        *status = k256 ? ws_launch<2, 256, false, false, true>(args, st) : ws_launch<2, 128, false, false, true>(args, st);
     } else if (d->a_chanmajor) {
         if (args.plan.max_slots > 2 || mask_tile >= 0) return 0;
         *status = k64 ? ws_launch<2, 64, true>(args, st) : ws_launch<2, 128, true>(args, st);

@@ -36,7 +36,7 @@ __device__ __forceinline__ void op_load_lds(const T* src, unsigned char* dst_wav
 }
 
 template <int KS1>   // MFMA K steps of the outer product: spad / 16 (4 or 8)
-__global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict__ out, const T* __restrict__ resid,
+__global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict__ out, const T* __restrict__ resid, int8_t* __restrict__ xtail,
                                                                  const T* __restrict__ at, const T* __restrict__ bt,
                                                                  const T* __restrict__ w2p, const T* __restrict__ bias,
                                                                  const float* __restrict__ norm, int r, float eps) {
@@ -174,6 +174,18 @@ __global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict_
             bv[1] = *reinterpret_cast<const u32x4*>(bias + ch + 8);
             rv[0] = *reinterpret_cast<const u32x4*>(resid + o);
             rv[1] = *reinterpret_cast<const u32x4*>(resid + o + 8);
+            if (xtail) {       // extended residual stream: the update is added at 24 bits
+                const u32x4 tv = *reinterpret_cast<const u32x4*>(xtail + o);
+                float upd[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) upd[v] = (float)(T)((acc2[m][c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7]) * inv);
+                u32x4 h0, h1, tn;
+                xs_update16(upd, rv[0], rv[1], tv, h0, h1, tn);
+                *reinterpret_cast<u32x4*>(out + o) = h0;
+                *reinterpret_cast<u32x4*>(out + o + 8) = h1;
+                *reinterpret_cast<u32x4*>(xtail + o) = tn;
+                continue;
+            }
             T y[16];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict_
 }
 
 template <int KS1>
-int opm_launch(T* out, const T* resid, const T* at, const T* bt, const T* w2p, const T* bias, const float* norm, int r,
+int opm_launch(T* out, const T* resid, int8_t* xtail, const T* at, const T* bt, const T* w2p, const T* bias, const float* norm, int r,
                float eps, hipStream_t st) {
     const size_t smem = 2 * (size_t)OP_A2 + 3 * OP_W2SLOT + 2 * (size_t)(OP_TJ * OP_EC * KS1 * 32);
     static FfkLdsReservation lds_reserved;
@@ -196,23 +208,23 @@ int opm_launch(T* out, const T* resid, const T* at, const T* bt, const T* w2p, c
         if (rc_lds != FFK_OK) return rc_lds;
     }
     const unsigned grid = (unsigned)((r / OP_TI) * (r / OP_TJ));
-    opm_fused_kernel<KS1><<<grid, OP_THREADS, smem, st>>>(out, resid, at, bt, w2p, bias, norm, r, eps);
+    opm_fused_kernel<KS1><<<grid, OP_THREADS, smem, st>>>(out, resid, xtail, at, bt, w2p, bias, norm, r, eps);
     return ffk_check_launch("ffk_opm_fused");
 }
 
 }  // namespace
 
-extern "C" int ffk_opm_fused(void* out, const void* resid, const void* a_t, const void* b_t, const void* w2p, const void* bias,
+extern "C" int ffk_opm_fused(void* out, const void* resid, void* xtail, const void* a_t, const void* b_t, const void* w2p, const void* bias,
                              const float* norm, int64_t r, int64_t spad, float eps, int dtype, void* stream) {
     FFK_REQUIRE(out && resid && a_t && b_t && w2p && bias && norm, FFK_ERR_NULL, "ffk_opm_fused: null pointer");
     FFK_REQUIRE(dtype == FFK_BF16, FFK_ERR_DTYPE, "ffk_opm_fused: bf16 only (dtype tag %d)", dtype);
     FFK_REQUIRE(r > 0 && r % 32 == 0 && r <= 32768, FFK_ERR_SHAPE, "ffk_opm_fused: r=%ld must be a positive multiple of 32", (long)r);
     FFK_REQUIRE(spad == 64 || spad == 128, FFK_ERR_UNSUPPORTED, "ffk_opm_fused: padded sequence count %ld must be 64 or 128", (long)spad);
     FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(resid) && ffk_aligned16(a_t) && ffk_aligned16(b_t) && ffk_aligned16(w2p) &&
-                    ffk_aligned16(bias),
+                    ffk_aligned16(bias) && ffk_aligned16(xtail),
                 FFK_ERR_ALIGN, "ffk_opm_fused: buffers must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     if (spad == 128)
-        return opm_launch<8>((T*)out, (const T*)resid, (const T*)a_t, (const T*)b_t, (const T*)w2p, (const T*)bias, norm, (int)r, eps, st);
-    return opm_launch<4>((T*)out, (const T*)resid, (const T*)a_t, (const T*)b_t, (const T*)w2p, (const T*)bias, norm, (int)r, eps, st);
+        return opm_launch<8>((T*)out, (const T*)resid, (int8_t*)xtail, (const T*)a_t, (const T*)b_t, (const T*)w2p, (const T*)bias, norm, (int)r, eps, st);
+    return opm_launch<4>((T*)out, (const T*)resid, (int8_t*)xtail, (const T*)a_t, (const T*)b_t, (const T*)w2p, (const T*)bias, norm, (int)r, eps, st);
 }

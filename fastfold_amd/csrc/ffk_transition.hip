@@ -39,7 +39,7 @@ __device__ __forceinline__ void tr_load_lds(const T* src, unsigned char* dst_wav
                                      (__attribute__((address_space(3))) void*)dst_wave, 16, 0, 0);
 }
 
-__global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x,
+__global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
                                                                         const T* __restrict__ gamma, const T* __restrict__ beta,
                                                                         const T* __restrict__ w1, const T* __restrict__ b1,
                                                                         const T* __restrict__ w2, const T* __restrict__ b2,
@@ -181,6 +181,20 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
         bv[1] = *reinterpret_cast<const u32x4*>(b2 + ch + 8);
         rv[0] = *reinterpret_cast<const u32x4*>(x + o);
         rv[1] = *reinterpret_cast<const u32x4*>(x + o + 8);
+        if (xtail) {           // extended residual stream: the update is added at 24 bits
+            const u32x4 tv = *reinterpret_cast<const u32x4*>(xtail + o);
+            float upd[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) upd[v] = (float)(T)(acc2[c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7]);
+            u32x4 h0, h1, tn;
+            xs_update16(upd, rv[0], rv[1], tv, h0, h1, tn);
+            if (ok) {
+                *reinterpret_cast<u32x4*>(out + o) = h0;
+                *reinterpret_cast<u32x4*>(out + o + 8) = h1;
+                *reinterpret_cast<u32x4*>(xtail + o) = tn;
+            }
+            continue;
+        }
         T y[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -196,7 +210,7 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
 
 }  // namespace
 
-extern "C" int ffk_transition_fused(void* out, const void* x, const void* gamma, const void* beta, const void* w1,
+extern "C" int ffk_transition_fused(void* out, const void* x, void* xtail, const void* gamma, const void* beta, const void* w1,
                                     const void* b1, const void* w2, const void* b2, int64_t M, int64_t C, int64_t hidden,
                                     float eps, int dtype, void* stream) {
     FFK_REQUIRE(out && x && gamma && beta && w1 && b1 && w2 && b2, FFK_ERR_NULL, "ffk_transition_fused: null pointer");
@@ -205,7 +219,7 @@ extern "C" int ffk_transition_fused(void* out, const void* x, const void* gamma,
                 (long)C, (long)hidden);
     FFK_REQUIRE(M > 0 && M < (1L << 31) * (long)TR_BM, FFK_ERR_SHAPE, "ffk_transition_fused: bad row count %ld", (long)M);
     FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(x) && ffk_aligned16(gamma) && ffk_aligned16(beta) && ffk_aligned16(w1) &&
-                    ffk_aligned16(w2) && ffk_aligned16(b2),
+                    ffk_aligned16(w2) && ffk_aligned16(b2) && ffk_aligned16(xtail),
                 FFK_ERR_ALIGN, "ffk_transition_fused: buffers must be 16-byte aligned");
     const size_t smem = 2 * (size_t)TR_W1SLOT + 2 * TR_W2SLOT + TR_H * sizeof(float);
     static FfkLdsReservation lds_reserved;
@@ -214,7 +228,7 @@ extern "C" int ffk_transition_fused(void* out, const void* x, const void* gamma,
         if (rc_lds != FFK_OK) return rc_lds;
     }
     const unsigned grid = (unsigned)ffk_cdiv(M, TR_BM);
-    transition_fused_kernel<<<grid, TR_THREADS, smem, (hipStream_t)stream>>>((T*)out, (const T*)x, (const T*)gamma, (const T*)beta,
+    transition_fused_kernel<<<grid, TR_THREADS, smem, (hipStream_t)stream>>>((T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta,
                                                                             (const T*)w1, (const T*)b1, (const T*)w2,
                                                                             (const T*)b2, (long)M, eps);
     return ffk_check_launch("ffk_transition_fused");

@@ -148,14 +148,20 @@ def linear(x2, w_pk, b_pk, N, *, act=FFK_ACT_NONE, out=None, resid=None, ln=None
 
 
 # --------------------------------------------------------------------- transition ----
-def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
-    """out = x + W2 relu(W1 LN(x) + b1) + b2 over rows of x [M, C]; out may alias x."""
+def xtail_ptr(xtail, off=0):
+    """Address of element ``off`` of an int8 residual tail (None stays None)."""
+    return None if xtail is None else xtail.data_ptr() + off
+
+
+def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget, xtail=None):
+    """out = x + W2 relu(W1 LN(x) + b1) + b2 over rows of x [M, C]; out may alias x.  ``xtail`` (here and in the
+    other sub-modules): int8 tensor of x's shape holding the tail bytes of x / out as an extended residual stream."""
     M, C = x.shape
     dt, dev = x.dtype, x.device
     es = es_of(dt)
     if dt == torch.bfloat16 and C == 128 and hidden == 512 and ln is not None:
         # both layers in one kernel, hidden activation kept on chip
-        _lib.transition_fused(out, x, ln[0], ln[1], w1_pk, b1_pk, w2, b2, M=M, C=C, hidden=hidden)
+        _lib.transition_fused(out, x, ln[0], ln[1], w1_pk, b1_pk, w2, b2, M=M, C=C, hidden=hidden, xtail=xtail)
         return out
     rows = max(128, min(M, (budget // (hidden * es)) // 128 * 128))
     hid = torch.empty(min(rows, M), hidden, dtype=dt, device=dev)
@@ -169,22 +175,27 @@ def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget):
                      for t in range(t0, min(nt, t0 + per))]
             _lib.fused_linear(x, w1_pk, tiles, M=n, K=C, ln=ln, a_off=r0 * C, w_row_off=t0 * 128)
         _lib.bgemm_nt(hid, w2, out.data_ptr() + r0 * C * es, M=n, N=C, K=hidden, lda=hidden, ldb=hidden, bias=b2,
-                      resid=x.data_ptr() + r0 * C * es, dtype=dt)
+                      resid=x.data_ptr() + r0 * C * es, dtype=dt, xtail=xtail_ptr(xtail, r0 * C))
     return out
 
 
 # ---------------------------------------------------------------------- attention ----
 def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_pk, out_bias_pk, c_out,
-              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None, head_dim=32):
+              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None, head_dim=32, budget=None, o_map=None, xtail=None):
     """Gated multi-head attention over N tokens for each of B2 batch rows.  The kernels work on 32-wide
     heads; a narrower head (``head_dim`` < 32) arrives zero-padded to 32 channels in ``w_pk`` / ``wo_pk``,
     which changes neither the scores nor the used output channels - only the score scale is its own.
 
-    x holds the C-channel rows addressed by ``a_map = (inner, s_o, s_i)``; w_pk is the packed
-    [q; k; v; gate(; bias)] weight.  The attention update is projected by wo_pk and written as
-    ``out = resid + update + out_bias`` with the same row addressing (``resid=None``: no residual).
-    With ``bias_in_launch`` the last N-tile of w_pk produces the [H, N, N] additive bias into
-    ``bias_t`` from the same normalised rows.
+    x holds the C-channel rows addressed by ``a_map = (inner, s_o, s_i)`` with ``inner`` either B2 * N (plain
+    row-major) or N (one batch row per outer step); w_pk is the packed [q; k; v; gate(; bias)] weight.  The
+    attention update is projected by wo_pk and written as ``out = resid + update + out_bias`` with the same row
+    addressing, or with ``o_map`` if the output rows have another width (``resid=None``: no residual).  With ``bias_in_launch`` the last N-tile of w_pk produces the
+    [H, N, N] additive bias into ``bias_t`` from the same normalised rows.
+
+    ``budget`` (bytes) bounds the operand buffers (q, k, v, gate and the head outputs: 5 * H * ceil(N / 32) KB
+    elements per batch row): the batch rows are then processed in slabs - projection, core, output projection per
+    slab.  Batch rows are independent and a slab's outputs overwrite only the rows it read, so this also holds
+    when ``out`` aliases ``x``; the additive bias, which reads all of x, is computed before the first slab.
     """
     dt, dev = x.dtype, x.device
     es = es_of(dt)
@@ -194,68 +205,80 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     M = B2 * N
     NT = (N + 31) // 32
     zero = (N % 32) != 0
-    q_t = alloc((B2, H, NT, 1024), dt, dev, zero)
-    k_t = alloc((B2, H, NT, 1024), dt, dev, zero)
-    v_t = alloc((B2, H, NT, 1024), dt, dev, zero)
+    a_inner, a_so, a_si = a_map
+    o_inner, o_so, o_si = a_map if o_map is None else o_map
+    if a_inner not in (M, N) or o_inner != a_inner:
+        raise RuntimeError("attention: row maps with inner=%d / %d fit neither B2 * N nor N" % (a_inner, o_inner))
+    per_row = 5 * H * NT * 1024 * es
+    slab = B2 if budget is None else min(B2, max(2, (budget // per_row) // 2 * 2))
+    q_t = alloc((slab, H, NT, 1024), dt, dev, zero)
+    k_t = alloc((slab, H, NT, 1024), dt, dev, zero)
+    v_t = alloc((slab, H, NT, 1024), dt, dev, zero)
     # With bf16, 128 input channels and whole key tiles the projection runs on the weights-stationary
     # kernel, which writes q, k and the gate in accumulator order straight from its registers.
     acc_order = dt == torch.bfloat16 and C in (64, 128, 256) and N % 32 == 0
     qk_kind = FFK_TILE_ACC if acc_order else FFK_TILE_QK
-    gate = torch.empty((B2, H, NT, 1024) if acc_order else (M, HC), dtype=dt, device=dev)
+    gate = torch.empty((slab, H, NT, 1024) if acc_order else (slab * N, HC), dtype=dt, device=dev)
+    o = torch.empty(slab * N, HC, dtype=dt, device=dev)
     tpg = HC // 128
     qscale = LOG2E / math.sqrt(float(head_dim))
     tkw = dict(inner=N, s_o=H * NT * 1024, s_h=NT * 1024)
-    tiles = []
-    for buf, kind, scale in ((q_t, qk_kind, qscale), (k_t, qk_kind, 1.0), (v_t, FFK_TILE_V, 1.0)):
-        for t in range(tpg):
-            tiles.append(make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, scale=scale, **tkw))
-    for t in range(tpg):
-        if acc_order:
-            tiles.append(make_tile(gate.data_ptr() + t * 4 * NT * 1024 * es, kind=FFK_TILE_ACC,
-                                   bias=gate_bias_pk.data_ptr() + t * 128 * es, act=FFK_ACT_SIGMOID, **tkw))
-        else:
-            tiles.append(make_tile(gate.data_ptr() + t * 128 * es, bias=gate_bias_pk.data_ptr() + t * 128 * es,
-                                   inner=M, s_i=HC, act=FFK_ACT_SIGMOID))
-    a_inner, a_so, a_si = a_map
     bias_tile = None
     if bias_in_launch:
         bias_tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H,
                               scale=LOG2E)
-    if bias_tile is not None and not acc_order:
-        tiles.append(bias_tile)
-        bias_tile = None
     # The skinny bias projection has its own pass over x.  It goes first: x was written by the launch before
     # this call and is still (partly) cache-resident, and the bias pass writes little, so the projection after
     # it finds x as warm as before - the other way round the projection's output (four times the size of x)
     # has pushed x out by the time the bias pass reads it (measured: -0.65 % block time at N = 1024).
-    if bias_tile is not None and C in (64, 128):
+    if bias_tile is not None and acc_order and C in (64, 128):
         _pair_bias_launch(bias_t, x, ln, w_pk[4 * tpg * 128:], pb_scratch, N=N, C=C, H=H, a_inner=a_inner,
                           a_so=a_so, a_si=a_si, scale=LOG2E)
         bias_tile = None
-    # the weights-stationary kernel holds at most 16 (K = 256) or 24 (K = 128) 32-channel units per launch
-    per = 4 if (acc_order and C == 256) else len(tiles)
-    for t0 in range(0, len(tiles), per):
-        _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
-                          w_row_off=t0 * 128)
-    if bias_tile is not None:
+    if bias_tile is not None and (acc_order or slab < B2):     # its own launch over all rows, before x changes
         _lib.fused_linear(x, w_pk, [bias_tile], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
                           w_row_off=4 * tpg * 128)
+        bias_tile = None
     def key_bias():
         kb = torch.empty(B2, NT * 32, dtype=torch.float32, device=dev)
         flags = torch.empty(B2, NT, dtype=torch.int32, device=dev)
         _lib.key_bias(kb, flags, mask, B=B2, N=N, mask_sb=mask_sb, mask_sn=mask_sn)
         return kb, flags
     kb, flags = _mask_derived(mask, ("key_bias", B2, N, mask_sb, mask_sn), key_bias) if mask is not None else key_bias()
-    o = torch.empty(M, HC, dtype=dt, device=dev)
-    _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb, flags, gate, B2=B2, H=H, Nq=N, Nk=N, gate_tiled=acc_order)
-    del q_t, k_t, v_t, gate
-    tiles = []
-    for t in range((c_out + 127) // 128):
-        tiles.append(make_tile(out.data_ptr() + t * 128 * es,
-                               bias=None if out_bias_pk is None else out_bias_pk.data_ptr() + t * 128 * es,
-                               resid=None if resid is None else resid.data_ptr() + t * 128 * es,
-                               inner=a_inner, s_o=a_so, s_i=a_si, ncols=min(128, c_out - t * 128)))
-    _lib.fused_linear(o, wo_pk, tiles, M=M, K=HC)
+    for b0 in range(0, B2, slab):
+        nb = min(slab, B2 - b0)
+        Ms = nb * N
+        # rows b0 * N ... of the map: a shifted base, and an inner extent that still covers the slab
+        off, inner = (b0 * N * a_si, Ms) if a_inner == M else (b0 * a_so, N)
+        o_off = b0 * N * o_si if a_inner == M else b0 * o_so
+        tiles = []
+        for buf, kind, scale in ((q_t, qk_kind, qscale), (k_t, qk_kind, 1.0), (v_t, FFK_TILE_V, 1.0)):
+            for t in range(tpg):
+                tiles.append(make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, scale=scale, **tkw))
+        for t in range(tpg):
+            if acc_order:
+                tiles.append(make_tile(gate.data_ptr() + t * 4 * NT * 1024 * es, kind=FFK_TILE_ACC,
+                                       bias=gate_bias_pk.data_ptr() + t * 128 * es, act=FFK_ACT_SIGMOID, **tkw))
+            else:
+                tiles.append(make_tile(gate.data_ptr() + t * 128 * es, bias=gate_bias_pk.data_ptr() + t * 128 * es,
+                                       inner=Ms, s_i=HC, act=FFK_ACT_SIGMOID))
+        if bias_tile is not None:      # single slab: the bias rides on the projection launch
+            tiles.append(bias_tile)
+        # the weights-stationary kernel holds at most 16 (K = 256) or 24 (K = 128) 32-channel units per launch
+        per = 4 if (acc_order and C == 256) else len(tiles)
+        for t0 in range(0, len(tiles), per):
+            _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=Ms, K=C, a_inner=inner, a_so=a_so, a_si=a_si, ln=ln,
+                              w_row_off=t0 * 128, a_off=off)
+        _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb[b0:b0 + nb], flags[b0:b0 + nb], gate, B2=nb, H=H, Nq=N, Nk=N,
+                           gate_tiled=acc_order)
+        tiles = []
+        for t in range((c_out + 127) // 128):
+            tiles.append(make_tile(out.data_ptr() + (o_off + t * 128) * es,
+                                   bias=None if out_bias_pk is None else out_bias_pk.data_ptr() + t * 128 * es,
+                                   resid=None if resid is None else resid.data_ptr() + (o_off + t * 128) * es,
+                                   xtail=xtail_ptr(xtail, o_off + t * 128),
+                                   inner=inner, s_o=o_so, s_i=o_si, ncols=min(128, c_out - t * 128)))
+        _lib.fused_linear(o, wo_pk, tiles, M=Ms, K=HC)
     return out
 
 
@@ -322,7 +345,7 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
 
 
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,
-                            dual_pk=None):
+                            dual_pk=None, xtail=None):
     """out = z + sigmoid(Wg LN(z) + bg) * (Wout LN2(p) + b_out),  p[i,j,:] = sum_k a[i,k,:] b[j,k,:]
     (outgoing) or sum_k a[k,i,:] b[k,j,:] (incoming), a/b the masked gated projections.
     ``dual_pk`` = (weights, biases) of pack_trimul_out: the gate is then computed in the output stage."""
@@ -357,7 +380,8 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     if dual:
         wd, bd, rowsums = dual_pk
         tiles = [make_tile(out.data_ptr() + t * 64 * es, bias=bd.data_ptr() + t * 128 * es, glu=1, ncols=64,
-                           resid=z.data_ptr() + t * 64 * es, inner=M, s_i=C) for t in range(C // 64)]
+                           resid=z.data_ptr() + t * 64 * es, xtail=xtail_ptr(xtail, t * 64), inner=M, s_i=C)
+                 for t in range(C // 64)]
         # both LayerNorms (of p and of z) are folded into the packed weights: no normalisation pass over either
         _lib.fused_linear(p, wd, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
                           ln_rowsums=rowsums, a2=z, a2_inner=M, a2_si=C)
@@ -366,14 +390,15 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     for t in range((C + 127) // 128):
         tiles.append(make_tile(out.data_ptr() + t * 128 * es, bias=out_bias_pk.data_ptr() + t * 128 * es,
                                gate=g.data_ptr() + t * 128 * es, gate_ld=C, resid=z.data_ptr() + t * 128 * es,
-                               inner=M, s_i=C, ncols=min(128, C - t * 128)))
+                               xtail=xtail_ptr(xtail, t * 128), inner=M, s_i=C, ncols=min(128, C - t * 128)))
     _lib.fused_linear(p, wout_pk, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
                       ln=ln2)
     return out
 
 
 # ------------------------------------------------------------------ outer product mean ----
-def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, bo, budget, eps=1e-3, wo_ed=None):
+def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, bo, budget, eps=1e-3, wo_ed=None,
+                       xtail=None):
     """out = z + (Wo vec(sum_s a[s,i,:] (x) b[s,j,:]) + bo) / (sum_s mask[s,i] mask[s,j] + eps),
     a, b the masked 32-channel projections of LN(m).  m is [s, r, C] rows, mask [s, r]."""
     dt, dev = m.dtype, m.device
@@ -393,7 +418,7 @@ def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, 
     nrm = _mask_derived(mask, ("opm_norm", s, r, spad), normaliser)
     if wo_ed is not None and dt == torch.bfloat16 and Cz == 128 and r % 32 == 0 and spad in (64, 128):
         # fused core: the [r, r, 1024] outer product never leaves the chip
-        _lib.opm_fused(out, z, ab[0], ab[1], wo_ed, bo, nrm, r=r, spad=spad, eps=eps)
+        _lib.opm_fused(out, z, ab[0], ab[1], wo_ed, bo, nrm, r=r, spad=spad, eps=eps, xtail=xtail)
         return out
     ci = max(1, min(r, budget // (r * 1024 * es)))
     O = torch.empty(ci * r, 1024, dtype=dt, device=dev)
@@ -402,7 +427,8 @@ def outer_product_mean(m, mask, z, out, *, s, r, C, Cz, ln, wab_pk, bab_pk, wo, 
         _lib.bgemm_nt(ab.data_ptr() + i0 * 32 * spad * es, ab[1], O, M=32 * n, N=32 * r, K=spad, lda=spad, ldb=spad,
                       inner=32, s_o=r * 1024, s_i=32, s_h=1024, s_d=1, dtype=dt)
         _lib.bgemm_nt(O, wo, out.data_ptr() + i0 * r * Cz * es, M=n * r, N=Cz, K=1024, lda=1024, ldb=1024, bias=bo,
-                      rowdiv=nrm.data_ptr() + i0 * r * 4, div_eps=eps, resid=z.data_ptr() + i0 * r * Cz * es, dtype=dt)
+                      rowdiv=nrm.data_ptr() + i0 * r * 4, div_eps=eps, resid=z.data_ptr() + i0 * r * Cz * es, dtype=dt,
+                      xtail=xtail_ptr(xtail, i0 * r * Cz))
     return out
 
 

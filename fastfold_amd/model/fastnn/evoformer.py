@@ -33,25 +33,29 @@ class Evoformer(nn.Module):
         self.is_multimer = is_multimer
 
     # -- un-padded core on [1, s, r, c_m] / [1, r, r, c_z] / [1, s, r] / [1, r, r] ----------
-    def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
+    def _core(self, m, z, msa_mask, pair_mask, inplace: bool, tails=(None, None)):
+        """``tails = (m_tail, z_tail)``: int8 tails of m / z as extended residual streams (the stack's bf16 mode),
+        or None for the plain stream of the reference."""
         F_.check_nonempty("Evoformer", m, z)
+        mt, zt = tails
         if self.is_multimer:
             # multimer order (evoformer.py:70-76, 133-137): outer product mean first, the MSA stack reads the
             # pair tensor it leaves, the pair stack runs last
             z_new = z if inplace else torch.empty_like(z)
-            self.communication._run(m, msa_mask, z, z_new)
-            m = self.msa.inplace(m, z_new, msa_mask) if inplace else self.msa.forward(m, z_new, msa_mask)
-            self.pair.inplace([z_new], pair_mask)
+            self.communication._run(m, msa_mask, z, z_new, zt)
+            m = self.msa.inplace(m, z_new, msa_mask, mt) if inplace else self.msa.forward(m, z_new, msa_mask, mt)
+            self.pair.inplace([z_new], pair_mask, zt)
             return m, z_new
         if inplace:
-            m = self.msa.inplace(m, z, msa_mask)
-            self.communication._run(m, msa_mask, z, z)
-            self.pair.inplace([z], pair_mask)
+            m = self.msa.inplace(m, z, msa_mask, mt)
+            self.communication._run(m, msa_mask, z, z, zt)
+            self.pair.inplace([z], pair_mask, zt)
             return m, z
-        m = self.msa.forward(m, z, msa_mask)
-        z = self.communication.forward(m, msa_mask, z)
-        self.pair.inplace([z], pair_mask)     # z is already a fresh tensor
-        return m, z
+        m = self.msa.forward(m, z, msa_mask, mt)
+        z_new = torch.empty_like(z)
+        self.communication._run(m, msa_mask, z, z_new, zt)
+        self.pair.inplace([z_new], pair_mask, zt)
+        return m, z_new
 
     def _enter(self, m, z, r):
         if self.first_block:
@@ -95,6 +99,11 @@ class Evoformer(nn.Module):
 class EvoformerStack(nn.Module):
     """Main Evoformer trunk (Algorithm 6): ``no_blocks`` blocks, then ``s = Linear(c_m, c_s)(m[0])``."""
 
+    # bf16 / fp16 runs keep eight extra mantissa bits of both residual streams in int8 side tensors between the
+    # blocks (see "extended residual stream" in include/ffk.h): rounding m and z to bf16 after each of the ~430
+    # sub-updates of 48 blocks alone costs 2e-2 .. 3e-2 relative L2 at the output.  False = the reference's plain stream.
+    extended_residual = True
+
     def __init__(self, c_m: int, c_z: int, c_s: int, no_blocks: int, blocks_per_ckpt: int,
                  clear_cache_between_blocks: bool = False, is_multimer: bool = False, **kwargs):
         super(EvoformerStack, self).__init__()
@@ -109,11 +118,17 @@ class EvoformerStack(nn.Module):
     def _run(self, m, z, msa_mask, pair_mask, inplace_first: bool):
         mm, zz = m.unsqueeze(0), z.unsqueeze(0)
         mk, pk = msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)
+        tails = (None, None)
+        if self.extended_residual and mm.dtype == torch.bfloat16 and mm.is_cuda:
+            # zero tails: the inputs are exact bf16 values; the tails die with this call, the bf16 tensors they
+            # leave are the correctly rounded results
+            tails = (torch.zeros(mm.shape, dtype=torch.int8, device=mm.device),
+                     torch.zeros(zz.shape, dtype=torch.int8, device=zz.device))
         with F_.mask_cache():          # key biases / normalisers depend on the masks only: once per stack, not per block
             for i, b in enumerate(self.blocks):
                 if self.clear_cache_between_blocks:
                     torch.cuda.empty_cache()
-                mm, zz = b._core(mm.contiguous(), zz.contiguous(), mk, pk, inplace=(inplace_first or i > 0))
+                mm, zz = b._core(mm.contiguous(), zz.contiguous(), mk, pk, inplace=(inplace_first or i > 0), tails=tails)
         return mm.squeeze(0), zz.squeeze(0)
 
     def forward(self, m: torch.Tensor, z: torch.Tensor, msa_mask: torch.Tensor, pair_mask: torch.Tensor,

@@ -3,9 +3,10 @@ parameter names and call signatures (fastfold/model/fastnn/ops.py), each forward
 short sequence of HIP kernel launches (see ``_fused.py``) instead of PyTorch ops.
 
 Differences that do not change results: there is no distributed code (DAP size 1: the
-reference's gather/scatter calls are identities) and chunking (``set_chunk_size``) only
-lowers the scratch-memory budget of the launches, since attention logits and transition /
-outer-product intermediates are already streamed.
+reference's gather/scatter calls are identities) and chunking (``set_chunk_size``) lowers
+the scratch-memory budget of the launches: attention logits and the fused transition / outer-product
+intermediates are never materialised, and what is (attention operand tiles, the hidden activations and
+outer products of the unfused paths) is produced a bounded slab of rows at a time.
 """
 import math
 import os
@@ -58,6 +59,17 @@ def _no_grad_guard(module, *tensors):
         raise NotImplementedError(
             "%s: the HIP path implements the forward pass only; run it under torch.no_grad()"
             % type(module).__name__)
+
+
+def _check_tail(xtail, x):
+    """The int8 tail of ``x`` as an extended residual stream (see include/ffk.h): same shape, bf16 stream only."""
+    if xtail is None:
+        return None
+    if x.dtype != torch.bfloat16 or xtail.dtype != torch.int8 or xtail.shape != x.shape or not xtail.is_contiguous() \
+            or xtail.device != x.device:
+        raise RuntimeError("residual tail must be a contiguous int8 tensor of the bf16 stream's shape %s on its device"
+                           % (tuple(x.shape),))
+    return xtail
 
 
 def _ln_pair(ln, dtype):
@@ -148,7 +160,7 @@ class Transition(nn.Module, _PackMixin):
         self.linear1 = Linear(d, n * d, initializer='relu')
         self.linear2 = Linear(n * d, d, initializer='zeros')
 
-    def _run(self, src, out):
+    def _run(self, src, out, xtail=None):
         F_.check_cuda(src)
         _no_grad_guard(self, src)
         dt, dev = src.dtype, src.device
@@ -162,7 +174,7 @@ class Transition(nn.Module, _PackMixin):
             self.linear2.weight.detach().to(dt).contiguous(), self.linear2.bias.detach().to(dt).contiguous()))
         x = src.view(-1, d)
         F_.transition(x, out.view(-1, d), ln=_ln_pair(self.norm, dt), w1_pk=w1, b1_pk=b1, w2=w2, b2=b2,
-                      hidden=hidden, budget=_budget())
+                      hidden=hidden, budget=_budget(), xtail=_check_tail(xtail, src))
         return out
 
     def forward(self, src):
@@ -190,7 +202,7 @@ class OutProductMean(nn.Module, _PackMixin):
         self.o_linear = Linear(n_feat_proj * n_feat_proj, n_feat_out, initializer='zero', use_bias=True)
         self.n_feat_proj = n_feat_proj
 
-    def _run(self, M, M_mask, Z_raw, out):
+    def _run(self, M, M_mask, Z_raw, out, xtail=None):
         F_.check_cuda(M, M_mask, Z_raw)
         _no_grad_guard(self, M, Z_raw)
         if self.n_feat_proj != 32:
@@ -214,7 +226,7 @@ class OutProductMean(nn.Module, _PackMixin):
             self.o_linear.weight.detach().to(dt).view(-1, 32, 32).transpose(1, 2).reshape(-1, 1024).contiguous()))
         F_.outer_product_mean(M.contiguous(), _mask_like(M_mask, M), Z_raw, out, s=s, r=r, C=C, Cz=Cz,
                               ln=_ln_pair(self.layernormM, dt), wab_pk=wab, bab_pk=bab, wo=wo, bo=bo, wo_ed=wo_ed,
-                              budget=_budget())
+                              budget=_budget(), xtail=_check_tail(xtail, Z_raw))
         return out
 
     def forward(self, M, M_mask, Z_raw):
@@ -311,7 +323,7 @@ class SelfAttention(nn.Module, _PackMixin):
         out = torch.empty(1, B2, N, self.out_dim, dtype=dt, device=dev)
         F_.attention(x, out, None, B2=B2, N=N, C=C, H=self.n_head, a_map=(B2 * N, 0, C), ln=None, w_pk=w_pk,
                      gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob, c_out=self.out_dim, mask=mk, mask_sb=sb,
-                     mask_sn=sn, bias_t=bias_t, head_dim=self.c)
+                     mask_sn=sn, bias_t=bias_t, head_dim=self.c, budget=_budget(), o_map=(B2 * N, 0, self.out_dim))
         return out
 
 
@@ -424,7 +436,7 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         self.output_bias = nn.parameter.Parameter(data=torch.zeros((d_pair,)), requires_grad=True)
         self.p_drop = p_drop
 
-    def _run(self, Z_raw, Z_mask, out):
+    def _run(self, Z_raw, Z_mask, out, xtail=None):
         F_.check_cuda(Z_raw, Z_mask)
         _no_grad_guard(self, Z_raw)
         dt, dev = Z_raw.dtype, Z_raw.device
@@ -454,7 +466,7 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         F_.triangle_multiplication(Z_raw, out, r=r, C=C, c=self.c, incoming=self._incoming,
                                    ln1=_ln_pair(self.layernorm1, dt), w_pk=w, b_pk=b, n_glu=n_glu,
                                    ln2=_ln_pair(self.layernorm2, dt), wout_pk=wout, out_bias_pk=bout,
-                                   mask=_mask_like(Z_mask, Z_raw), dual_pk=dual)
+                                   mask=_mask_like(Z_mask, Z_raw), dual_pk=dual, xtail=_check_tail(xtail, Z_raw))
         return out
 
     def forward(self, Z_raw, Z_mask):
@@ -492,7 +504,7 @@ class _TriangleAttention(nn.Module, _PackMixin):
                                        last_bias_fuse=True)
         self.out_bias = nn.parameter.Parameter(data=torch.zeros((d_pair,)), requires_grad=True)
 
-    def _run(self, Z_raw, Z_mask, out):
+    def _run(self, Z_raw, Z_mask, out, xtail=None):
         F_.check_cuda(Z_raw, Z_mask)
         _no_grad_guard(self, Z_raw)
         dt, dev = Z_raw.dtype, Z_raw.device
@@ -515,7 +527,7 @@ class _TriangleAttention(nn.Module, _PackMixin):
         F_.attention(Z_raw, out, Z_raw, B2=r, N=r, C=C, H=self.n_head, a_map=a_map,
                      ln=_ln_pair(self.layernorm1, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
                      c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=bias_t, bias_in_launch=True, pb_scratch=pbs,
-                     head_dim=self.c)
+                     head_dim=self.c, budget=_budget(), xtail=_check_tail(xtail, Z_raw))
         return out
 
     def forward(self, Z_raw, Z_mask):

@@ -22,22 +22,23 @@ class PairCore(nn.Module):
                                                                             c=self.hidden_c, n_head=self.n_head)
         self.PairTransition = ChunkTransition(d=d_pair)
 
-    def forward(self, pair, pair_mask):
-        """pair [1, r, r, d_pair], pair_mask [1, r, r] -> new pair (input untouched)."""
+    def forward(self, pair, pair_mask, xtail=None):
+        """pair [1, r, r, d_pair], pair_mask [1, r, r] -> new pair (input untouched).  ``xtail``: int8 tail of the
+        pair tensor as an extended residual stream (read with the input, rewritten for the output)."""
         pair = pair.contiguous()
         out = torch.empty_like(pair)
-        self.TriangleMultiplicationOutgoing._run(pair, pair_mask, out)
-        self._rest(out, pair_mask)
+        self.TriangleMultiplicationOutgoing._run(pair, pair_mask, out, xtail)
+        self._rest(out, pair_mask, xtail)
         return out
 
-    def _rest(self, z, pair_mask):
-        self.TriangleMultiplicationIncoming._run(z, pair_mask, z)
-        self.TriangleAttentionStartingNode._run(z, pair_mask, z)
-        self.TriangleAttentionEndingNode._run(z, pair_mask, z)
-        self.PairTransition._run(z, z)
+    def _rest(self, z, pair_mask, xtail=None):
+        self.TriangleMultiplicationIncoming._run(z, pair_mask, z, xtail)
+        self.TriangleAttentionStartingNode._run(z, pair_mask, z, xtail)
+        self.TriangleAttentionEndingNode._run(z, pair_mask, z, xtail)
+        self.PairTransition._run(z, z, xtail)
 
-    def inplace(self, pair, pair_mask):
+    def inplace(self, pair, pair_mask, xtail=None):
         pair[0] = pair[0].contiguous()
-        self.TriangleMultiplicationOutgoing._run(pair[0], pair_mask, pair[0])
-        self._rest(pair[0], pair_mask)
+        self.TriangleMultiplicationOutgoing._run(pair[0], pair_mask, pair[0], xtail)
+        self._rest(pair[0], pair_mask, xtail)
         return pair

@@ -219,6 +219,13 @@ def synth_inputs(seed, n_seq, n_res, c_m=256, c_z=128, mask_tail_frac=0.0):
     return m, z, msa_mask, pair_mask
 
 
+def bf16_round(x):
+    """fp32 array rounded to the nearest bf16 value (round-to-nearest-even on the upper 16 bits), still fp32."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(x))
+
+
 def synth_template_inputs(seed, n_templ, n_res, c_t=64, mask_tail_frac=0.0):
     """t [n_templ, r, r, c_t] ~ N(0,1) fp32 and the pair mask [r, r] shared by the templates."""
     t = synth_inputs(seed, n_templ, n_res * n_res, c_m=c_t, c_z=1)[0].reshape(n_templ, n_res, n_res, c_t)

@@ -103,6 +103,16 @@ int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const 
 
 
 /* ------------------------------------------------------------------------------------
+ * Extended residual stream.  A 48-block bf16 stack adds about 300 updates to each of its two activation tensors;
+ * rounding the sum to bf16 after every one of them is a random walk of half-ulp errors that ends near 2e-2 relative,
+ * above the tolerance of the bf16 mode.  Every entry point that adds an update to such a tensor (`resid`) therefore
+ * accepts an optional tail tensor of signed bytes with the same shape: the pair (h, t) of a bf16 element and its tail
+ * byte stands for the fp32 bit pattern (bits(h) << 16) + (t << 8), i.e. eight more mantissa bits, h being that value
+ * rounded to bf16 - a reader that ignores the tail sees an ordinary, correctly rounded bf16 tensor.  The tail is
+ * read and rewritten in place (a zero-filled tail is an exact bf16 tensor; dropping the tails at the end leaves the
+ * correctly rounded result), bf16 only.  No counterpart in the reference, which keeps the plain bf16 stream. */
+
+/* ------------------------------------------------------------------------------------
  * Fused linear:  out = epilogue( prologue(A)[M,K] . W[N,K]^T )      (bf16 / fp32 MFMA)
  *
  * A tile of rows of A (all K columns, K in {32..256}, K % 32 == 0) is loaded into LDS once,
@@ -159,6 +169,10 @@ typedef struct ffk_tile {
     float scale;
     int32_t gate_rows;     /* 0, or the period of the gate's row index (see gate) */
     int32_t reserved;
+    void* xtail;           /* NULL, or the tail bytes of an extended residual stream (see above): int8, addressed with
+                              the element offsets of out; requires resid (bf16, STRIDED with s_d == 1).  The epilogue then
+                              adds its update to the 24-bit value (resid, xtail), writes the rounded bf16 value to out and
+                              the new tail back to xtail */
 } ffk_tile;
 
 typedef struct ffk_linear_desc {
@@ -223,6 +237,7 @@ typedef struct ffk_bgemm_desc {
     const void* bias;      /* [N] operand dtype, or NULL */
     const void* resid;     /* or NULL */
     const float* rowdiv;   /* fp32 [M] (per batch: + b * M), or NULL */
+    void* xtail;           /* NULL, or the tail bytes of resid / out as an extended residual stream (bf16, s_d == 1) */
     int64_t lda, ldb, a_bs, b_bs, o_bs;
     int64_t s_o, s_i, s_h, s_d;
     int32_t inner;
@@ -290,20 +305,22 @@ int ffk_pair_bias_static(void* bias_t, const void* z, const void* gamma, const v
  *     out[i, j, c] = resid[i, j, c] + ( sum_{d,e} (sum_s a[s,i,d] b[s,j,e]) * w[c, d, e] + bias[c] ) / (norm[i, j] + eps)
  * a_t, b_t : [r*32, spad] the masked projections, transposed (row i*32 + d, K = sequences, zero padded
  *            to spad = 64 or 128); w2p : [128, 1024] with column e*32 + d (the reference weight has d*32 + e);
- * norm : fp32 [r, r]; resid / out : [r*r, 128] (may alias); r % 32 == 0.
+ * norm : fp32 [r, r]; resid / out : [r*r, 128] (may alias); xtail : NULL or the [r*r, 128] tail bytes of
+ * resid / out as an extended residual stream; r % 32 == 0.
  * The [r, r, 1024] outer product is never written to memory.
  * Replaces: the einsum / o_linear / division chain of OutProductMean.forward
  * (fastfold/model/fastnn/ops.py:156-171; nn/outer_product_mean.py:93-127). */
-int ffk_opm_fused(void* out, const void* resid, const void* a_t, const void* b_t, const void* w2p,
+int ffk_opm_fused(void* out, const void* resid, void* xtail, const void* a_t, const void* b_t, const void* w2p,
                   const void* bias, const float* norm, int64_t r, int64_t spad, float eps, int dtype,
                   void* stream);
 
 /* Fused pair transition (bf16, C = 128, hidden = 512):
  *     out = x + W2 . relu( W1 . LayerNorm(x; gamma, beta, eps) + b1 ) + b2
- * x, out : [M, C] row-major (may alias); w1 : [hidden, C]; w2 : [C, hidden]; b1 : [hidden]; b2 : [C].
+ * x, out : [M, C] row-major (may alias); xtail : NULL or the [M, C] tail bytes of x / out as an extended residual
+ * stream (the LayerNorm reads x alone); w1 : [hidden, C]; w2 : [C, hidden]; b1 : [hidden]; b2 : [C].
  * The hidden activation never leaves the chip.
  * Replaces: Transition.forward / ChunkTransition.forward (fastfold/model/fastnn/ops.py:79-82,104-123). */
-int ffk_transition_fused(void* out, const void* x, const void* gamma, const void* beta, const void* w1,
+int ffk_transition_fused(void* out, const void* x, void* xtail, const void* gamma, const void* beta, const void* w1,
                          const void* b1, const void* w2, const void* b2, int64_t M, int64_t C,
                          int64_t hidden, float eps, int dtype, void* stream);
 

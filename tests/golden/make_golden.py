@@ -7,6 +7,7 @@ and inputs.  Run only in the build container, where /root/reference is mounted:
     python tests/golden/make_golden.py extra      # extra-MSA stack
     python tests/golden/make_golden.py template   # template pair stack
     python tests/golden/make_golden.py pointwise  # template point-wise attention
+    python tests/golden/make_golden.py cfg4       # one Evoformer block at N_seq=128, N_res=1024 (sampled outputs)
 
 The fixture pins what closed forms cannot: the composition of a block (order of the
 sub-updates, residual placement, OPM reading the updated MSA), the q/k/v and left/right
@@ -151,8 +152,59 @@ def main_pointwise():
     print("wrote", os.path.join(HERE, "template_pointwise_nn_golden.npz"))
 
 
+CFG4_CASES = [
+    # name, seed, fan_in_scaled
+    ("cfg4_fanin", 71, True),
+    ("cfg4_std002", 72, False),
+]
+
+
+def cfg4_sample_indices(seed, n_seq, n_valid):
+    """Index sets of the stored sample: 16 sequences, 48 row residues, 48 column residues, all un-masked, drawn
+    without replacement (random positions inside the kernels' 32- and 256-wide tiles, unlike a strided sample)."""
+    rng = np.random.RandomState(seed + 5)
+    return (np.sort(rng.choice(n_seq, 16, replace=False)), np.sort(rng.choice(n_valid, 48, replace=False)),
+            np.sort(rng.choice(n_valid, 48, replace=False)))
+
+
+def main_cfg4():
+    """The benchmark's headline shape: one block, N_seq = 128, N_res = 1024, last 5 % of the residues masked, inputs
+    rounded to bf16 (what the bf16 HIP path receives).  The reference runs in fp32 with its own chunking
+    (chunk_size = 64) to bound memory; only a sample of the outputs is stored."""
+    from fastfold.model.nn.evoformer import EvoformerStack  # the reference
+    from fastfold_amd.synthetic import bf16_round
+
+    s, r, tail = 128, 1024, 0.05
+    nv = r - int(round(tail * r))
+    out = {}
+    for name, seed, fis in CFG4_CASES:
+        stack = EvoformerStack(c_m=256, c_z=128, c_hidden_msa_att=32, c_hidden_opm=32, c_hidden_mul=128,
+                               c_hidden_pair_att=32, c_s=384, no_heads_msa=8, no_heads_pair=4, no_blocks=1,
+                               transition_n=4, msa_dropout=0.15, pair_dropout=0.25, blocks_per_ckpt=1,
+                               inf=1e9, eps=1e-8).eval()
+        sd = synth_nn_state(seed=seed, no_blocks=1, fan_in_scaled=fis)
+        stack.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+        m, z, msa_mask, pair_mask = synth_inputs(seed, s, r, mask_tail_frac=tail)
+        m, z = bf16_round(m), bf16_round(z)
+        with torch.no_grad():
+            mo, zo, so = stack(torch.from_numpy(m), torch.from_numpy(z), torch.from_numpy(msa_mask),
+                               torch.from_numpy(pair_mask), chunk_size=64, _mask_trans=False)
+        S, I, J = cfg4_sample_indices(seed, s, nv)
+        out[name + ".S"], out[name + ".I"], out[name + ".J"] = S, I, J
+        out[name + ".m"] = mo.numpy()[S][:, J]
+        out[name + ".z"] = zo.numpy()[I][:, J]
+        out[name + ".s"] = so.numpy()[J]
+        out[name + ".cfg"] = np.array([seed, 1, s, r, int(round(tail * 100)), int(fis)], dtype=np.int64)
+        print(name, "m", float(np.abs(mo.numpy() - m)[:, :nv].mean()), "z", float(np.abs(zo.numpy() - z)[:nv, :nv].mean()),
+              flush=True)
+    np.savez_compressed(os.path.join(HERE, "evoformer_cfg4_nn_golden.npz"), **out)
+    print("wrote", os.path.join(HERE, "evoformer_cfg4_nn_golden.npz"))
+
+
 if __name__ == "__main__":
-    if "pointwise" in sys.argv[1:]:
+    if "cfg4" in sys.argv[1:]:
+        main_cfg4()
+    elif "pointwise" in sys.argv[1:]:
         main_pointwise()
     elif "template" in sys.argv[1:]:
         main_template()
