@@ -213,8 +213,20 @@ def long_sequence(dev):
             "tflops": round(block_gflop(s, r) / ms, 1), "peak_device_GB": round(torch.cuda.max_memory_allocated() / 1e9, 1)}
 
 
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(threads):
-    """The CPU oracle timed on the host cores: one fp32 block at N_seq=128, N_res=256."""
+    """The CPU oracle (plain-PyTorch fp32 restatement of the reference's nn Evoformer block, ``_mask_trans=False``)
+    timed on the host cores: benchmark configuration 1 (one block, N_seq = 32, N_res = 64; 3 warm-up + 10 timed
+    passes, median) and, as a second point, one block at N_seq = 128, N_res = 256 (1 + 5 passes)."""
     import numpy as np
     import torch
     from fastfold_amd.synthetic import synth_inputs, synth_nn_state
@@ -222,19 +234,29 @@ def cpu_baseline(threads):
     torch.set_num_threads(threads)
     st = OracleStack(no_blocks=1).eval()
     st.load_state_dict({k: torch.from_numpy(v) for k, v in synth_nn_state(seed=0, no_blocks=1).items()})
-    m, z, mm, pm = (torch.from_numpy(t) for t in synth_inputs(0, 128, 256))
-    ts = []
-    with torch.no_grad():
-        st(m, z, mm, pm, _mask_trans=False)
-        t_end = time.time() + 20.0
-        while len(ts) < 5 and (time.time() < t_end or len(ts) < 2):
-            t0 = time.time()
-            st(m, z, mm, pm, _mask_trans=False)
-            ts.append((time.time() - t0) * 1e3)
-    return {"value": round(float(np.median(ts)), 2), "unit": "ms/block", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": "1 Evoformer block, fp32, N_seq=128 N_res=256 (configs[2] shape), oracle/evoformer_ref.py, "
-                      "median of %d runs after 1 warm-up" % len(ts)}
+
+    def timed(s, r, warm, n, budget_s):
+        m, z, mm, pm = (torch.from_numpy(t) for t in synth_inputs(0, s, r))
+        ts = []
+        with torch.no_grad():
+            for _ in range(warm):
+                st(m, z, mm, pm, _mask_trans=False)
+            t_end = time.time() + budget_s
+            while len(ts) < n and (time.time() < t_end or len(ts) < 2):
+                t0 = time.time()
+                st(m, z, mm, pm, _mask_trans=False)
+                ts.append((time.time() - t0) * 1e3)
+        return ts
+
+    t1 = timed(32, 64, 3, 10, 10.0)
+    t3 = timed(128, 256, 1, 5, 20.0)
+    return {"value": round(float(np.median(t1)), 2), "unit": "ms/block", "cores": torch.get_num_threads(),
+            "kind": "port", "min": round(float(np.min(t1)), 2), "os_cpu_count": os.cpu_count(), "cpu_model": _cpu_model(),
+            "sample": "configs[0]: 1 Evoformer block, fp32, N_seq=32 N_res=64 (10.9 GFLOP), oracle/evoformer_ref.py, "
+                      "median of %d runs after 3 warm-ups; threads = the box's CPU share (OMP_NUM_THREADS), not "
+                      "os.cpu_count()" % len(t1),
+            "second_sample": {"workload": "1 block, fp32, N_seq=128 N_res=256 (configs[2] shape, 216.1 GFLOP)",
+                              "value": round(float(np.median(t3)), 2), "unit": "ms/block", "runs": len(t3)}}
 
 
 def main():
@@ -248,8 +270,10 @@ def main():
     ap.add_argument("--no-micro", action="store_true")
     ap.add_argument("--only-feeders", action="store_true",
                     help="time only the extra-MSA and template pair stacks (for profiling them on their own)")
-    ap.add_argument("--long-sequence", action="store_true",
-                    help="also time one block at N_res = 4096 (a few seconds and 26 GB of device memory more)")
+    ap.add_argument("--no-long-sequence", action="store_true",
+                    help="skip the block at N_res = 4096 (a few seconds and about 30 GB of device memory)")
+    ap.add_argument("--plain-residual", action="store_true",
+                    help="A/B switch: the reference's plain bf16 residual stream instead of the extended one")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the Evoformer on ONE GPU (DAP size 1, no collectives); "
@@ -267,6 +291,8 @@ def main():
         print(json.dumps({"feeders": feeder_stacks(dev, r)}))
         return
     stack = build_stack(args.blocks, dev, torch.bfloat16)
+    if args.plain_residual:
+        stack.extended_residual = False
     m, z, mm, pm = (torch.from_numpy(t).to(dev, torch.bfloat16) for t in synth_inputs(0, s, r, mask_tail_frac=wl["tail"]))
 
     def step():
@@ -312,7 +338,8 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": wl["name"], "blocks": args.blocks, "n_seq": s, "n_res": r,
                    "block_gflop": round(block_gflop(s, r), 1),
-                   "stack_tflops": round(block_gflop(s, r) * args.blocks / ms_per_step, 1)},
+                   "stack_tflops": round(block_gflop(s, r) * args.blocks / ms_per_step, 1),
+                   "residual_stream": "bf16" if args.plain_residual else "bf16 + int8 tail (24-bit)"},
         "roofline": roofline,
     }
     if args.workload == "cfg4" and not args.no_micro:
@@ -331,7 +358,7 @@ def main():
         del m3, z3, mm3, pm3
     del stack, out
     torch.cuda.empty_cache()
-    if args.long_sequence:
+    if not args.no_long_sequence and args.workload == "cfg4":
         line["long_sequence"] = long_sequence(dev)
         torch.cuda.empty_cache()
     if not args.no_micro:
