@@ -21,6 +21,11 @@ from .ops import Linear, OutProductMean
 from .triangle import PairCore
 
 
+def _private_copy(view, owner):
+    out = view.contiguous()
+    return out.clone() if out.data_ptr() == owner.data_ptr() else out
+
+
 class Evoformer(nn.Module):
 
     def __init__(self, c_m: int, c_z: int, first_block: bool, last_block: bool, is_multimer: bool = False):
@@ -63,7 +68,9 @@ class Evoformer(nn.Module):
         if m.dim() != 4 or z.dim() != 4 or m.shape[2] != r + 1 or z.shape[1] != r + 1:
             raise RuntimeError("Evoformer: a non-first block expects padded [1, s, r+1, c] / [1, r+1, r+1, c] "
                                "inputs, got %s / %s" % (tuple(m.shape), tuple(z.shape)))
-        return m[:, :, :r, :].contiguous(), z[:, :r, :r, :].contiguous()
+        # the core runs in place on these: they must be copies even where the un-padding slice is already
+        # contiguous (a single sequence, a single residue) and ``.contiguous()`` would hand back the caller's memory
+        return _private_copy(m[:, :, :r, :], m), _private_copy(z[:, :r, :r, :], z)
 
     def _leave(self, m, z):
         if self.last_block:

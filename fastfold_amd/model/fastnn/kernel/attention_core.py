@@ -6,7 +6,10 @@
 for q, k, v ``[b1, b2, h, n, d]``, mask ``[b1, b2, n]`` (0/1, over keys) and bias ``[b1, h, n, n]``.
 The logits are never materialised: the operands are re-tiled into the 32x32 MFMA order and handed to
 the flash attention kernel (``ffk_attention_fwd``).  Forward only, like the reference.  The kernel is
-specialised for the Evoformer's head dim (32); other head dims raise ``RuntimeError``.
+specialised for the Evoformer's head dim (32); narrower heads (8 and 16, the extra-MSA and template stacks)
+are zero-padded to 32 channels, which changes neither the scores nor the used output channels; the
+reference's Triton kernel also takes 64 and 128 (triton/attention_core.py:143), which no module of the
+path uses and which raise ``RuntimeError`` here.
 """
 import math
 
@@ -22,8 +25,18 @@ def _attention_core(q, k, v, mask=None, bias=None):
         raise RuntimeError("fused_attention_core: q, k, v must be [b1, b2, h, n, d] of one shape, got %s %s %s"
                            % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
     b1, b2, h, n, d = q.shape
-    if d != 32:
-        raise RuntimeError("fused_attention_core: head dim %d is not supported (the kernel is built for 32)" % d)
+    if d not in (8, 16, 32):
+        raise RuntimeError("fused_attention_core: head dim %d is not supported: the kernel is built for 32 and takes "
+                           "8 and 16 zero-padded; 64 and 128 (accepted by the reference's Triton kernel) are not built" % d)
+    if d != 32:      # zero channels add nothing to q.k and give zero output channels, which are dropped below
+        pad = torch.nn.functional.pad
+        out = _attention_core_d32(pad(q, (0, 32 - d)), pad(k, (0, 32 - d)), pad(v, (0, 32 - d)), mask, bias, d)
+        return out.view(b1, b2, n, h, 32)[..., :d].reshape(b1, b2, n, h * d)
+    return _attention_core_d32(q, k, v, mask, bias, d)
+
+
+def _attention_core_d32(q, k, v, mask, bias, d_scale):
+    b1, b2, h, n, d = q.shape
     if mask is not None and tuple(mask.shape) != (b1, b2, n):
         raise RuntimeError("fused_attention_core: mask must be [b1, b2, n], got %s" % (tuple(mask.shape),))
     if bias is not None and tuple(bias.shape) != (b1, h, n, n):
@@ -32,7 +45,7 @@ def _attention_core(q, k, v, mask=None, bias=None):
     if out.numel() == 0:
         return out
     nt = layouts.n_tiles(n)
-    scale = _lib.LOG2E / math.sqrt(d)            # the kernel exponentiates in base 2
+    scale = _lib.LOG2E / math.sqrt(d_scale)      # the kernel exponentiates in base 2; the scale is the true head dim's
     kb = torch.empty(b2, nt * 32, dtype=torch.float32, device=q.device)
     fl = torch.empty(b2, nt, dtype=torch.int32, device=q.device)
     for i in range(b1):

@@ -42,8 +42,16 @@ def _dm_strides(dm, like):
     return dm, tuple(st)
 
 
+def _forward_only(name, *tensors):
+    """The three ops launch forward kernels only; the reference's TorchScript versions are differentiable.  Rather
+    than return outputs without a grad_fn (gradients would silently vanish), refuse inputs that require grad."""
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise NotImplementedError("%s: the HIP path implements the forward pass only; run it under torch.no_grad()" % name)
+
+
 def bias_sigmod_ele(y, bias, z):
     """sigmoid(y + bias) * z   (fused_ops.py:5-7)."""
+    _forward_only("bias_sigmod_ele", y, bias, z)
     y_, z_, b_ = y.contiguous(), z.contiguous(), bias.contiguous().to(y.dtype)
     _lib.check_device(y_, z_, b_)
     C = y_.shape[-1]
@@ -57,6 +65,7 @@ def bias_sigmod_ele(y, bias, z):
 def bias_dropout_add(x: torch.Tensor, bias: torch.Tensor, dropmask: torch.Tensor, residual: torch.Tensor,
                      prob: float, training: bool) -> torch.Tensor:
     """residual + (x + bias) * dropout(dropmask)   (fused_ops.py:10-15)."""
+    _forward_only("bias_dropout_add", x, bias, residual)
     x4, r4 = _as4d(x.contiguous()), _as4d(residual.contiguous())
     b_ = bias.contiguous().to(x.dtype)
     dm = F.dropout(dropmask, p=prob, training=training)
@@ -73,6 +82,7 @@ def bias_dropout_add(x: torch.Tensor, bias: torch.Tensor, dropmask: torch.Tensor
 def bias_ele_dropout_residual(ab: torch.Tensor, b: torch.Tensor, g: torch.Tensor, dropout_mask: torch.Tensor,
                               Z_raw: torch.Tensor, prob: float, training: bool) -> torch.Tensor:
     """Z_raw + dropout(dropout_mask) * (g * (ab + b))   (fused_ops.py:18-22)."""
+    _forward_only("bias_ele_dropout_residual", ab, b, g, Z_raw)
     ab4, g4, z4 = _as4d(ab.contiguous()), _as4d(g.contiguous()), _as4d(Z_raw.contiguous())
     b_ = b.contiguous().to(ab.dtype)
     dm = F.dropout(dropout_mask, p=prob, training=training)

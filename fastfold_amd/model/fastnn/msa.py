@@ -15,6 +15,11 @@ from .ops import (ChunkMSAColumnGlobalAttention, ChunkTransition, OutProductMean
 from .triangle import PairCore
 
 
+def _private_copy(view, owner):
+    out = view.contiguous()
+    return out.clone() if out.data_ptr() == owner.data_ptr() else out
+
+
 class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
 
     def __init__(self, d_node, d_pair, c=32, n_head=8, p_drop=0.15):
@@ -206,7 +211,8 @@ class ExtraMSABlock(nn.Module):
         if m.dim() != 4 or z.dim() != 4 or m.shape[1] != s + 1 or m.shape[2] != r + 1 or z.shape[1] != r + 1:
             raise RuntimeError("ExtraMSABlock: a non-first block expects padded [1, s+1, r+1, c] / [1, r+1, r+1, c] "
                                "inputs, got %s / %s" % (tuple(m.shape), tuple(z.shape)))
-        return m[:, :s, :r, :].contiguous(), z[:, :r, :r, :].contiguous()
+        # private copies (the core runs in place) even where the slice is contiguous as it stands
+        return _private_copy(m[:, :s, :r, :], m), _private_copy(z[:, :r, :r, :], z)
 
     def _leave(self, m, z):
         if self.last_block:

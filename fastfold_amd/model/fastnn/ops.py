@@ -40,8 +40,21 @@ def _budget():
 
 
 class _PackMixin:
-    """Caches kernel-ready copies of the parameters, keyed by dtype/device and rebuilt when a
-    source parameter is modified (``_version``) or moved."""
+    """Caches kernel-ready copies of the parameters, keyed by dtype/device and rebuilt when a source parameter is
+    modified in place (its ``_version`` changes), replaced or moved, when the module is cast / moved (``_apply``) and
+    when a state dict is loaded.  A write through ``param.data`` (``p.data.copy_(w)``) changes none of these: call
+    ``invalidate_packed()`` on the module (or any parent, via ``module.apply``) after such a write."""
+
+    def invalidate_packed(self):
+        self.__dict__.pop("_pack_cache", None)
+
+    def _apply(self, fn, *args, **kwargs):
+        self.invalidate_packed()
+        return super()._apply(fn, *args, **kwargs)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.invalidate_packed()
+        return super()._load_from_state_dict(*args, **kwargs)
 
     def _packed(self, key, params, build):
         cache = self.__dict__.setdefault("_pack_cache", {})

@@ -199,7 +199,14 @@ def test_fused_attention_core_op(dev, dtype, tol, b1, b2, h, n):
     assert out.shape == (b1, b2, n, h * 32) and out.dtype == dtype
     ref = ops_np.attention_core(_np(q), _np(k), _np(v), _np(mask), _np(bias))
     assert _rel(_np(out), ref) < tol
-    with pytest.raises(RuntimeError):
-        fused_attention_core(q[..., :16].contiguous(), k[..., :16].contiguous(), v[..., :16].contiguous(), mask, bias)
+    # narrower heads run zero-padded (8 and 16: the widths of the extra-MSA and template stacks)
+    for d in (16, 8):
+        qd, kd, vd = (t[..., :d].contiguous() for t in (q, k, v))
+        outd = fused_attention_core(qd, kd, vd, mask, bias)
+        assert outd.shape == (b1, b2, n, h * d)
+        assert _rel(_np(outd), ops_np.attention_core(_np(qd), _np(kd), _np(vd), _np(mask), _np(bias))) < tol
+    # 64 / 128 (taken by the reference's Triton kernel, used by no module of the path) are refused by name
+    with pytest.raises(RuntimeError, match="64 and 128"):
+        fused_attention_core(torch.cat([q, q], -1), torch.cat([k, k], -1), torch.cat([v, v], -1), mask, bias)
     with pytest.raises(RuntimeError):
         fused_attention_core(q.cpu(), k.cpu(), v.cpu(), mask.cpu(), bias.cpu())

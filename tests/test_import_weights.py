@@ -123,3 +123,60 @@ def test_import_into_fastnn_stack(tmp_path):
     assert set(want) == set(have)
     for k, v in want.items():
         assert torch.equal(have[k], v.to(have[k].dtype)), k
+
+
+def _af2_case(seed=9, nb=2, s=6, r=10):
+    from oracle import af2_einsum_ref as af2
+    from fastfold_amd.synthetic import synth_inputs
+    params = af2.random_params(seed, nb)
+    m, z, mm, pm = synth_inputs(seed, s, r, mask_tail_frac=0.2)
+    return af2, params, m, z, mm, pm
+
+
+def test_importer_against_alphafold_einsum_oracle():
+    """Two independent routes from the same AlphaFold-layout arrays: AlphaFold's einsum conventions
+    (oracle/af2_einsum_ref.py, float64, no translation table) and importer -> nn layout -> CPU oracle.  A wrong
+    transposition, head split, left / right swap or key name in the importer's table breaks the agreement."""
+    from oracle.evoformer_ref import EvoformerStack as OracleStack
+    af2, params, m, z, mm, pm = _af2_case()
+    want_m, want_z, want_s = af2.evoformer_stack(m, z, mm, pm, params)
+    st = OracleStack(no_blocks=2).eval()
+    st.load_state_dict(iw.evoformer_nn_state_dict_from_jax(params), strict=True)
+    with torch.no_grad():
+        gm, gz, gs = st(*(torch.from_numpy(t) for t in (m, z, mm, pm)), _mask_trans=False)
+    nv = 8
+    assert float(np.abs(want_z[:nv, :nv] - z[:nv, :nv]).mean()) > 0.3           # O(1) updates
+    scale = float(np.abs(want_z).max())
+    assert np.abs(gm.numpy() - want_m)[:, :nv].max() <= 1e-4 * scale
+    assert np.abs(gz.numpy() - want_z)[:nv, :nv].max() <= 1e-4 * scale
+    assert np.abs(gs.numpy() - want_s)[:nv].max() <= 1e-4 * scale
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_imported_weights_on_the_hip_path(dev, dtype, tmp_path):
+    """A synthetic AlphaFold-layout ``.npz`` -> ``import_jax_evoformer_`` -> HIP forward, against AlphaFold's own
+    einsum conventions applied to the same arrays (no real checkpoint exists offline)."""
+    from fastfold_amd.model.fastnn import EvoformerStack
+    from fastfold_amd.synthetic import bf16_round
+    s, r, nv = 24, 40, 32
+    af2, params, m, z, mm, pm = _af2_case(seed=10, nb=2, s=s, r=r)
+    m, z = bf16_round(m), bf16_round(z)
+    path = tmp_path / "params_model_synth.npz"
+    np.savez(path, **params)
+    stack = EvoformerStack(c_m=256, c_z=128, c_s=384, no_blocks=2, blocks_per_ckpt=1).to(dev, dtype).eval()
+    res = iw.import_jax_evoformer_(stack, str(path))
+    assert not res.missing_keys and not res.unexpected_keys
+    want_m, want_z, want_s = af2.evoformer_stack(m, z, mm, pm, params)
+    with torch.no_grad():
+        gm, gz, gs = stack(*(torch.from_numpy(t).to(dev, dtype) for t in (m, z, mm, pm)), chunk_size=None)
+    gm, gz, gs = (t.float().cpu().numpy() for t in (gm, gz, gs))
+    if dtype == torch.float32:
+        scale = float(np.abs(want_z).max())
+        assert np.abs(gm - want_m)[:, :nv].max() <= 1e-4 * scale and np.abs(gz - want_z)[:nv, :nv].max() <= 1e-4 * scale
+        assert np.abs(gs - want_s)[:nv].max() <= 1e-4 * scale
+    else:
+        def rel(a, b):
+            return float(np.linalg.norm(a - b) / np.linalg.norm(b))
+        assert rel(gm[:, :nv], want_m[:, :nv]) <= 2e-2 and rel(gz[:nv, :nv], want_z[:nv, :nv]) <= 2e-2
+        assert rel(gs[:nv], want_s[:nv]) <= 2e-2

@@ -302,3 +302,56 @@ def test_empty_inputs_raise(dev):
         m, z = torch.zeros(s, r, 256, device=dev), torch.zeros(r, r, 128, device=dev)
         with torch.no_grad(), pytest.raises(RuntimeError, match="empty input"):
             blk(m, z, torch.ones(s, r, device=dev), torch.ones(r, r, device=dev))
+
+
+def test_forward_leaves_inputs_untouched_for_a_single_sequence(dev):
+    """A middle block's ``forward`` un-pads with a slice that is already contiguous when N_seq = 1; it must still
+    work on a private copy (the reference's forward never writes to its inputs)."""
+    blk = _block(dev, torch.float32, "Evoformer")
+    blk.first_block, blk.last_block = False, False
+    s, r = 1, 12
+    g = torch.Generator().manual_seed(0)
+    m = torch.randn(1, s, r + 1, 256, generator=g).to(dev)
+    z = torch.randn(1, r + 1, r + 1, 128, generator=g).to(dev)
+    mm, pm = torch.ones(s, r, device=dev), torch.ones(r, r, device=dev)
+    m0, z0 = m.clone(), z.clone()
+    with torch.no_grad():
+        a, b = blk(m, z, mm, pm)
+    assert torch.equal(m, m0) and torch.equal(z, z0)
+    assert a.shape == m.shape and float((a[:, :, :r] - m0[:, :, :r]).abs().max()) > 1e-3
+
+
+def test_packed_weights_follow_the_parameters(dev):
+    """Kernel-ready weight copies are rebuilt after in-place parameter updates, ``load_state_dict`` and casts; a
+    write through ``.data`` needs ``invalidate_packed()``."""
+    from fastfold_amd.model.fastnn.ops import Linear
+    lin = Linear(64, 32).to(dev)
+    x = torch.randn(5, 64, device=dev)
+    with torch.no_grad():
+        y0 = lin(x)
+        lin.weight.mul_(2.0)                                     # in-place op: version counter
+        assert torch.allclose(lin(x) - lin.bias, 2 * (y0 - lin.bias), atol=1e-4)
+        sd = {k: v.clone() for k, v in lin.state_dict().items()}
+        sd["weight"] = sd["weight"] * 0.5
+        lin.load_state_dict(sd)                                  # copy_ under no_grad, plus the explicit hook
+        assert torch.allclose(lin(x), y0, atol=1e-4)
+        lin.weight.data.copy_(sd["weight"] * 3.0)                # invisible to the version counter
+        lin.invalidate_packed()
+        assert torch.allclose(lin(x) - lin.bias, 3 * (y0 - lin.bias), atol=1e-4)
+        lin = lin.to(torch.bfloat16)                             # _apply drops the cache
+        assert lin(x.to(torch.bfloat16)).dtype == torch.bfloat16
+
+
+def test_elementwise_ops_refuse_to_drop_gradients(dev):
+    from fastfold_amd.model.fastnn.kernel import bias_dropout_add, bias_ele_dropout_residual, bias_sigmod_ele
+    x = torch.randn(1, 4, 6, 32, device=dev, requires_grad=True)
+    b = torch.zeros(32, device=dev)
+    dm = torch.ones(1, 1, 6, 32, device=dev)
+    with pytest.raises(NotImplementedError):
+        bias_sigmod_ele(x, b, x.detach())
+    with pytest.raises(NotImplementedError):
+        bias_dropout_add(x, b, dm, x.detach(), prob=0.1, training=False)
+    with pytest.raises(NotImplementedError):
+        bias_ele_dropout_residual(x.detach(), b, x, dm, x.detach(), prob=0.1, training=False)
+    with torch.no_grad():
+        assert bias_sigmod_ele(x, b, x).shape == x.shape
