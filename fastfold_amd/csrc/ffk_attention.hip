@@ -14,6 +14,7 @@
 // vector pipe has none.  Per-tile flags skip the key-mask add for tiles without masked keys and
 // drop trailing fully-masked tiles; the running output is rescaled only when a row maximum moves.
 #include "ffk_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -248,6 +249,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     // just before that use.
 #pragma unroll
     for (int i = 0; i < Ops16<T>::NV; ++i) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&qf.v[i])));
+    // The walk over the key tiles.  CAREFUL = false is the common case: the first tile sets the reference and no
+    // later tile looks at its probabilities - the row sum is tested once, after the walk (see below).
+    auto walk = [&](auto careful_c) {
+    constexpr bool CAREFUL = decltype(careful_c)::value;
     fetch(0, 0);
     fetch(kt_end > 1 ? 1 : 0, 1);
     int flag_nxt = fl[0];
@@ -314,8 +319,10 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
         bool move_ref = first;
         if (!first) {
             prob_tile();
-            move_ref = __builtin_amdgcn_ballot_w64(!(tsum <= REF_LIMIT)) != 0;
-            if (move_ref) score_tile();
+            if (CAREFUL) {
+                move_ref = __builtin_amdgcn_ballot_w64(!(tsum <= REF_LIMIT)) != 0;
+                if (move_ref) score_tile();
+            }
         }
         if (move_ref) {
             float mt = fmaxf(s[0], s[1]);
@@ -340,9 +347,32 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
         for (int i = 0; i < NF; ++i) MM::mma(o_acc, vc.frag(i), pf[i]);
 
     }
-
-    // the requests past the last tile must have landed before this workgroup's LDS can be handed on
+    // the requests past the last tile must have landed before the ring is reused or handed on
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+
+    // Optimistic walk first.  Probabilities are non-negative, so a finite row sum within 2^OPT_SLACK proves that
+    // no score of the row lay more than OPT_SLACK (log2 units) above the first tile's maximum: nothing overflowed,
+    // and fp32 accumulation keeps its relative precision at any such scale.  Otherwise (steeply rising scores, a
+    // first tile that is completely masked) the whole workgroup walks again with the reference moved tile by tile.
+    walk(std::false_type());
+    {
+        constexpr float OPT_LIMIT = 1.8446744e19f;    // 2^64
+        int* redo = reinterpret_cast<int*>(lds + NSLOT * NTILES * 1024 + ATT_THREADS * 16);
+        if (tid == 0) *redo = 0;
+        lds_barrier();
+        const bool bad = __builtin_amdgcn_ballot_w64(!(l_run <= OPT_LIMIT)) != 0;
+        if (bad && lane == 0) *redo = 1;
+        lds_barrier();
+        if (*redo != 0) {                              // workgroup-uniform
+            lds_barrier();
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o_acc[v] = negm[v] = 0.0f;
+            l_run = 0.0f;
+            first = true;
+            walk(std::true_type());
+        }
+    }
 
     // rows whose keys are all masked have l == 0 and produce zeros
     const float l_tot = l_run + lane_xor<32>(l_run);
@@ -395,7 +425,7 @@ __global__ void key_bias_kernel(float* kb, int* flags, const T* mask, long N, lo
 template <typename T, bool HAS_BIAS>
 int launch_attention_b(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
                        const int* flags, const void* gate, long B2, long H, long Nq, long Nk, int aflags, hipStream_t st) {
-    const size_t smem = (3 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 + ATT_THREADS * 16) * sizeof(T);   // operand ring + gate
+    const size_t smem = (3 * (size_t)(HAS_BIAS ? 8 : 4) * 1024 + ATT_THREADS * 16) * sizeof(T) + 16;   // operand ring + gate + redo flag
     static FfkLdsReservation lds_reserved;
     {
         const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)attention_kernel<T, HAS_BIAS>, smem, "ffk_attention_fwd");
