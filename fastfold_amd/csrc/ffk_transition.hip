@@ -1,6 +1,8 @@
-// Fused pair transition (see ffk_transition_fused in include/ffk.h):
-//     out = x + W2 . relu( W1 . LayerNorm(x) + b1 ) + b2        (128 -> 512 -> 128 channels, bf16)
-// with the 512-channel hidden activation never leaving the registers.
+// Fused transition (see ffk_transition_fused in include/ffk.h):
+//     out = x + W2 . relu( W1 . LayerNorm(x) + b1 ) + b2        (C -> 4C -> C channels, C = 128 or 256, bf16)
+// with the hidden activation never leaving the registers.  The description below is for C = 128 (pair
+// transition); the MSA transition (C = 256) walks the hidden layer in 32 chunks of 32 channels, so that its
+// weight rings take the same 64 KB and two workgroups still fit a CU.
 //
 // A workgroup (4 wavefronts) owns 128 rows, a wavefront 32 of them from start to end.  Set-up: the rows
 // are fetched once, normalised in registers (16 lanes per row) and passed through LDS into the MFMA
@@ -23,12 +25,21 @@ namespace {
 typedef bf16_t T;
 constexpr int TR_THREADS = 256;
 constexpr int TR_BM = 128;                     // rows per workgroup
-constexpr int TR_C = 128, TR_H = 512;
-constexpr int TR_HC = 64;                      // hidden channels per chunk
-constexpr int TR_NCHUNK = TR_H / TR_HC;        // 8
-constexpr int TR_W1SLOT = TR_HC * TR_C * 2;    // 64 rows of 256 bytes (16 KB)
-constexpr int TR_W2SLOT = TR_C * TR_HC * 2;    // 128 rows of 128 bytes (16 KB)
-constexpr int TR_XP = TR_C * 2 + 16;           // pitch of the normalised rows (set-up only)
+template <int C> struct TrGeo {
+    static constexpr int H = 4 * C;
+    static constexpr int HC = C == 128 ? 64 : 32;   // hidden channels per chunk
+    static constexpr int NCHUNK = H / HC;
+    static constexpr int W1SLOT = HC * C * 2;       // HC rows of 2 C bytes (16 KB)
+    static constexpr int W2SLOT = C * HC * 2;       // C rows of 2 HC bytes (16 KB)
+    static constexpr int XP = C * 2 + 16;           // pitch of the normalised rows (set-up only)
+    static constexpr int NC1 = C / 8;               // 16-byte columns of a W1 row
+    static constexpr int NC2 = HC / 8;              // 16-byte columns of a W2 row
+    static constexpr int RP2 = 256 / (HC * 2);      // W2 rows per 256 bytes of LDS: the swizzle period
+    static constexpr int KS1 = C / 16, KS2 = HC / 16, HT = HC / 32, CT = C / 32;
+    static constexpr size_t SMEM_RINGS = 2 * (size_t)W1SLOT + 2 * W2SLOT + H * sizeof(float);
+    static constexpr size_t SMEM_ROWS = (size_t)TR_BM * XP;
+    static constexpr size_t SMEM = SMEM_RINGS > SMEM_ROWS ? SMEM_RINGS : SMEM_ROWS;
+};
 
 __device__ __forceinline__ int tr_tau(int i) { return ((i >> 2) & 1) * 16 + (i >> 3) * 4 + (i & 3); }
 // i = 8a + 4h + b  ->  16 (a / 2) + 8h + 4 (a % 2) + b
@@ -39,16 +50,19 @@ __device__ __forceinline__ void tr_load_lds(const T* src, unsigned char* dst_wav
                                      (__attribute__((address_space(3))) void*)dst_wave, 16, 0, 0);
 }
 
+template <int TR_C>
 __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
                                                                         const T* __restrict__ gamma, const T* __restrict__ beta,
                                                                         const T* __restrict__ w1, const T* __restrict__ b1,
                                                                         const T* __restrict__ w2, const T* __restrict__ b2,
                                                                         long M, float eps) {
     typedef Mma<T> MM;
+    typedef TrGeo<TR_C> G;
+    constexpr int TR_H = G::H, TR_HC = G::HC, TR_NCHUNK = G::NCHUNK, TR_W1SLOT = G::W1SLOT, TR_W2SLOT = G::W2SLOT, TR_XP = G::XP;
     extern __shared__ __align__(16) unsigned char smem[];
-    unsigned char* s_w1 = smem;                           // [2][64][256 B]
-    unsigned char* s_w2 = smem + 2 * TR_W1SLOT;           // [2][128][128 B]
-    float* s_b1 = reinterpret_cast<float*>(s_w2 + 2 * TR_W2SLOT);   // [512]
+    unsigned char* s_w1 = smem;                           // [2][HC][2 C bytes]
+    unsigned char* s_w2 = smem + 2 * TR_W1SLOT;           // [2][C][2 HC bytes]
+    float* s_b1 = reinterpret_cast<float*>(s_w2 + 2 * TR_W2SLOT);   // [H]
     unsigned char* s_x = smem;                            // [128][TR_XP], set-up only (aliases the rings)
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -58,41 +72,45 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
 
     // ---- set-up: rows -> LayerNorm in registers -> LDS -> this wave's fragments ----
     {
-        const int c8 = tid & 15, r0 = tid >> 4;           // 16 lanes per row, 16 rows per pass, 8 passes
+        constexpr int LPR = TR_C / 8, RPP = TR_THREADS / LPR, NPASS = TR_BM / RPP;   // lanes per row, rows per pass
+        const int c8 = tid % LPR, r0 = tid / LPR;
         const Vec16<T> g = ld16(gamma + c8 * 8), b = ld16(beta + c8 * 8);
-        Vec16<T> v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            long m = m0 + r0 + 16 * i;
-            m = m < M ? m : M - 1;                        // clamped: rows past the end are never stored
-            v[i] = ld16(x + m * TR_C + c8 * 8);
-        }
+        for (int i0 = 0; i0 < NPASS; i0 += 8) {
+            Vec16<T> v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float f[8], s = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                f[e] = (float)v[i].e[e];
-                s += f[e];
+            for (int i = 0; i < 8; ++i) {
+                long m = m0 + r0 + RPP * (i0 + i);
+                m = m < M ? m : M - 1;                    // clamped: rows past the end are never stored
+                v[i] = ld16(x + m * TR_C + c8 * 8);
             }
-            const float mu = group_sum(s, 16) * (1.0f / TR_C);
-            float q = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                f[e] -= mu;
-                q += f[e] * f[e];
+            for (int i = 0; i < 8; ++i) {
+                float f[8], s = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    f[e] = (float)v[i].e[e];
+                    s += f[e];
+                }
+                const float mu = group_sum(s, LPR) * (1.0f / TR_C);
+                float q = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    f[e] -= mu;
+                    q += f[e] * f[e];
+                }
+                const float rs = rsqrtf(group_sum(q, LPR) * (1.0f / TR_C) + eps);
+                Vec16<T> y;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) y.e[e] = (T)(f[e] * rs * (float)g.e[e] + (float)b.e[e]);
+                *reinterpret_cast<Vec16<T>*>(s_x + (r0 + RPP * (i0 + i)) * TR_XP + c8 * 16) = y;
             }
-            const float rs = rsqrtf(group_sum(q, 16) * (1.0f / TR_C) + eps);
-            Vec16<T> y;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) y.e[e] = (T)(f[e] * rs * (float)g.e[e] + (float)b.e[e]);
-            *reinterpret_cast<Vec16<T>*>(s_x + (r0 + 16 * i) * TR_XP + c8 * 16) = y;
         }
     }
     lds_barrier();
-    bf16x8 xf[8];                                          // rows 32 wave + l32, all of K = 128
+    bf16x8 xf[G::KS1];                                     // rows 32 wave + l32, all of K = C
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
+    for (int ks = 0; ks < G::KS1; ++ks)
         xf[ks] = *reinterpret_cast<const bf16x8*>(s_x + (wave * 32 + l32) * TR_XP + ks * 32 + half * 16);
     lds_barrier();                                         // the row buffer is free: the rings may overwrite it
     for (int i = tid; i < TR_H; i += TR_THREADS) s_b1[i] = (float)b1[i];
@@ -102,15 +120,15 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
     const T* w1src[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int v = i * TR_THREADS + tid, rho = v >> 4, c = v & 15;
+        const int v = i * TR_THREADS + tid, rho = v / G::NC1, c = v % G::NC1;
         w1src[i] = w1 + (long)((rho & ~31) + tr_sigma(rho & 31)) * TR_C + ((c ^ (rho & 15)) * 8);
     }
     // W2 chunk: LDS row rho (0..127) holds weight row 32 * (rho / 32) + tau(rho % 32); 8 columns
     const T* w2src[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int v = i * TR_THREADS + tid, rho = v >> 3, c = v & 7;
-        w2src[i] = w2 + (long)((rho & ~31) + tr_tau(rho & 31)) * TR_H + ((c ^ ((rho >> 1) & 7)) * 8);
+        const int v = i * TR_THREADS + tid, rho = v / G::NC2, c = v % G::NC2;
+        w2src[i] = w2 + (long)((rho & ~31) + tr_tau(rho & 31)) * TR_H + ((c ^ ((rho / G::RP2) & (G::NC2 - 1))) * 8);
     }
     auto fetch = [&](int q) {
         unsigned char* d1 = s_w1 + (q & 1) * TR_W1SLOT + wave * 1024;
@@ -121,18 +139,20 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
         for (int i = 0; i < 4; ++i) tr_load_lds(w2src[i] + q * TR_HC, d2 + i * (TR_THREADS * 16));
     };
 
-    f32x16 acc2[4];                                        // out^T tiles: channels 32 ct + 16 half + v, row l32
+    f32x16 acc2[G::CT];                                    // out^T tiles: channels 32 ct + 16 half + v, row l32
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < G::CT; ++c)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc2[c][v] = 0.0f;
 
-    int w1off[8];                                          // W1 fragment of hidden tile 0: row l32, column 2 ks + half
+    // W1 fragment of hidden tile 0: row l32, column 2 ks + half.  The swizzle touches the low four column bits only,
+    // so K steps 8 .. 15 (C = 256) are the first eight plus 256 bytes.
+    int w1off[8];
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) w1off[ks] = l32 * 256 + (((2 * ks + half) ^ (l32 & 15)) << 4);
-    int w2off[4];                                          // W2 fragment of c-tile 0: row l32, column 2 ks + half
+    for (int ks = 0; ks < 8; ++ks) w1off[ks] = l32 * (TR_C * 2) + (((2 * ks + half) ^ (l32 & 15)) << 4);
+    int w2off[G::KS2];                                     // W2 fragment of c-tile 0: row l32, column 2 ks + half
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) w2off[ks] = l32 * 128 + (((2 * ks + half) ^ ((l32 >> 1) & 7)) << 4);
+    for (int ks = 0; ks < G::KS2; ++ks) w2off[ks] = l32 * (TR_HC * 2) + (((2 * ks + half) ^ ((l32 / G::RP2) & (G::NC2 - 1))) << 4);
 
     fetch(0);
     for (int q = 0; q < TR_NCHUNK; ++q) {
@@ -141,9 +161,9 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
         if (q + 1 < TR_NCHUNK) fetch(q + 1);
         const unsigned char* wa = s_w1 + (q & 1) * TR_W1SLOT;
         const unsigned char* wb = s_w2 + (q & 1) * TR_W2SLOT;
-        bf16x8 hf[2][2];                                   // [hidden tile][K step]: the chunk's N operand
+        bf16x8 hf[G::HT][2];                               // [hidden tile][K step]: the chunk's N operand
 #pragma unroll
-        for (int ht = 0; ht < 2; ++ht) {
+        for (int ht = 0; ht < G::HT; ++ht) {
             f32x16 h;
             // registers 0..7: hidden 8 half + 0..7 of the tile, registers 8..15: 16 + 8 half + 0..7
             const float* bp = s_b1 + q * TR_HC + ht * 32 + 8 * half;
@@ -154,18 +174,18 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
                 for (int b = 0; b < 4; ++b) h[4 * a + b] = b4[b];
             }
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks)
-                MM::mma(h, *reinterpret_cast<const bf16x8*>(wa + ht * 32 * 256 + w1off[ks]), xf[ks]);
+            for (int ks = 0; ks < G::KS1; ++ks)
+                MM::mma(h, *reinterpret_cast<const bf16x8*>(wa + ht * 32 * (TR_C * 2) + w1off[ks & 7] + (ks >> 3) * 256), xf[ks]);
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int t = 0; t < 8; ++t) hf[ht][j][t] = (T)relu_f(h[8 * j + t]);
         }
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
+        for (int ks = 0; ks < G::KS2; ++ks)
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-                MM::mma(acc2[c], *reinterpret_cast<const bf16x8*>(wb + c * 32 * 128 + w2off[ks]), hf[ks >> 1][ks & 1]);
+            for (int c = 0; c < G::CT; ++c)
+                MM::mma(acc2[c], *reinterpret_cast<const bf16x8*>(wb + c * 32 * (TR_HC * 2) + w2off[ks]), hf[ks >> 1][ks & 1]);
     }
 
     // ---- epilogue: lane = row, registers = 16 consecutive channels ----
@@ -173,7 +193,7 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
     const bool ok = row < M;
     const long rc = ok ? row : M - 1;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < G::CT; ++c) {
         const int ch = c * 32 + 16 * half;
         const long o = rc * TR_C + ch;
         u32x4 bv[2], rv[2];
@@ -215,21 +235,27 @@ extern "C" int ffk_transition_fused(void* out, const void* x, void* xtail, const
                                     float eps, int dtype, void* stream) {
     FFK_REQUIRE(out && x && gamma && beta && w1 && b1 && w2 && b2, FFK_ERR_NULL, "ffk_transition_fused: null pointer");
     FFK_REQUIRE(dtype == FFK_BF16, FFK_ERR_DTYPE, "ffk_transition_fused: bf16 only (dtype tag %d)", dtype);
-    FFK_REQUIRE(C == TR_C && hidden == TR_H, FFK_ERR_UNSUPPORTED, "ffk_transition_fused: built for 128 -> 512 -> 128, got %ld -> %ld",
-                (long)C, (long)hidden);
+    FFK_REQUIRE((C == 128 || C == 256) && hidden == 4 * C, FFK_ERR_UNSUPPORTED,
+                "ffk_transition_fused: built for 128 -> 512 -> 128 and 256 -> 1024 -> 256, got %ld -> %ld", (long)C, (long)hidden);
     FFK_REQUIRE(M > 0 && M < (1L << 31) * (long)TR_BM, FFK_ERR_SHAPE, "ffk_transition_fused: bad row count %ld", (long)M);
     FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(x) && ffk_aligned16(gamma) && ffk_aligned16(beta) && ffk_aligned16(w1) &&
                     ffk_aligned16(w2) && ffk_aligned16(b2) && ffk_aligned16(xtail),
                 FFK_ERR_ALIGN, "ffk_transition_fused: buffers must be 16-byte aligned");
-    const size_t smem = 2 * (size_t)TR_W1SLOT + 2 * TR_W2SLOT + TR_H * sizeof(float);
-    static FfkLdsReservation lds_reserved;
-    {
-        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel, smem, "ffk_transition_fused");
-        if (rc_lds != FFK_OK) return rc_lds;
-    }
     const unsigned grid = (unsigned)ffk_cdiv(M, TR_BM);
-    transition_fused_kernel<<<grid, TR_THREADS, smem, (hipStream_t)stream>>>((T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta,
-                                                                            (const T*)w1, (const T*)b1, (const T*)w2,
-                                                                            (const T*)b2, (long)M, eps);
+    if (C == 128) {
+        static FfkLdsReservation lds_reserved;
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel<128>, TrGeo<128>::SMEM, "ffk_transition_fused");
+        if (rc_lds != FFK_OK) return rc_lds;
+        transition_fused_kernel<128><<<grid, TR_THREADS, TrGeo<128>::SMEM, (hipStream_t)stream>>>(
+            (T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta, (const T*)w1, (const T*)b1, (const T*)w2,
+            (const T*)b2, (long)M, eps);
+    } else {
+        static FfkLdsReservation lds_reserved;
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel<256>, TrGeo<256>::SMEM, "ffk_transition_fused");
+        if (rc_lds != FFK_OK) return rc_lds;
+        transition_fused_kernel<256><<<grid, TR_THREADS, TrGeo<256>::SMEM, (hipStream_t)stream>>>(
+            (T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta, (const T*)w1, (const T*)b1, (const T*)w2,
+            (const T*)b2, (long)M, eps);
+    }
     return ffk_check_launch("ffk_transition_fused");
 }

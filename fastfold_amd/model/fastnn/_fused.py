@@ -153,13 +153,17 @@ def xtail_ptr(xtail, off=0):
     return None if xtail is None else xtail.data_ptr() + off
 
 
+# False: every transition runs as projection + GEMM with the hidden activation in HBM (tests compare the two)
+_FUSED_TRANSITION = True
+
+
 def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget, xtail=None):
     """out = x + W2 relu(W1 LN(x) + b1) + b2 over rows of x [M, C]; out may alias x.  ``xtail`` (here and in the
     other sub-modules): int8 tensor of x's shape holding the tail bytes of x / out as an extended residual stream."""
     M, C = x.shape
     dt, dev = x.dtype, x.device
     es = es_of(dt)
-    if dt == torch.bfloat16 and C == 128 and hidden == 512 and ln is not None:
+    if dt == torch.bfloat16 and C in (128, 256) and hidden == 4 * C and ln is not None and _FUSED_TRANSITION:
         # both layers in one kernel, hidden activation kept on chip
         _lib.transition_fused(out, x, ln[0], ln[1], w1_pk, b1_pk, w2, b2, M=M, C=C, hidden=hidden, xtail=xtail)
         return out

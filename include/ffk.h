@@ -324,7 +324,7 @@ int ffk_opm_fused(void* out, const void* resid, void* xtail, const void* a_t, co
                   const void* bias, const float* norm, int64_t r, int64_t spad, float eps, int dtype,
                   void* stream);
 
-/* Fused pair transition (bf16, C = 128, hidden = 512):
+/* Fused transition (bf16; C = 128 with hidden = 512: pair transition, C = 256 with hidden = 1024: MSA transition):
  *     out = x + W2 . relu( W1 . LayerNorm(x; gamma, beta, eps) + b1 ) + b2
  * x, out : [M, C] row-major (may alias); xtail : NULL or the [M, C] tail bytes of x / out as an extended residual
  * stream (the LayerNorm reads x alone); w1 : [hidden, C]; w2 : [C, hidden]; b1 : [hidden]; b2 : [C].

@@ -368,31 +368,36 @@ def test_opm_fused_kernel(dev, r, s):
         _lib.opm_fused(out, resid, a_t, b_t, w_ed, bias, norm, r=r + 8, spad=s, eps=1e-3)
 
 
+@pytest.mark.parametrize("C", [128, 256])
 @pytest.mark.parametrize("M", [256, 1000, 70000])
-def test_transition_fused_kernel(dev, M):
-    """ffk_transition_fused against float64 numpy, including a ragged last workgroup and in-place use."""
+def test_transition_fused_kernel(dev, M, C):
+    """ffk_transition_fused (pair width 128, MSA width 256) against float64 numpy, including a ragged last workgroup
+    and in-place use."""
     from fastfold_amd import _lib
     dtype = torch.bfloat16
-    g = torch.Generator().manual_seed(M)
-    x = (torch.randn(M, 128, generator=g) * 1.5 + 0.2).to(dev, dtype)
-    gam = (1 + 0.1 * torch.randn(128, generator=g)).to(dev, dtype)
-    bet = (0.1 * torch.randn(128, generator=g)).to(dev, dtype)
-    w1 = (torch.randn(512, 128, generator=g) / 128 ** 0.5).to(dev, dtype)
-    b1 = torch.randn(512, generator=g).to(dev, dtype)
-    w2 = (torch.randn(128, 512, generator=g) / 512 ** 0.5).to(dev, dtype)
-    b2 = torch.randn(128, generator=g).to(dev, dtype)
+    Hd = 4 * C
+    g = torch.Generator().manual_seed(M + C)
+    x = (torch.randn(M, C, generator=g) * 1.5 + 0.2).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    w1 = (torch.randn(Hd, C, generator=g) / C ** 0.5).to(dev, dtype)
+    b1 = torch.randn(Hd, generator=g).to(dev, dtype)
+    w2 = (torch.randn(C, Hd, generator=g) / Hd ** 0.5).to(dev, dtype)
+    b2 = torch.randn(C, generator=g).to(dev, dtype)
     out = torch.full_like(x, 7.0)
-    _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=128, hidden=512)
+    _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=C, hidden=Hd)
     xn = _np(torch.from_numpy(ops_np.layer_norm(_np(x), _np(gam), _np(bet))).to(torch.bfloat16))
     h = np.maximum(ops_np.linear(xn, _np(w1), _np(b1)), 0)
     h = _np(torch.from_numpy(h).to(torch.bfloat16))                         # hidden is rounded to bf16 on chip
     upd = ops_np.linear(h, _np(w2), _np(b2))
     assert _rel(_np(out) - _np(x), upd) < TOL[dtype]
     x2 = x.clone()
-    _lib.transition_fused(x2, x2, gam, bet, w1, b1, w2, b2, M=M, C=128, hidden=512)
+    _lib.transition_fused(x2, x2, gam, bet, w1, b1, w2, b2, M=M, C=C, hidden=Hd)
     assert torch.equal(x2, out)
     with pytest.raises(RuntimeError):
         _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=64, hidden=256)
+    with pytest.raises(RuntimeError):
+        _lib.transition_fused(out, x, gam, bet, w1, b1, w2, b2, M=M, C=C, hidden=2 * C)
 
 
 @pytest.mark.parametrize("r", [64, 104])

@@ -127,9 +127,10 @@ def test_bgemm_residual_tail(dev, M, N, K):
     assert np.sqrt((err ** 2).mean()) < 5e-3 and err.max() < 0.05
 
 
-def test_transition_fused_residual_tail(dev):
+@pytest.mark.parametrize("C", [128, 256])
+def test_transition_fused_residual_tail(dev, C):
     from fastfold_amd import _lib
-    M, C, Hd = 700, 128, 512
+    M, Hd = 700, 4 * C
     g = torch.Generator().manual_seed(3)
     gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, BF)
     bet = (0.1 * torch.randn(C, generator=g)).to(dev, BF)
