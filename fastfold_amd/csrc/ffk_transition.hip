@@ -25,7 +25,7 @@ namespace {
 typedef bf16_t T;
 constexpr int TR_THREADS = 256;
 constexpr int TR_BM = 128;                     // rows per workgroup
-template <int C> struct TrGeo {
+template <int C, int NS> struct TrGeo {
     static constexpr int H = 4 * C;
     static constexpr int HC = C == 128 ? 64 : 32;   // hidden channels per chunk
     static constexpr int NCHUNK = H / HC;
@@ -36,7 +36,7 @@ template <int C> struct TrGeo {
     static constexpr int NC2 = HC / 8;              // 16-byte columns of a W2 row
     static constexpr int RP2 = 256 / (HC * 2);      // W2 rows per 256 bytes of LDS: the swizzle period
     static constexpr int KS1 = C / 16, KS2 = HC / 16, HT = HC / 32, CT = C / 32;
-    static constexpr size_t SMEM_RINGS = 2 * (size_t)W1SLOT + 2 * W2SLOT + H * sizeof(float);
+    static constexpr size_t SMEM_RINGS = NS * (size_t)W1SLOT + NS * W2SLOT + H * sizeof(float);
     static constexpr size_t SMEM_ROWS = (size_t)TR_BM * XP;
     static constexpr size_t SMEM = SMEM_RINGS > SMEM_ROWS ? SMEM_RINGS : SMEM_ROWS;
 };
@@ -50,19 +50,22 @@ __device__ __forceinline__ void tr_load_lds(const T* src, unsigned char* dst_wav
                                      (__attribute__((address_space(3))) void*)dst_wave, 16, 0, 0);
 }
 
-template <int TR_C>
-__global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
+// NS: slots of the weight rings.  Two slots (one chunk in flight) when two workgroups share a CU and cover each
+// other's waits; four when the launch has at most one workgroup per CU and the chunk stream has to hide the whole
+// memory latency by itself (a chunk is multiplied in less than half a microsecond).
+template <int TR_C, int NS>
+__global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
                                                                         const T* __restrict__ gamma, const T* __restrict__ beta,
                                                                         const T* __restrict__ w1, const T* __restrict__ b1,
                                                                         const T* __restrict__ w2, const T* __restrict__ b2,
                                                                         long M, float eps) {
     typedef Mma<T> MM;
-    typedef TrGeo<TR_C> G;
+    typedef TrGeo<TR_C, NS> G;
     constexpr int TR_H = G::H, TR_HC = G::HC, TR_NCHUNK = G::NCHUNK, TR_W1SLOT = G::W1SLOT, TR_W2SLOT = G::W2SLOT, TR_XP = G::XP;
     extern __shared__ __align__(16) unsigned char smem[];
-    unsigned char* s_w1 = smem;                           // [2][HC][2 C bytes]
-    unsigned char* s_w2 = smem + 2 * TR_W1SLOT;           // [2][C][2 HC bytes]
-    float* s_b1 = reinterpret_cast<float*>(s_w2 + 2 * TR_W2SLOT);   // [H]
+    unsigned char* s_w1 = smem;                           // [NS][HC][2 C bytes]
+    unsigned char* s_w2 = smem + NS * TR_W1SLOT;          // [NS][C][2 HC bytes]
+    float* s_b1 = reinterpret_cast<float*>(s_w2 + NS * TR_W2SLOT);  // [H]
     unsigned char* s_x = smem;                            // [128][TR_XP], set-up only (aliases the rings)
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -130,13 +133,14 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
         const int v = i * TR_THREADS + tid, rho = v / G::NC2, c = v % G::NC2;
         w2src[i] = w2 + (long)((rho & ~31) + tr_tau(rho & 31)) * TR_H + ((c ^ ((rho / G::RP2) & (G::NC2 - 1))) * 8);
     }
-    auto fetch = [&](int q) {
-        unsigned char* d1 = s_w1 + (q & 1) * TR_W1SLOT + wave * 1024;
+    auto fetch = [&](int q) {                              // past the last chunk it is fetched again (into a free slot)
+        const int qc = q < TR_NCHUNK ? q : TR_NCHUNK - 1;
+        unsigned char* d1 = s_w1 + (q % NS) * TR_W1SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) tr_load_lds(w1src[i] + (long)q * TR_HC * TR_C, d1 + i * (TR_THREADS * 16));
-        unsigned char* d2 = s_w2 + (q & 1) * TR_W2SLOT + wave * 1024;
+        for (int i = 0; i < 4; ++i) tr_load_lds(w1src[i] + (long)qc * TR_HC * TR_C, d1 + i * (TR_THREADS * 16));
+        unsigned char* d2 = s_w2 + (q % NS) * TR_W2SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) tr_load_lds(w2src[i] + q * TR_HC, d2 + i * (TR_THREADS * 16));
+        for (int i = 0; i < 4; ++i) tr_load_lds(w2src[i] + qc * TR_HC, d2 + i * (TR_THREADS * 16));
     };
 
     f32x16 acc2[G::CT];                                    // out^T tiles: channels 32 ct + 16 half + v, row l32
@@ -154,13 +158,15 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
 #pragma unroll
     for (int ks = 0; ks < G::KS2; ++ks) w2off[ks] = l32 * (TR_HC * 2) + (((2 * ks + half) ^ ((l32 / G::RP2) & (G::NC2 - 1))) << 4);
 
-    fetch(0);
+#pragma unroll
+    for (int q = 0; q < NS - 1; ++q) fetch(q);
     for (int q = 0; q < TR_NCHUNK; ++q) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // chunk q has landed (this wave's part)
-        __builtin_amdgcn_s_barrier();                        // ... everyone's; nobody still reads the other slots
-        if (q + 1 < TR_NCHUNK) fetch(q + 1);
-        const unsigned char* wa = s_w1 + (q & 1) * TR_W1SLOT;
-        const unsigned char* wb = s_w2 + (q & 1) * TR_W2SLOT;
+        // chunk q has landed (this wave's part) once only the NS - 2 younger chunks (8 loads each) are outstanding
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (NS - 2)) : "memory");
+        __builtin_amdgcn_s_barrier();                        // ... everyone's; nobody still reads the slot of chunk q - 1
+        fetch(q + NS - 1);
+        const unsigned char* wa = s_w1 + (q % NS) * TR_W1SLOT;
+        const unsigned char* wb = s_w2 + (q % NS) * TR_W2SLOT;
         bf16x8 hf[G::HT][2];                               // [hidden tile][K step]: the chunk's N operand
 #pragma unroll
         for (int ht = 0; ht < G::HT; ++ht) {
@@ -187,6 +193,8 @@ __global__ __launch_bounds__(TR_THREADS, 2) void transition_fused_kernel(T* __re
             for (int c = 0; c < G::CT; ++c)
                 MM::mma(acc2[c], *reinterpret_cast<const bf16x8*>(wb + c * 32 * (TR_HC * 2) + w2off[ks]), hf[ks >> 1][ks & 1]);
     }
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the re-fetches past the last chunk
 
     // ---- epilogue: lane = row, registers = 16 consecutive channels ----
     const long row = m0 + wave * 32 + l32;
@@ -242,20 +250,22 @@ extern "C" int ffk_transition_fused(void* out, const void* x, void* xtail, const
                     ffk_aligned16(w2) && ffk_aligned16(b2) && ffk_aligned16(xtail),
                 FFK_ERR_ALIGN, "ffk_transition_fused: buffers must be 16-byte aligned");
     const unsigned grid = (unsigned)ffk_cdiv(M, TR_BM);
+    const bool deep = grid <= 256 + 128;                     // at most ~one workgroup per CU: four-slot rings
+#define FFK_TR_LAUNCH(CC, NS)                                                                                           \
+    do {                                                                                                                \
+        static FfkLdsReservation lds_reserved;                                                                          \
+        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel<CC, NS>, TrGeo<CC, NS>::SMEM, \
+                                           "ffk_transition_fused");                                                     \
+        if (rc_lds != FFK_OK) return rc_lds;                                                                            \
+        transition_fused_kernel<CC, NS><<<grid, TR_THREADS, TrGeo<CC, NS>::SMEM, (hipStream_t)stream>>>(                \
+            (T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta, (const T*)w1, (const T*)b1, (const T*)w2, \
+            (const T*)b2, (long)M, eps);                                                                                \
+    } while (0)
     if (C == 128) {
-        static FfkLdsReservation lds_reserved;
-        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel<128>, TrGeo<128>::SMEM, "ffk_transition_fused");
-        if (rc_lds != FFK_OK) return rc_lds;
-        transition_fused_kernel<128><<<grid, TR_THREADS, TrGeo<128>::SMEM, (hipStream_t)stream>>>(
-            (T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta, (const T*)w1, (const T*)b1, (const T*)w2,
-            (const T*)b2, (long)M, eps);
+        if (deep) FFK_TR_LAUNCH(128, 4); else FFK_TR_LAUNCH(128, 2);
     } else {
-        static FfkLdsReservation lds_reserved;
-        const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)transition_fused_kernel<256>, TrGeo<256>::SMEM, "ffk_transition_fused");
-        if (rc_lds != FFK_OK) return rc_lds;
-        transition_fused_kernel<256><<<grid, TR_THREADS, TrGeo<256>::SMEM, (hipStream_t)stream>>>(
-            (T*)out, (const T*)x, (int8_t*)xtail, (const T*)gamma, (const T*)beta, (const T*)w1, (const T*)b1, (const T*)w2,
-            (const T*)b2, (long)M, eps);
+        if (deep) FFK_TR_LAUNCH(256, 4); else FFK_TR_LAUNCH(256, 2);
     }
+#undef FFK_TR_LAUNCH
     return ffk_check_launch("ffk_transition_fused");
 }
