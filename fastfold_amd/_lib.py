@@ -134,7 +134,7 @@ class Tile(ctypes.Structure):
         ("s_o", c_int64), ("s_i", c_int64), ("s_h", c_int64), ("s_d", c_int64),
         ("gate_ld", c_int64), ("m_so", c_int64), ("m_si", c_int64),
         ("inner", c_int), ("kind", c_int), ("act", c_int), ("ncols", c_int), ("glu", c_int),
-        ("scale", c_float), ("gate_rows", c_int), ("s_blk", c_int),
+        ("scale", c_float), ("gate_rows", c_int), ("reserved", c_int),
         ("xtail", c_void_p),
     ]
 
@@ -158,7 +158,7 @@ SIGNATURES["ffk_fused_linear"] = [ctypes.POINTER(LinearDesc), _P]
 
 def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, gate_ld=0, rowmask=None,
               m_so=0, m_si=0, s_o=0, s_i=0, s_h=32, s_d=1, inner=1, act=FFK_ACT_NONE, ncols=128, glu=0,
-              scale=1.0, gate_rows=0, xtail=None, s_blk=0):
+              scale=1.0, gate_rows=0, xtail=None):
     """Builds one epilogue descriptor; tensors may be passed directly (their data_ptr is taken).  ``xtail`` is the
     int8 tail tensor (or its address) of ``resid`` / ``out`` as an extended residual stream."""
     def p(t):
@@ -169,7 +169,6 @@ def make_tile(out, *, kind=FFK_TILE_STRIDED, bias=None, resid=None, gate=None, g
     t.gate_ld, t.m_so, t.m_si = gate_ld, m_so, m_si
     t.inner, t.kind, t.act, t.ncols, t.glu, t.scale = inner, kind, act, ncols, glu, scale
     t.gate_rows = gate_rows
-    t.s_blk = s_blk
     t.xtail = p(xtail)
     return t
 
@@ -228,7 +227,6 @@ class BgemmDesc(ctypes.Structure):
         ("inner", c_int), ("M", c_int), ("N", c_int), ("K", c_int), ("batch", c_int),
         ("dtype", c_int), ("act", c_int), ("out_f32", c_int),
         ("scale", c_float), ("div_eps", c_float),
-        ("k_blocked", c_int), ("reserved", c_int), ("a_kbs", c_int64), ("b_kbs", c_int64),
     ]
 
 
@@ -239,10 +237,9 @@ SIGNATURES["ffk_key_bias"] = [_P, _P, _P, _L, _L, _L, _L, _I, _P]
 
 def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, inner=None, s_o=0, s_i=None,
              s_h=32, s_d=1, bias=None, resid=None, rowdiv=None, div_eps=0.0, act=FFK_ACT_NONE, scale=1.0,
-             out_f32=False, dtype=None, xtail=None, a_kbs=0, b_kbs=0):
+             out_f32=False, dtype=None, xtail=None):
     """Launches ``ffk_bgemm_nt``; default output addressing is row-major [M, N] (``s_i`` = N).  ``xtail``: int8 tail
-    of ``resid`` / ``out`` as an extended residual stream.  ``a_kbs`` / ``b_kbs`` non-zero: K-blocked operands (element
-    (m, k) at (k // 32) * kbs + m * 32 + k % 32)."""
+    of ``resid`` / ``out`` as an extended residual stream."""
     def p(t):
         return None if t is None else (t if isinstance(t, int) else t.data_ptr())
     d = BgemmDesc()
@@ -254,7 +251,6 @@ def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, i
     d.M, d.N, d.K, d.batch = M, N, K, batch
     d.dtype = dtype_tag(a.dtype if dtype is None else dtype)
     d.act, d.out_f32, d.scale, d.div_eps = act, 1 if out_f32 else 0, scale, div_eps
-    d.k_blocked, d.a_kbs, d.b_kbs = (1 if a_kbs or b_kbs else 0), a_kbs, b_kbs
     call("ffk_bgemm_nt", ctypes.byref(d), stream_ptr())
 
 

@@ -298,8 +298,6 @@ extern "C" int ffk_bgemm_nt(const ffk_bgemm_desc* d, void* stream) {
         int status = FFK_OK;
         if (ffk_bgemm_big_try(d, st, &status)) return status;
     }
-    FFK_REQUIRE(!d->k_blocked, FFK_ERR_UNSUPPORTED,
-                "ffk_bgemm_nt: K-blocked operands need bf16, K %% 32 == 0, K >= 96, M >= 256, N >= 64 and a bf16 output");
     if (d->dtype == FFK_BF16) {
         return d->out_f32 ? launch_bgemm<bf16_t, float>(*d, st) : launch_bgemm<bf16_t, bf16_t>(*d, st);
     } else if (d->dtype == FFK_F32) {

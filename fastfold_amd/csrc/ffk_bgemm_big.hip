@@ -75,9 +75,6 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
     // bank conflicts position (row, c) holds global column  c ^ ((row >> 2) & 3)  of the chunk.
     // The chunk stream runs on across tiles: while the last chunks of one tile are multiplied and its
     // results stored, the first chunks of the next tile are already arriving.
-    // K-blocked operands keep the 32-wide chunk of consecutive rows contiguous (a wave's request is one KB instead
-    // of sixteen 64-byte pieces 2 * lda bytes apart); the chunk of a row then advances by the block stride.
-    const long kstep_a = d.k_blocked ? d.a_kbs : BG_BK, kstep_b = d.k_blocked ? d.b_kbs : BG_BK;
     const T* src[NLD];
     unsigned f_t = 0;          // tile (of this workgroup) being fetched
     int f_kc = 0;              // next chunk of it
@@ -94,18 +91,18 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             if (i < BM / 128) {
                 long m = fm0 + row;
                 m = m < M ? m : M - 1;                       // clamped once; such rows are never stored
-                src[i] = A + m * (d.k_blocked ? 32 : d.lda) + g * 8;
+                src[i] = A + m * d.lda + g * 8;
             } else {
                 long n = fn0 + row - BM;
                 n = n < N ? n : N - 1;
-                src[i] = B + n * (d.k_blocked ? 32 : d.ldb) + g * 8;
+                src[i] = B + n * d.ldb + g * 8;
             }
         }
     };
     auto fetch_next = [&]() {
         unsigned char* slot = smem + (g_fetch & (BG_SLOTS - 1)) * SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < NLD; ++i) bg_load_lds(src[i] + f_kc * (i < BM / 128 ? kstep_a : kstep_b), slot + i * 8192);
+        for (int i = 0; i < NLD; ++i) bg_load_lds(src[i] + f_kc * BG_BK, slot + i * 8192);
         ++g_fetch;
         if (++f_kc == kchunks) {                             // on to the next tile; past the last one the
             unsigned item;                                   // same chunks are re-read into free slots (harmless)
@@ -285,7 +282,6 @@ int bg_launch(const ffk_bgemm_desc& d, hipStream_t st) {
 int ffk_bgemm_big_try(const ffk_bgemm_desc* d, hipStream_t st, int* status) {
     if (d->dtype != FFK_BF16 || d->out_f32 || d->K % BG_BK != 0 || d->K < 3 * BG_BK || d->s_d != 1) return 0;
     if (d->M < 256 || d->N < 64 || d->N % 16 != 0) return 0;
-    if (d->k_blocked && (d->a_kbs % 8 || d->b_kbs % 8 || d->a_kbs < 32L * d->M || d->b_kbs < 32L * d->N)) return 0;
     if (d->xtail && (!d->resid || (reinterpret_cast<uintptr_t>(d->xtail) & 15) != 0)) return 0;
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al16(d->out) || (d->resid && !al16(d->resid)) || (d->bias && !al16(d->bias))) return 0;

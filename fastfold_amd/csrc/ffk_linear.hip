@@ -545,9 +545,6 @@ extern "C" int ffk_fused_linear(const ffk_linear_desc* d, void* stream) {
         int status = FFK_OK;
         if (ffk_linear_ws_try(d, (hipStream_t)stream, &status)) return status;
     }
-    for (int i = 0; i < d->n_tiles; ++i)
-        FFK_REQUIRE(d->tiles[i].s_blk == 0, FFK_ERR_UNSUPPORTED,
-                    "ffk_fused_linear: tile %d: s_blk needs bf16, K = 64 / 128 / 256 and a channel-major tile with inner %% 32 == 0", i);
     FFK_REQUIRE(!d->a2, FFK_ERR_UNSUPPORTED,
                 "ffk_fused_linear: a second operand needs bf16, K = 128, a channel-major first operand and GLU tiles only");
     if (all_c) return ffk_linear_slab_launch(d, (hipStream_t)stream);

@@ -64,7 +64,6 @@ struct WsSlot {
     const T* gate;
     int8_t* xtail;           // tail bytes of resid / out as an extended residual stream, or nullptr
     long s_o, s_i, s_d, gate_ld;
-    long s_blk;              // extra stride per 32 values of the inner index (channel-major tiles, K-blocked operands)
     unsigned inner;
     unsigned gate_rows;      // 0, or the period of the gate's row index
     int ncols_left;          // valid channels from the unit's first channel on
@@ -284,7 +283,7 @@ __device__ __forceinline__ void ws_store_cols_compact(const WsSlot& t, const f32
             *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
     } else if (ok && l32 < t.ncols_left) {
-        T* p = out + (long)hi * t.s_o + lo + (long)(lo >> 5) * t.s_blk + (long)l32 * t.s_d;
+        T* p = out + (long)hi * t.s_o + lo + (long)l32 * t.s_d;
         *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
         *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
     }
@@ -467,7 +466,7 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
             *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
     } else if (ok && l32 < t.ncols_left) {
-        T* p = out + (long)hi * t.s_o + lo + (long)(lo >> 5) * t.s_blk + (long)l32 * t.s_d;
+        T* p = out + (long)hi * t.s_o + lo + (long)l32 * t.s_d;
         *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(&y[0]);
         *reinterpret_cast<u32x4*>(p + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
     }
@@ -614,7 +613,6 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             sp[s].s_o = ts.s_o;
             sp[s].s_i = ts.s_i;
             sp[s].s_d = ts.s_d;
-            sp[s].s_blk = ts.s_blk;
             sp[s].gate_ld = ts.gate_ld;
             sp[s].gate_rows = (unsigned)ts.gate_rows;
             sp[s].inner = (unsigned)ts.inner;
@@ -1011,7 +1009,6 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (t.inner <= 0 || t.ncols <= 0 || !al16(t.out)) return false;
-    if (t.s_blk != 0 && (ws_by_rows(t) || t.kind != FFK_TILE_STRIDED)) return false;
     if (ws_by_rows(t)) {
         if (t.kind == FFK_TILE_STRIDED) {
             if (t.ncols % 8 != 0 || t.s_o % 8 || t.s_i % 8 || t.s_h % 8) return false;
@@ -1026,7 +1023,6 @@ bool ws_tile_ok(const ffk_linear_desc& d, const ffk_tile& t) {
     if (t.resid || t.gate || t.xtail) return false;
     if (t.kind == FFK_TILE_V) return t.inner % 32 == 0 && t.ncols % 32 == 0 && t.s_o % 8 == 0 && t.s_h % 8 == 0;
     if (t.kind != FFK_TILE_STRIDED) return false;
-    if (t.s_blk != 0 && (t.inner % 32 != 0 || t.s_blk % 8 != 0)) return false;
     return d.M % 16 == 0 && t.inner % 16 == 0 && t.s_i == 1 && t.s_o % 8 == 0 && t.s_h % 8 == 0 && t.s_d % 8 == 0;
 }
 

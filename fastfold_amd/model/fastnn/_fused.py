@@ -348,12 +348,6 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
     return dtype == torch.bfloat16 and C == 128 and c == 128 and r % 8 == 0
 
 
-def trimul_k_blocked(dtype, r, C):
-    """The contraction's operands are written K-blocked where the projection kernel that writes them (bf16,
-    weights in registers) and the large-tile contraction kernel (r >= 256) both take that layout."""
-    return dtype == torch.bfloat16 and C in (64, 128) and r % 32 == 0 and r >= 256
-
-
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,
                             dual_pk=None, xtail=None):
     """out = z + sigmoid(Wg LN(z) + bg) * (Wout LN2(p) + b_out),  p[i,j,:] = sum_k a[i,k,:] b[j,k,:]
@@ -365,8 +359,6 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     kpad = round_up(r, vec_of(dt))
     zero = kpad != r
     lr = alloc((2, c, r, kpad), dt, dev, zero)
-    # K-blocked operands [2, c, kpad / 32, r, 32]: the contraction then fetches contiguous KBs (see ffk_bgemm_desc)
-    kblk = trimul_k_blocked(dt, r, C)
     dual = dual_pk is not None and trimul_gate_in_output_stage(dt, r, C, c)
     g = None if dual else torch.empty(M, C, dtype=dt, device=dev)
     tiles = []
@@ -378,8 +370,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
         for t in range(c // 64):
             ti = side * (c // 64) + t
             tiles.append(make_tile(lr.data_ptr() + (side * c + t * 64) * r * kpad * es,
-                                   bias=b_pk.data_ptr() + ti * 128 * es, glu=1, ncols=64, inner=r,
-                                   s_o=32 if kblk else kpad, s_i=1, s_blk=32 * r - 32 if kblk else 0,
+                                   bias=b_pk.data_ptr() + ti * 128 * es, glu=1, ncols=64, inner=r, s_o=kpad, s_i=1,
                                    s_h=32 * r * kpad, s_d=r * kpad, rowmask=mask, m_so=m_so, m_si=m_si))
     for t in range((C + 127) // 128 if not dual else 0):
         kw = dict(inner=r, s_o=C, s_i=r * C) if incoming else dict(inner=M, s_i=C)
@@ -388,7 +379,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     _lib.fused_linear(z, w_pk, tiles, M=M, K=C, a_inner=a_map[0], a_so=a_map[1], a_si=a_map[2], ln=ln1)
     p = torch.empty(c, r, kpad, dtype=dt, device=dev)
     _lib.bgemm_nt(lr[0], lr[1], p, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=c, a_bs=r * kpad, b_bs=r * kpad,
-                  o_bs=r * kpad, s_i=kpad, a_kbs=32 * r if kblk else 0, b_kbs=32 * r if kblk else 0)
+                  o_bs=r * kpad, s_i=kpad)
     del lr
     if dual:
         wd, bd, rowsums = dual_pk

@@ -168,11 +168,7 @@ typedef struct ffk_tile {
     int32_t glu;
     float scale;
     int32_t gate_rows;     /* 0, or the period of the gate's row index (see gate) */
-    int32_t s_blk;         /* 0, or an extra element stride applied once per 32 values of the inner index: the element
-                              offset gains ((m % inner) / 32) * s_blk.  With s_o = 32, s_i = 1 and s_blk = 32 * inner - 32
-                              a channel-major tile is written "K-blocked", [inner / 32][m / inner][32], the operand
-                              layout ffk_bgemm_nt reads with k_blocked.  STRIDED tiles with s_d != 1 (channel-major) and
-                              inner % 32 == 0 only; other uses return FFK_ERR_UNSUPPORTED */
+    int32_t reserved;
     void* xtail;           /* NULL, or the tail bytes of an extended residual stream (see above): int8, addressed with
                               the element offsets of out; requires resid (bf16, STRIDED with s_d == 1).  The epilogue then
                               adds its update to the 24-bit value (resid, xtail), writes the rounded bf16 value to out and
@@ -248,12 +244,6 @@ typedef struct ffk_bgemm_desc {
     int32_t M, N, K, batch;
     int32_t dtype, act, out_f32;
     float scale, div_eps;
-    int32_t k_blocked;     /* 0: operand rows are K-contiguous (lda / ldb).  1: both operands are K-blocked - element (m, k)
-                              of A at a + (k / 32) * a_kbs + m * 32 + k % 32 (B likewise with b_kbs), so that the 32-wide K
-                              chunk of any run of rows is one contiguous block; lda / ldb are ignored.  bf16, K % 32 == 0,
-                              M >= 256 only (the large-tile kernel); otherwise FFK_ERR_UNSUPPORTED */
-    int32_t reserved;
-    int64_t a_kbs, b_kbs;
 } ffk_bgemm_desc;
 
 int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);

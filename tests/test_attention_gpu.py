@@ -149,28 +149,6 @@ def test_bgemm_trimul_contraction(dev, dtype, tol, r):
     assert _rel(_np(out)[:, :, :r].transpose(1, 2, 0), ref) < tol
 
 
-@pytest.mark.parametrize("r,batch", [(256, 3), (320, 9), (1024, 8)])
-def test_bgemm_k_blocked_operands(dev, r, batch):
-    """The same contraction with both operands stored K-blocked ([K / 32][row][32]) gives the same bits as with
-    K-contiguous rows; the small-tile kernel refuses the layout."""
-    from fastfold_amd import _lib
-    g = torch.Generator().manual_seed(r + batch)
-    left = torch.randn(batch, r, r, generator=g).to(dev, torch.bfloat16)
-    right = torch.randn(batch, r, r, generator=g).to(dev, torch.bfloat16)
-    want = torch.empty(batch, r, r, dtype=torch.bfloat16, device=dev)
-    _lib.bgemm_nt(left, right, want, M=r, N=r, K=r, lda=r, ldb=r, batch=batch, a_bs=r * r, b_bs=r * r, o_bs=r * r, s_i=r)
-    lb, rb = (t.view(batch, r, r // 32, 32).permute(0, 2, 1, 3).contiguous() for t in (left, right))
-    got = torch.zeros_like(want)
-    _lib.bgemm_nt(lb, rb, got, M=r, N=r, K=r, lda=r, ldb=r, batch=batch, a_bs=r * r, b_bs=r * r, o_bs=r * r, s_i=r,
-                  a_kbs=32 * r, b_kbs=32 * r)
-    assert torch.equal(got, want)
-    ref = torch.matmul(left.float(), right.float().transpose(1, 2))
-    assert float((got.float() - ref).abs().max() / ref.abs().max()) < 1e-2
-    with pytest.raises(RuntimeError, match="K-blocked"):
-        _lib.bgemm_nt(lb, rb, got, M=64, N=64, K=r, lda=r, ldb=r, batch=batch, a_bs=r * r, b_bs=r * r, o_bs=r * r, s_i=r,
-                      a_kbs=32 * r, b_kbs=32 * r)
-
-
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("s,r", [(24, 10), (128, 9), (50, 33)])
 def test_bgemm_outer_product_and_projection(dev, dtype, tol, s, r):

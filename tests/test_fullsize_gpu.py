@@ -126,27 +126,3 @@ def test_extra_msa_large_masked_invariance_and_column_independence(dev):
         full = col(tm[None], tmm[None])
         part = col(tm[None, :, 32:40].contiguous(), tmm[None, :, 32:40].contiguous())
         assert torch.equal(full[0, :, 32:40], part[0])
-
-
-def test_triangle_multiplication_k_blocked_operands(dev, monkeypatch):
-    """At N_res >= 256 the triangle multiplications hand their operands to the contraction K-blocked; a block run
-    with that layout switched off gives the same bits (outgoing and incoming, with a masked tail)."""
-    import copy
-    from fastfold_amd.model.fastnn import _fused
-    from fastfold_amd.synthetic import bf16_round, synth_inputs, synth_nn_state
-    from fastfold_amd.utils.inject_fastnn import inject_fastnn
-    from oracle.evoformer_ref import OracleModel
-    s, r = 16, 288
-    model = OracleModel(no_blocks=1).eval()
-    sd = synth_nn_state(seed=31, no_blocks=1, fan_in_scaled=True)
-    model.evoformer.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()})
-    fast = inject_fastnn(copy.deepcopy(model)).evoformer.to(dev, torch.bfloat16).eval()
-    m, z, mm, pm = synth_inputs(31, s, r, mask_tail_frac=0.1)
-    args = [torch.from_numpy(bf16_round(a)).to(dev, torch.bfloat16) for a in (m, z, mm, pm)]
-    assert _fused.trimul_k_blocked(torch.bfloat16, r, 128)
-    with torch.no_grad():
-        blocked = fast(*args, chunk_size=None)
-        monkeypatch.setattr(_fused, "trimul_k_blocked", lambda *a: False)
-        plain = fast(*args, chunk_size=None)
-    for a, b in zip(blocked, plain):
-        assert torch.equal(a, b)
