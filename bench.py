@@ -268,6 +268,8 @@ def main():
     ap.add_argument("--blocks", type=int, default=48)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
+    ap.add_argument("--only-micro", action="store_true",
+                    help="run only the operator micro-benchmarks of benchmark configuration 2 (for profiling them)")
     ap.add_argument("--only-feeders", action="store_true",
                     help="time only the extra-MSA and template pair stacks (for profiling them on their own)")
     ap.add_argument("--no-long-sequence", action="store_true",
@@ -287,6 +289,9 @@ def main():
     dev = torch.device("cuda:0")
     wl = WORKLOADS[args.workload]
     s, r = wl["n_seq"], wl["n_res"]
+    if args.only_micro:
+        print(json.dumps({"ops": micro_ops(dev)}))
+        return
     if args.only_feeders:
         print(json.dumps({"feeders": feeder_stacks(dev, r)}))
         return
@@ -305,11 +310,14 @@ def main():
     # HIP events bracket every attention launch of the first timed step only: an event pair costs the
     # stream about 10 us per launch, which the other steps do not have to carry
     rec = _lib.time_kernel("ffk_attention_fwd")
+    others = {name: _lib.time_kernel(name) for name in ("ffk_bgemm_nt", "ffk_transition_fused", "ffk_opm_fused")}
     t0 = time.perf_counter()
     for i in range(args.steps):
         out = step()
         if i == 0:
             _lib.time_kernel("ffk_attention_fwd", enable=False)
+            for name in others:
+                _lib.time_kernel(name, enable=False)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     assert all(bool(torch.isfinite(t.float()).all()) for t in out), "non-finite output"
@@ -331,6 +339,34 @@ def main():
                 "launches": n, "avg_launch_ms": round(ms / max(n, 1), 4),
                 "flops_per_launch_avg": round(flops / max(n, 1) / 1e9, 2)}
 
+    # the other matrix-pipe kernels of the block, timed the same way (HIP events around their launches in the
+    # first timed step): algorithmic flops of the launch / its duration, against the dense bf16 peak
+    def summarise(records, gflop_of):
+        acc = {}
+        for e0, e1, a in records:
+            k = gflop_of(a)
+            if k is None:
+                continue
+            name, gf = k
+            t = acc.setdefault(name, [0, 0.0, gf])
+            t[0] += 1
+            t[1] += e0.elapsed_time(e1)
+        return {name: {"launches": n_, "avg_ms": round(ms_ / n_, 4), "gflop": round(gf, 1),
+                       "TFLOP/s": round(gf / (ms_ / n_), 1), "frac_of_peak": round(gf / (ms_ / n_) / PEAK_BF16_TFLOPS, 3)}
+                for name, (n_, ms_, gf) in acc.items()}
+
+    def bgemm_kind(a):
+        d = a[0]._obj
+        if d.batch == 128 and d.M == r and d.N == r:
+            return "trimul_contraction_bgemm_big", 2.0 * d.batch * d.M * d.N * d.K / 1e9
+        return None
+    kernels = {}
+    kernels.update(summarise(others["ffk_bgemm_nt"], bgemm_kind))
+    kernels.update(summarise(others["ffk_transition_fused"],
+                             lambda a: ("transition_fused_C%d" % a[10], 4.0 * a[9] * a[10] * a[11] / 1e9)))
+    kernels.update(summarise(others["ffk_opm_fused"],
+                             lambda a: ("opm_fused", 2.0 * r * r * (32 * 32 * s + 1024 * 128) / 1e9)))
+
     line = {
         "metric": "Evoformer-block latency, bf16, N_seq=%d, N_res=%d (stack of %d blocks)" % (s, r, args.blocks),
         "value": round(ms_per_step / args.blocks, 4), "unit": "ms/block",
@@ -341,6 +377,7 @@ def main():
                    "stack_tflops": round(block_gflop(s, r) * args.blocks / ms_per_step, 1),
                    "residual_stream": "bf16" if args.plain_residual else "bf16 + int8 tail (24-bit)"},
         "roofline": roofline,
+        "kernels": kernels,
     }
     if args.workload == "cfg4" and not args.no_micro:
         # the same stack at benchmark configuration 3 (N_res = 256), reported beside the headline number
