@@ -5,7 +5,8 @@
 
 for q, k, v ``[b1, b2, h, n, d]``, mask ``[b1, b2, n]`` (0/1, over keys) and bias ``[b1, h, n, n]``.
 The logits are never materialised: the operands are re-tiled into the 32x32 MFMA order and handed to
-the flash attention kernel (``ffk_attention_fwd``).  Forward only, like the reference.  The kernel is
+the flash attention kernel (``ffk_attention_fwd``); the backward pass (``ffk_attention_bwd``) recomputes them the
+same way.  The kernel is
 specialised for the Evoformer's head dim (32); narrower heads (8 and 16, the extra-MSA and template stacks)
 are zero-padded to 32 channels, which changes neither the scores nor the used output channels; the
 reference's Triton kernel also takes 64 and 128 (triton/attention_core.py:143), which no module of the
@@ -58,16 +59,58 @@ def _attention_core_d32(q, k, v, mask, bias, d_scale):
     return out
 
 
+def _attention_core_backward(q, k, v, mask, bias, out, dout, need_dbias):
+    """dq, dk, dv (shapes of q, k, v) and dbias ([b1, h, n, n] or None) through ``ffk_attention_bwd``."""
+    b1, b2, h, n, d = q.shape
+    dt, dev = q.dtype, q.device
+    if d != 32:
+        pad = torch.nn.functional.pad
+        q, k, v = (pad(t, (0, 32 - d)) for t in (q, k, v))
+        out = pad(out.view(b1, b2, n, h, d), (0, 32 - d)).reshape(b1, b2, n, h * 32)
+        dout = pad(dout.view(b1, b2, n, h, d), (0, 32 - d)).reshape(b1, b2, n, h * 32)
+    nt = layouts.n_tiles(n)
+    scale = _lib.LOG2E / math.sqrt(d)
+    dq, dk, dv = (torch.empty(b1, b2, h, n, 32, dtype=dt, device=dev) for _ in range(3))
+    dbias = torch.zeros(b1, h, n, n, dtype=torch.float32, device=dev) if (need_dbias and bias is not None) else None
+    kb = torch.empty(b2, nt * 32, dtype=torch.float32, device=dev)
+    fl = torch.empty(b2, nt, dtype=torch.int32, device=dev)
+    lse = torch.empty(b2 * h * nt * 32, dtype=torch.float32, device=dev)
+    dsum = torch.empty_like(lse)
+    for i in range(b1):
+        mk = mask[i].to(dt).contiguous() if mask is not None else torch.ones(b2, n, dtype=dt, device=dev)
+        _lib.key_bias(kb, fl, mk, B=b2, N=n, mask_sb=n, mask_sn=1)
+        q2 = (q[i].float() * scale).to(dt)                       # the operand the forward kernel saw
+        b2s = (bias[i].float() * _lib.LOG2E).to(dt).contiguous() if bias is not None else None
+        do_ = dout[i].reshape(b2, n, h, 32).permute(0, 2, 1, 3).contiguous()
+        o_ = out[i].reshape(b2, n, h, 32).permute(0, 2, 1, 3).contiguous()
+        _lib.attention_bwd(dq[i], dk[i], dv[i], None if dbias is None else dbias[i], lse, dsum,
+                           layouts.tile_qk(q2), layouts.tile_v(q2), layouts.tile_qk(k[i]), layouts.tile_v(k[i]),
+                           layouts.tile_qk(v[i]), None if b2s is None else layouts.tile_bias(b2s), b2s, kb,
+                           layouts.tile_qk(do_), layouts.tile_v(do_), layouts.tile_qk(o_),
+                           B2=b2, H=h, Nq=n, Nk=n, dq_scale=1.0 / math.sqrt(d), dk_scale=1.0 / _lib.LOG2E)
+    if d != 32:
+        dq, dk, dv = (t[..., :d].contiguous() for t in (dq, dk, dv))
+    return dq, dk, dv, (None if dbias is None else dbias.to(dt))
+
+
 class FusedAttenionCoreFunc(torch.autograd.Function):
-    """Name (including its spelling) as in the reference (attention_core.py:34)."""
+    """Name (including its spelling) as in the reference (attention_core.py:34).  The reference's function has no
+    backward (training goes through matmul / fused_softmax / matmul there, fastnn/ops.py:310-322); this one has:
+    dq, dk, dv and dbias from ``ffk_attention_bwd``, which recomputes the logits tile by tile."""
 
     @staticmethod
     def forward(ctx, q, k, v, mask=None, bias=None):
-        return _attention_core(q, k, v, mask, bias)
+        out = _attention_core(q, k, v, mask, bias)
+        if any(t is not None and t.requires_grad for t in (q, k, v, bias)):
+            ctx.save_for_backward(q, k, v, mask, bias, out)
+        return out
 
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("fused_attention_core is forward-only, as in the reference")
+    def backward(ctx, dout):
+        q, k, v, mask, bias, out = ctx.saved_tensors
+        dq, dk, dv, dbias = _attention_core_backward(q, k, v, mask, bias, out, dout.contiguous(),
+                                                     bias is not None and ctx.needs_input_grad[4])
+        return dq, dk, dv, None, dbias
 
 
 fused_attention_core = FusedAttenionCoreFunc.apply

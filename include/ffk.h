@@ -275,6 +275,31 @@ int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v
                       const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
                       int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int flags, int dtype, void* stream);
 
+/* Backward of ffk_attention_fwd without a gate (the autograd path of fused_attention_core):
+ *     given do = d loss / d out, computes dq, dk, dv and (optionally) dbias of
+ *     out[b2, q, h, :] = softmax_k( q.k / sqrt(d) + bias[h, q, k] + keybias[b2, k] ) . v
+ * with the logits recomputed tile by tile (nothing of size Nq x Nk is stored except dbias).  Operands come in the
+ * 32 x 32 tile orders of ffk_attention_fwd, each in the order(s) its roles need:
+ *   q_qk, q_acc : q scaled by log2(e) / sqrt(d), [B2][H][ceil(Nq/32)][1024] in FFK_TILE_QK and in FFK_TILE_V order
+ *   k_qk, k_acc : k, [B2][H][ceil(Nk/32)][1024] in FFK_TILE_QK and in FFK_TILE_V order
+ *   v_qk        : v in FFK_TILE_QK order
+ *   do_qk, do_acc, o_qk : do and the forward output, as [B2][H][Nq][32] tensors tiled like q
+ *   bias_t      : bias * log2(e) in FFK_TILE_BIAS order, bias_rm : the same values row-major [H][Nq][Nk]; both or neither
+ *   keybias     : as for ffk_attention_fwd
+ *   lse, dsum   : fp32 scratch [B2][H][ceil(Nq/32)*32] (row log-sum-exp in the log2 domain and sum_d do.o; written by
+ *                 the first kernel, read by the second)
+ *   dq : [B2][H][Nq][32], dk, dv : [B2][H][Nk][32] (operand dtype);  dbias : fp32 [H][Nq][Nk], ZEROED by the caller,
+ *                 accumulated over b2 with atomic adds (summation order not fixed), or NULL
+ *   dq_scale = 1 / sqrt(d), dk_scale = 1 / log2(e): undo the factors folded into the q operand.
+ * Rows whose keys are all masked get zero gradients (the forward pass gives them zero output).
+ * Replaces: autograd through the matmul / fused_softmax / matmul chain of SelfAttention.forward
+ * (fastfold/model/fastnn/ops.py:310-322; softmax backward kernels softmax_cuda_kernel.cu:252-334,524-614). */
+int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk,
+                      const void* q_acc, const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
+                      const void* bias_rm, const float* keybias, const void* do_qk, const void* do_acc,
+                      const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, float dq_scale,
+                      float dk_scale, int dtype, void* stream);
+
 /* Pair bias of a biased attention, straight into the operand tiles ffk_attention_fwd reads:
  *     bias_t[h][q/32][k/32][tile(k, q)] = scale * ( LayerNorm(z[q, k, :]; gamma, beta, eps) . w[h, :] )
  * z holds N*N rows of C channels; logical row m = q*N + k lives at (m / a_inner) * a_so + (m % a_inner) * a_si
