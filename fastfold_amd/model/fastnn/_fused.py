@@ -348,6 +348,13 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
     return dtype == torch.bfloat16 and C == 128 and c == 128 and r % 8 == 0
 
 
+# Elements between the channel planes of the triangle multiplication's operands and of its contraction result, beyond the
+# r * kpad the data needs.  With planes exactly 2 MB apart (N_res = 1024, bf16) the 32 lanes of a channel-major store of
+# the projection kernel - one channel each - all land in the same memory channel; 128 bytes of padding spread them
+# (block 6.97 -> 6.885 ms in a same-box A/B at N_res = 1024; 64, 192 and 1088 elements measure the same).
+_TRIMUL_CHAN_PAD = 64
+
+
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,
                             dual_pk=None, xtail=None):
     """out = z + sigmoid(Wg LN(z) + bg) * (Wout LN2(p) + b_out),  p[i,j,:] = sum_k a[i,k,:] b[j,k,:]
@@ -358,7 +365,9 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     M = r * r
     kpad = round_up(r, vec_of(dt))
     zero = kpad != r
-    lr = alloc((2, c, r, kpad), dt, dev, zero)
+    # channel planes of the operands and of the contraction result are cs elements apart (_TRIMUL_CHAN_PAD beyond r * kpad)
+    cs = r * kpad + _TRIMUL_CHAN_PAD
+    lr = alloc((2, c, cs), dt, dev, zero)
     dual = dual_pk is not None and trimul_gate_in_output_stage(dt, r, C, c)
     g = None if dual else torch.empty(M, C, dtype=dt, device=dev)
     tiles = []
@@ -369,17 +378,17 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     for side in range(2):
         for t in range(c // 64):
             ti = side * (c // 64) + t
-            tiles.append(make_tile(lr.data_ptr() + (side * c + t * 64) * r * kpad * es,
+            tiles.append(make_tile(lr.data_ptr() + (side * c + t * 64) * cs * es,
                                    bias=b_pk.data_ptr() + ti * 128 * es, glu=1, ncols=64, inner=r, s_o=kpad, s_i=1,
-                                   s_h=32 * r * kpad, s_d=r * kpad, rowmask=mask, m_so=m_so, m_si=m_si))
+                                   s_h=32 * cs, s_d=cs, rowmask=mask, m_so=m_so, m_si=m_si))
     for t in range((C + 127) // 128 if not dual else 0):
         kw = dict(inner=r, s_o=C, s_i=r * C) if incoming else dict(inner=M, s_i=C)
         tiles.append(make_tile(g.data_ptr() + t * 128 * es, bias=b_pk.data_ptr() + (n_glu + t) * 128 * es,
                                act=FFK_ACT_SIGMOID, ncols=min(128, C - t * 128), **kw))
     _lib.fused_linear(z, w_pk, tiles, M=M, K=C, a_inner=a_map[0], a_so=a_map[1], a_si=a_map[2], ln=ln1)
-    p = torch.empty(c, r, kpad, dtype=dt, device=dev)
-    _lib.bgemm_nt(lr[0], lr[1], p, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=c, a_bs=r * kpad, b_bs=r * kpad,
-                  o_bs=r * kpad, s_i=kpad)
+    p = torch.empty(c, cs, dtype=dt, device=dev)
+    _lib.bgemm_nt(lr[0], lr[1], p, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=c, a_bs=cs, b_bs=cs,
+                  o_bs=cs, s_i=kpad)
     del lr
     if dual:
         wd, bd, rowsums = dual_pk
@@ -387,7 +396,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
                            resid=z.data_ptr() + t * 64 * es, xtail=xtail_ptr(xtail, t * 64), inner=M, s_i=C)
                  for t in range(C // 64)]
         # both LayerNorms (of p and of z) are folded into the packed weights: no normalisation pass over either
-        _lib.fused_linear(p, wd, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
+        _lib.fused_linear(p, wd, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=cs,
                           ln_rowsums=rowsums, a2=z, a2_inner=M, a2_si=C)
         return out
     tiles = []
@@ -395,7 +404,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
         tiles.append(make_tile(out.data_ptr() + t * 128 * es, bias=out_bias_pk.data_ptr() + t * 128 * es,
                                gate=g.data_ptr() + t * 128 * es, gate_ld=C, resid=z.data_ptr() + t * 128 * es,
                                xtail=xtail_ptr(xtail, t * 128), inner=M, s_i=C, ncols=min(128, C - t * 128)))
-    _lib.fused_linear(p, wout_pk, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=r * kpad,
+    _lib.fused_linear(p, wout_pk, tiles, M=M, K=c, a_inner=r, a_so=kpad, a_si=1, a_chanmajor=True, a_cs=cs,
                       ln=ln2)
     return out
 

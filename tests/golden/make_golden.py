@@ -8,6 +8,7 @@ and inputs.  Run only in the build container, where /root/reference is mounted:
     python tests/golden/make_golden.py template   # template pair stack
     python tests/golden/make_golden.py pointwise  # template point-wise attention
     python tests/golden/make_golden.py cfg4       # one Evoformer block at N_seq=128, N_res=1024 (sampled outputs)
+    python tests/golden/make_golden.py cfg4_deep 48   # the 48-block stack at that shape (about an hour of CPU)
 
 The fixture pins what closed forms cannot: the composition of a block (order of the
 sub-updates, residual placement, OPM reading the updated MSA), the q/k/v and left/right
@@ -201,8 +202,48 @@ def main_cfg4():
     print("wrote", os.path.join(HERE, "evoformer_cfg4_nn_golden.npz"))
 
 
+def main_cfg4_deep(no_blocks=48):
+    """The headline acceptance: the 48-block stack at N_seq = 128, N_res = 1024, last 5 % of the residues masked, the
+    benchmark's N(0, 0.02^2) weights, inputs rounded to bf16.  The reference runs in fp32 with chunk_size = 64 (about
+    an hour on eight host cores); a sample of the outputs (random un-masked sequences / residues) and the norms of the
+    full outputs and of the accumulated update are stored."""
+    import time
+    from fastfold.model.nn.evoformer import EvoformerStack  # the reference
+    from fastfold_amd.synthetic import bf16_round
+
+    s, r, tail, seed = 128, 1024, 0.05, 73
+    nv = r - int(round(tail * r))
+    stack = EvoformerStack(c_m=256, c_z=128, c_hidden_msa_att=32, c_hidden_opm=32, c_hidden_mul=128,
+                           c_hidden_pair_att=32, c_s=384, no_heads_msa=8, no_heads_pair=4, no_blocks=no_blocks,
+                           transition_n=4, msa_dropout=0.15, pair_dropout=0.25, blocks_per_ckpt=1,
+                           inf=1e9, eps=1e-8).eval()
+    sd = synth_nn_state(seed=seed, no_blocks=no_blocks, fan_in_scaled=False)
+    stack.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+    m, z, msa_mask, pair_mask = synth_inputs(seed, s, r, mask_tail_frac=tail)
+    m, z = bf16_round(m), bf16_round(z)
+    t0 = time.time()
+    with torch.no_grad():
+        mo, zo, so = stack(torch.from_numpy(m), torch.from_numpy(z), torch.from_numpy(msa_mask),
+                           torch.from_numpy(pair_mask), chunk_size=64, _mask_trans=False)
+    print("reference: %d blocks in %.0f s" % (no_blocks, time.time() - t0), flush=True)
+    S, I, J = cfg4_sample_indices(seed, s, nv)
+    mo, zo, so = mo.numpy(), zo.numpy(), so.numpy()
+    name = "cfg4_deep%d" % no_blocks
+    out = {name + ".S": S, name + ".I": I, name + ".J": J,
+           name + ".m": mo[S][:, J], name + ".z": zo[I][:, J], name + ".s": so[J],
+           name + ".cfg": np.array([seed, no_blocks, s, r, int(round(tail * 100)), 0], dtype=np.int64),
+           # norms over the un-masked region: of the outputs and of the accumulated update (out - in)
+           name + ".norms": np.array([np.linalg.norm(mo[:, :nv]), np.linalg.norm(zo[:nv, :nv]), np.linalg.norm(so[:nv]),
+                                      np.linalg.norm((mo - m)[:, :nv]), np.linalg.norm((zo - z)[:nv, :nv])], dtype=np.float64)}
+    path = os.path.join(HERE, "evoformer_%s_nn_golden.npz" % name)
+    np.savez_compressed(path, **out)
+    print("wrote", path)
+
+
 if __name__ == "__main__":
-    if "cfg4" in sys.argv[1:]:
+    if "cfg4_deep" in sys.argv[1:]:
+        main_cfg4_deep(int(sys.argv[sys.argv.index("cfg4_deep") + 1]) if len(sys.argv) > sys.argv.index("cfg4_deep") + 1 else 48)
+    elif "cfg4" in sys.argv[1:]:
         main_cfg4()
     elif "pointwise" in sys.argv[1:]:
         main_pointwise()

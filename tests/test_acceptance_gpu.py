@@ -3,7 +3,7 @@ vectors; tolerance of the bf16 mode: relative L2 <= 2e-2 on the MSA, pair and si
 
 * the 48-block stack at N_seq = 128, N_res = 256 against the fp32 CPU oracle called with ``_mask_trans=False``, on
   the outputs and on the accumulated update (out - in), so that a vanishing update cannot hide in the residual;
-* one block at N_seq = 128, N_res = 1024 (last 5 % of the residues masked) against a sample of the outputs of the
+* the 48-block stack and one block at N_seq = 128, N_res = 1024 (last 5 % of the residues masked) against a sample of the outputs of the
   reference's own ``fastfold.model.nn.evoformer.EvoformerStack`` (``tests/golden/make_golden.py cfg4``);
 * one block at N_seq = 64, N_res = 4096 with ``set_chunk_size(64)`` through ``.inplace``: properties the size does
   not change, and the peak memory;
@@ -81,6 +81,42 @@ def test_deep_stack_bf16_against_fp32_oracle(dev, nb, fan_in_scaled):
     if fan_in_scaled:
         assert size_m > 0.5 and size_z > 0.5
     assert um <= 4e-2 and uz <= 4e-2
+
+
+# ------------------------------------------------------------------ 48 blocks, N_res = 1024 ----
+CFG4_DEEP_GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "evoformer_cfg4_deep48_nn_golden.npz")
+
+
+def test_cfg4_deep_stack_against_reference_sample(dev):
+    """The headline acceptance: the 48-block bf16 stack at N_seq = 128, N_res = 1024 (last 5 % of the residues masked,
+    N(0, 0.02^2) weights) against the stored sample of the fp32 outputs of the reference's own ``nn.EvoformerStack``
+    (``tests/golden/make_golden.py cfg4_deep 48``): relative L2 <= 2e-2 on the MSA, pair and single outputs, and on the
+    accumulated update (out - in), whose size relative to the input is checked against the reference's too."""
+    g = np.load(CFG4_DEEP_GOLDEN)
+    case = "cfg4_deep48"
+    seed, nb, s, r, tail, fis = (int(v) for v in g[case + ".cfg"])
+    S, I, J = g[case + ".S"], g[case + ".I"], g[case + ".J"]
+    nv = r - int(round(tail / 100.0 * r))
+    _, fast = _models(seed, nb, dev, fan_in_scaled=bool(fis))
+    m, z, mm, pm = synth_inputs(seed, s, r, mask_tail_frac=tail / 100.0)
+    m, z = bf16_round(m), bf16_round(z)
+    with torch.no_grad():
+        gm, gz, gs = fast.evoformer(_t(m, dev), _t(z, dev), _t(mm, dev), _t(pm, dev), chunk_size=None)
+    gm, gz, gs = _f(gm), _f(gz), _f(gs)
+    assert np.isfinite(gm).all() and np.isfinite(gz).all() and np.isfinite(gs).all()
+    # size of the accumulated update over the whole un-masked region, against the reference's
+    rn = g[case + ".norms"]
+    um, uz = float(np.linalg.norm((gm - m)[:, :nv])), float(np.linalg.norm((gz - z)[:nv, :nv]))
+    assert abs(um / rn[3] - 1) < 2e-2 and abs(uz / rn[4] - 1) < 2e-2
+    m0, z0 = m[S][:, J], z[I][:, J]
+    gm, gz, gs = gm[S][:, J], gz[I][:, J], gs[J]
+    rm, rz, rs = g[case + ".m"], g[case + ".z"], g[case + ".s"]
+    em, ez, es = _rel_l2(gm, rm), _rel_l2(gz, rz), _rel_l2(gs, rs)
+    dm, dz = _rel_l2(gm - m0, rm - m0), _rel_l2(gz - z0, rz - z0)
+    print("\n%s: rel-L2 m %.3e z %.3e s %.3e | accumulated update: m %.3e z %.3e (|update| / |input|: m %.2f z %.2f)"
+          % (case, em, ez, es, dm, dz, rn[3] / np.linalg.norm(m[:, :nv]), rn[4] / np.linalg.norm(z[:nv, :nv])))
+    assert em <= 2e-2 and ez <= 2e-2 and es <= 2e-2
+    assert dm <= 4e-2 and dz <= 4e-2
 
 
 # ------------------------------------------------------------------ one block, N_res = 1024 ----
