@@ -196,11 +196,14 @@ def test_block_interface_padding_and_chaining(dev):
     assert isinstance(fast.blocks[0], Evoformer)
 
 
+@pytest.mark.parametrize("extended", [True, False])
 @pytest.mark.parametrize("nb,s,r,tail", [(4, 24, 72, 0.1)])
-def test_stack_bf16_rel_l2(dev, nb, s, r, tail):
-    """bf16 stack vs fp32 oracle: relative L2 <= 2e-2 on m and z (north star), O(1) updates."""
+def test_stack_bf16_rel_l2(dev, nb, s, r, tail, extended):
+    """bf16 stack vs fp32 oracle: relative L2 <= 2e-2 on m and z (north star), O(1) updates; with the extended
+    residual stream (the default) and with the reference's plain bf16 stream (the switch bench.py --plain-residual uses)."""
     model = _oracle(31, nb)
     fast = _fast(model, dev, torch.bfloat16)
+    fast.extended_residual = extended
     m, z, mm, pm = synth_inputs(31, s, r, mask_tail_frac=tail)
     mb, zb = (_f(_t(x, dev, torch.bfloat16)) for x in (m, z))
     with torch.no_grad():
