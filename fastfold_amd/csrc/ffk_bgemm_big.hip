@@ -287,6 +287,9 @@ int ffk_bgemm_big_try(const ffk_bgemm_desc* d, hipStream_t st, int* status) {
     if (!al16(d->out) || (d->resid && !al16(d->resid)) || (d->bias && !al16(d->bias))) return 0;
     if (d->s_o % 8 || d->s_i % 8 || d->s_h % 8 || d->o_bs % 8) return 0;
     if (d->s_h != 32 && d->N % 32 != 0) return 0;            // 32-column blocks must be whole when they are strided
-    *status = d->N > 128 ? bg_launch<128>(*d, st) : bg_launch<64>(*d, st);
+    // 256 x 256 tiles, unless they would leave CUs without a tile while 256 x 128 tiles would not (small batched launches)
+    const long wide_tiles = (long)ffk_cdiv(d->M, 256) * ffk_cdiv(d->N, 256) * d->batch;
+    const bool narrow = d->N <= 128 || (wide_tiles < 256 && d->N % 128 == 0);
+    *status = narrow ? bg_launch<64>(*d, st) : bg_launch<128>(*d, st);
     return 1;
 }

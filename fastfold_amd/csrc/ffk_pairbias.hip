@@ -3,7 +3,8 @@
 // written directly in the keys x queries operand tiles the attention kernel consumes.
 //
 // The op is a skinny projection (C = 128 or 64 channels -> H <= 8 heads) and purely HBM-bound (one read of
-// z).  One workgroup owns a 32 x 32 block of (q, k) and walks it in four 16 x 16 quarter blocks: the
+// z).  One workgroup owns a 32 x 32 block of (q, k) and walks it in four 16 x 16 quarter blocks (launches of fewer
+// than 512 blocks give every quarter a workgroup of its own): the
 // 256 rows of a quarter are fetched with 16 lanes per row (coalesced 256-byte rows, 16 loads in
 // flight per thread, the next quarter's loads issued before this one is finished) into LDS.  The
 // LayerNorm is folded into the projection,
@@ -68,8 +69,11 @@ __global__ __launch_bounds__(PB_THREADS) void pair_bias_kernel(bf16_t* __restric
             buf[i] = ld16(z + (long)hi * a_so + (long)lo * a_si + c8 * 8);
         }
     };
-    fetch(0);
-    for (int quarter = 0; quarter < 4; ++quarter) {
+    // quarters of the block this workgroup walks: all four, or one of them (gridDim.z = 4: launches of few blocks,
+    // where a workgroup per block would leave most CUs idle)
+    const int nquarters = 4 / (int)gridDim.z, q_first = (int)blockIdx.z * nquarters, q_last = q_first + nquarters - 1;
+    fetch(q_first);
+    for (int quarter = q_first; quarter <= q_last; ++quarter) {
         __syncthreads();                             // previous quarter's rows are consumed
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
@@ -85,7 +89,7 @@ __global__ __launch_bounds__(PB_THREADS) void pair_bias_kernel(bf16_t* __restric
             if (c8 == 0) s_sq[r] = q2;
         }
         __syncthreads();
-        if (quarter < 3) fetch(quarter + 1);         // in flight while this quarter is finished below
+        if (quarter < q_last) fetch(quarter + 1);    // in flight while this quarter is finished below
 
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -166,7 +170,7 @@ int pair_bias_run(const char* who, void* bias_t, const void* z, const void* gamm
         static FfkLdsReservation lds_reserved;                                                                          \
         const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)pair_bias_kernel<CC>, smem, who);                 \
         if (rc_lds != FFK_OK) return rc_lds;                                                                            \
-        pair_bias_kernel<CC><<<dim3(T, T), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wop, c01, (int)N, \
+        pair_bias_kernel<CC><<<dim3(T, T, T * T < 512 ? 4 : 1), PB_THREADS, smem, st>>>((bf16_t*)bias_t, (const bf16_t*)z, wop, c01, (int)N, \
                                                                    (int)H, (int)a_inner, a_so, a_si, scale, eps);       \
     }
     if (C == 128) PB_LAUNCH(128) else PB_LAUNCH(64)
