@@ -182,10 +182,18 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
 #pragma unroll
             for (int ks = 0; ks < G::KS1; ++ks)
                 MM::mma(h, *reinterpret_cast<const bf16x8*>(wa + ht * 32 * (TR_C * 2) + w1off[ks & 7] + (ks >> 3) * 256), xf[ks]);
+            // relu after the rounding, on the packed bf16 bit patterns: a negative bf16 is a negative 16-bit integer, so
+            // one packed integer max per pair replaces one clamp per value (rounding is monotonic: same bits)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < 2; ++j) {
+                bf16x8 r;
 #pragma unroll
-                for (int t = 0; t < 8; ++t) hf[ht][j][t] = (T)relu_f(h[8 * j + t]);
+                for (int t = 0; t < 8; ++t) r[t] = (T)h[8 * j + t];
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const s16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+                const s16x8 c = __builtin_elementwise_max(__builtin_bit_cast(s16x8, r), zero);
+                hf[ht][j] = __builtin_bit_cast(bf16x8, c);
+            }
         }
 #pragma unroll
         for (int ks = 0; ks < G::KS2; ++ks)
