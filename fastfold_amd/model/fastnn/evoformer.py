@@ -17,7 +17,7 @@ import torch.nn.functional as F
 
 from . import _fused as F_
 from .msa import MSACore
-from .ops import Linear, OutProductMean
+from .ops import Linear, OutProductMean, _needs_grad
 from .triangle import PairCore
 
 
@@ -62,6 +62,18 @@ class Evoformer(nn.Module):
         self.pair.inplace([z_new], pair_mask, zt)
         return m, z_new
 
+    def _core_train(self, m, z, msa_mask, pair_mask):
+        """The differentiable block (evoformer.py:64-76) on the un-padded tensors: every update is out of place and
+        made of operators with a backward pass."""
+        F_.check_nonempty("Evoformer", m, z)
+        if self.is_multimer:
+            z_ori = self.communication(m, msa_mask, z)
+            z = self.pair(z_ori, pair_mask)
+            return self.msa(m, z_ori, msa_mask), z
+        m = self.msa(m, z, msa_mask)
+        z = self.communication(m, msa_mask, z)
+        return m, self.pair(z, pair_mask)
+
     def _enter(self, m, z, r):
         if self.first_block:
             return m.unsqueeze(0).contiguous(), z.unsqueeze(0).contiguous()
@@ -83,6 +95,12 @@ class Evoformer(nn.Module):
         (evoformer.py:36-37): chunking is the process-global ``set_chunk_size`` and transitions
         are never masked."""
         r = pair_mask.size(-1)
+        if _needs_grad(self, m, z):
+            if self.first_block:
+                m, z = m.unsqueeze(0), z.unsqueeze(0)
+            else:
+                m, z = m[:, :, :r, :], z[:, :r, :r, :]
+            return self._leave(*self._core_train(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)))
         m, z = self._enter(m, z, r)
         m, z = self._core(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0), inplace=not self.first_block)
         return self._leave(m, z)
@@ -138,6 +156,28 @@ class EvoformerStack(nn.Module):
                 mm, zz = b._core(mm.contiguous(), zz.contiguous(), mk, pk, inplace=(inplace_first or i > 0), tails=tails)
         return mm.squeeze(0), zz.squeeze(0)
 
+    def _run_train(self, m, z, msa_mask, pair_mask):
+        """The differentiable stack: plain residual stream, blocks re-run in the backward pass in groups of
+        ``blocks_per_ckpt`` while the module is in training mode (evoformer.py:262-266)."""
+        from torch.utils.checkpoint import checkpoint
+        mm, zz = m.unsqueeze(0), z.unsqueeze(0)
+        mk, pk = msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)
+        blocks = list(self.blocks)
+        per = self.blocks_per_ckpt if (self.training and self.blocks_per_ckpt) else None
+
+        def run(group, a, b):
+            for blk in group:
+                if self.clear_cache_between_blocks:
+                    torch.cuda.empty_cache()
+                a, b = blk._core_train(a, b, mk, pk)
+            return a, b
+        if per is None:
+            mm, zz = run(blocks, mm, zz)
+        else:
+            for i in range(0, len(blocks), per):
+                mm, zz = checkpoint(run, blocks[i:i + per], mm, zz, use_reentrant=False)
+        return mm.squeeze(0), zz.squeeze(0)
+
     def forward(self, m: torch.Tensor, z: torch.Tensor, msa_mask: torch.Tensor, pair_mask: torch.Tensor,
                 chunk_size: int = None, _mask_trans: bool = True
                 ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
@@ -145,6 +185,9 @@ class EvoformerStack(nn.Module):
         m [N_seq, N_res, C_m], z [N_res, N_res, C_z], msa_mask [N_seq, N_res], pair_mask [N_res, N_res]
         -> (m, z, s [N_res, C_s]).  Inputs are left untouched.
         """
+        if _needs_grad(self, m, z):
+            m, z = self._run_train(m, z, msa_mask, pair_mask)
+            return m, z, self.linear(m[..., 0, :, :])
         m, z = self._run(m, z, msa_mask, pair_mask, inplace_first=False)
         s = self.linear(m[..., 0, :, :])
         return m, z, s

@@ -11,7 +11,7 @@ import torch.nn.functional as F
 from fastfold_amd.model.fastnn.kernel import LayerNorm
 from . import _fused as F_
 from .ops import (ChunkMSAColumnGlobalAttention, ChunkTransition, OutProductMean, SelfAttention, Transition,
-                  _PackMixin, _budget, _check_tail, _ln_pair, _mask_like, _no_grad_guard)
+                  _PackMixin, _budget, _check_tail, _ln_pair, _mask_like, _needs_grad, _no_grad_guard)
 from .triangle import PairCore
 
 
@@ -66,7 +66,18 @@ class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
                      xtail=_check_tail(xtail, M_raw))
         return out
 
+    def _train(self, M_raw, Z, M_mask):
+        """msa.py:60-74, operator by operator."""
+        from .kernel import bias_dropout_add
+        M = self.layernormM(M_raw)
+        b = F.linear(self.layernormZ(Z), self.linear_b_weights.to(Z.dtype))
+        M = self.attention(M, M_mask, (b, None))
+        dropout_mask = torch.ones_like(M[:, 0:1, :, :])
+        return bias_dropout_add(M, self.out_bias, dropout_mask, M_raw, prob=self.p_drop, training=self.training)
+
     def forward(self, M_raw, Z, M_mask):
+        if _needs_grad(self, M_raw, Z):
+            return self._train(M_raw, Z, M_mask)
         M_raw = M_raw.contiguous()
         return self._run(M_raw, Z, M_mask, torch.empty_like(M_raw))
 
@@ -111,7 +122,15 @@ class MSAColumnAttention(nn.Module, _PackMixin):
                      xtail=_check_tail(xtail, M_raw))
         return out
 
+    def _train(self, M_raw, M_mask):
+        """msa.py:92-104, operator by operator."""
+        M = self.layernormM(M_raw.transpose(-2, -3))
+        M = self.attention(M, M_mask.transpose(-1, -2))
+        return M_raw + M.transpose(-2, -3)
+
     def forward(self, M_raw, M_mask):
+        if _needs_grad(self, M_raw):
+            return self._train(M_raw, M_mask)
         M_raw = M_raw.contiguous()
         return self._run(M_raw, M_mask, torch.empty_like(M_raw))
 
@@ -129,6 +148,12 @@ class MSACore(nn.Module):
         (the input tensor is left untouched; the two later updates run in place on the copy).
         ``xtail``: int8 tail of the *new* node tensor as an extended residual stream (zero on entry when the input
         is a plain bf16 tensor)."""
+        if _needs_grad(self, node, pair):
+            if xtail is not None:
+                raise RuntimeError("MSACore: the extended residual stream is forward-only")
+            node = self.MSARowAttentionWithPairBias(node, pair, node_mask)
+            node = self.MSAColumnAttention(node, node_mask)
+            return self.MSATransition(node)
         node = node.contiguous()
         out = torch.empty_like(node)
         self.MSARowAttentionWithPairBias._run(node, pair, node_mask, out, xtail)

@@ -74,6 +74,18 @@ def _no_grad_guard(module, *tensors):
             % type(module).__name__)
 
 
+def _needs_grad(module, *tensors):
+    """True when autograd has to see this call: gradients are enabled and an input or a parameter of ``module``
+    requires one.  Such calls take the differentiable composition (``_train`` methods: the reference's own sequence
+    of operators - HIP LayerNorm / attention-core / elementwise kernels with backward passes, library GEMMs for the
+    ``Linear`` layers); everything else takes the fused forward-only launches."""
+    if not torch.is_grad_enabled():
+        return False
+    if any(t is not None and t.requires_grad for t in tensors):
+        return True
+    return any(p.requires_grad for p in module.parameters())
+
+
 def _check_tail(xtail, x):
     """The int8 tail of ``x`` as an extended residual stream (see include/ffk.h): same shape, bf16 stream only."""
     if xtail is None:
@@ -154,7 +166,11 @@ class Linear(nn.Linear, _PackMixin):
 
     def forward(self, input, act=_lib.FFK_ACT_NONE):
         F_.check_cuda(input)
-        _no_grad_guard(self, input)
+        if _needs_grad(self, input):
+            if act != _lib.FFK_ACT_NONE:
+                raise NotImplementedError("Linear: fused activations are forward-only")
+            return torch.nn.functional.linear(input, self.weight.to(input.dtype),
+                                              self.bias.to(input.dtype) if self.use_bias else None)
         w, b = self._pk(input.dtype, input.device)
         x2 = input.reshape(-1, self.in_features)
         kp = self._kpad()
@@ -190,7 +206,14 @@ class Transition(nn.Module, _PackMixin):
                       hidden=hidden, budget=_budget(), xtail=_check_tail(xtail, src))
         return out
 
+    def _train(self, src):
+        """ops.py:79-82, operator by operator."""
+        x = self.norm(src)
+        return src + self.linear2(torch.relu(self.linear1(x)))
+
     def forward(self, src):
+        if _needs_grad(self, src):
+            return self._train(src)
         src = src.contiguous()
         return self._run(src, torch.empty_like(src))
 
@@ -242,7 +265,20 @@ class OutProductMean(nn.Module, _PackMixin):
                               budget=_budget(), xtail=_check_tail(xtail, Z_raw))
         return out
 
+    def _train(self, M, M_mask, Z_raw):
+        """ops.py:141-173 (the un-chunked branch); the normaliser is kept in fp32."""
+        M = self.layernormM(M)
+        mask = M_mask.unsqueeze(-1).to(M.dtype)
+        left = mask * self.linear_a(M)
+        right = mask * self.linear_b(M)
+        norm = torch.einsum('bsid,bsjd->bijd', mask.float(), mask.float()) + 1e-3
+        out = torch.einsum('bsid,bsje->bijde', left, right).flatten(-2)
+        out = self.o_linear(out)
+        return (out.float() / norm).to(Z_raw.dtype) + Z_raw
+
     def forward(self, M, M_mask, Z_raw):
+        if _needs_grad(self, M, Z_raw):
+            return self._train(M, M_mask, Z_raw)
         Z_raw = Z_raw.contiguous()
         return self._run(M, M_mask, Z_raw, torch.empty_like(Z_raw))
 
@@ -304,6 +340,25 @@ class SelfAttention(nn.Module, _PackMixin):
                     F_.pack_rows([_pad_heads(self.o_linear.weight, H, c, 1)], dtype, device))
         return self._packed(key, params, build)
 
+    def _train(self, in_data, mask, nonbatched_bias=None):
+        """ops.py:289-331 with the logits / softmax / weighted average of :310-322 inside the attention-core kernels
+        (forward and backward recompute the logits tile by tile; they are never stored)."""
+        from .kernel import bias_sigmod_ele, fused_attention_core
+        bias = None
+        if nonbatched_bias is not None:
+            bias = nonbatched_bias[0]
+            if not (isinstance(nonbatched_bias[-1], int) and nonbatched_bias[-1] == -1):
+                bias = bias.permute(0, 3, 1, 2)                 # 'b q k h -> b h q k'
+            bias = bias.contiguous()
+        qkv = self.to_qkv(in_data).chunk(3, dim=-1)
+        q, k, v = (t.unflatten(-1, (self.n_head, self.c)).transpose(-2, -3).contiguous() for t in qkv)
+        if mask is not None:
+            mask = mask.to(in_data.dtype).contiguous()
+        weighted_avg = fused_attention_core(q, k, v, mask, bias)          # [b1, b2, n, h * d]
+        if self.gating:
+            weighted_avg = bias_sigmod_ele(self.gating_linear(in_data), self.gating_bias, weighted_avg)
+        return self.o_linear(weighted_avg)
+
     def forward(self, in_data, mask, nonbatched_bias=None):
         """
         :param in_data: [batch_size1, batch_size2, len_qkv, qkv_dim]
@@ -312,7 +367,8 @@ class SelfAttention(nn.Module, _PackMixin):
                                 (bias [batch_size1, n_head, len_q, len_kv], -1)
         """
         F_.check_cuda(in_data, mask)
-        _no_grad_guard(self, in_data)
+        if _needs_grad(self, in_data, None if nonbatched_bias is None else nonbatched_bias[0]):
+            return self._train(in_data, mask, nonbatched_bias)
         dt, dev = in_data.dtype, in_data.device
         self._check(dt)
         if in_data.dim() != 4 or in_data.shape[0] != 1:
@@ -482,7 +538,26 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
                                    mask=_mask_like(Z_mask, Z_raw), dual_pk=dual, xtail=_check_tail(xtail, Z_raw))
         return out
 
+    def _train(self, Z_raw, Z_mask):
+        """triangle.py:41-75 / :97-131, operator by operator."""
+        from .kernel import bias_ele_dropout_residual
+        Z = self.layernorm1(Z_raw)
+        lr = Z_mask.unsqueeze(-1).to(Z.dtype) * self.left_right_projection(Z)
+        lr = lr * torch.sigmoid(self.left_right_gate(Z))
+        left, right = lr.chunk(2, dim=-1)
+        g = torch.sigmoid(self.output_gate(Z))
+        if self._incoming:      # p[c, i, j] = sum_k left[k, i, c] right[k, j, c]
+            p = torch.matmul(permute_final_dims(left, (2, 1, 0)), permute_final_dims(right, (2, 0, 1)))
+        else:                   # p[c, i, j] = sum_k left[i, k, c] right[j, k, c]
+            p = torch.matmul(permute_final_dims(left, (2, 0, 1)), permute_final_dims(right, (2, 1, 0)))
+        ab = self.output_projection(self.layernorm2(permute_final_dims(p, (1, 2, 0))))
+        dropout_mask = torch.ones_like(Z[:, 0:1, :, :])
+        return bias_ele_dropout_residual(ab, self.output_bias, g, dropout_mask, Z_raw, prob=self.p_drop,
+                                         training=self.training)
+
     def forward(self, Z_raw, Z_mask):
+        if _needs_grad(self, Z_raw):
+            return self._train(Z_raw, Z_mask)
         Z_raw = Z_raw.contiguous()
         return self._run(Z_raw, Z_mask, torch.empty_like(Z_raw))
 
@@ -543,7 +618,25 @@ class _TriangleAttention(nn.Module, _PackMixin):
                      head_dim=self.c, budget=_budget(), xtail=_check_tail(xtail, Z_raw))
         return out
 
+    def _train(self, Z_raw, Z_mask):
+        """triangle.py:156-173 (starting node) / :202-222 (ending node: the same on the transposed pair tensor, with
+        the dropout mask shared along the other axis)."""
+        from .kernel import bias_dropout_add
+        Z = Z_raw.transpose(-2, -3) if self._ending else Z_raw
+        mask = Z_mask.transpose(-1, -2) if self._ending else Z_mask
+        Z = self.layernorm1(Z)
+        b = self.linear_b(Z)
+        Z = self.attention(Z, mask, (b, None))
+        if self._ending:
+            Z = Z.transpose(-2, -3)
+            dropout_mask = torch.ones_like(Z[:, :, 0:1, :])
+        else:
+            dropout_mask = torch.ones_like(Z[:, 0:1, :, :])
+        return bias_dropout_add(Z, self.out_bias, dropout_mask, Z_raw, prob=self.p_drop, training=self.training)
+
     def forward(self, Z_raw, Z_mask):
+        if _needs_grad(self, Z_raw):
+            return self._train(Z_raw, Z_mask)
         Z_raw = Z_raw.contiguous()
         return self._run(Z_raw, Z_mask, torch.empty_like(Z_raw))
 

@@ -3,7 +3,7 @@ import torch
 import torch.nn as nn
 
 from .ops import (AsyncChunkTriangleMultiplicationIncoming, AsyncChunkTriangleMultiplicationOutgoing,
-                  ChunkTransition, ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode)
+                  ChunkTransition, ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode, _needs_grad)
 
 
 class PairCore(nn.Module):
@@ -25,6 +25,14 @@ class PairCore(nn.Module):
     def forward(self, pair, pair_mask, xtail=None):
         """pair [1, r, r, d_pair], pair_mask [1, r, r] -> new pair (input untouched).  ``xtail``: int8 tail of the
         pair tensor as an extended residual stream (read with the input, rewritten for the output)."""
+        if _needs_grad(self, pair):
+            if xtail is not None:
+                raise RuntimeError("PairCore: the extended residual stream is forward-only")
+            pair = self.TriangleMultiplicationOutgoing(pair, pair_mask)
+            pair = self.TriangleMultiplicationIncoming(pair, pair_mask)
+            pair = self.TriangleAttentionStartingNode(pair, pair_mask)
+            pair = self.TriangleAttentionEndingNode(pair, pair_mask)
+            return self.PairTransition(pair)
         pair = pair.contiguous()
         out = torch.empty_like(pair)
         self.TriangleMultiplicationOutgoing._run(pair, pair_mask, out, xtail)

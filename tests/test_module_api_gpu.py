@@ -223,16 +223,23 @@ def test_extra_msa_stack_default_masks(dev):
 
 
 def test_forward_only_guard(dev):
-    """The HIP path has no backward: a call whose input asks for gradients raises instead of returning a
-    tensor cut off from the graph."""
-    from fastfold_amd.model.fastnn.ops import Linear
+    """A call whose input asks for gradients takes the differentiable composition; the in-place variants are
+    forward-only launches and raise instead of returning a tensor cut off from the graph."""
+    from fastfold_amd.model.fastnn.ops import ChunkTransition, Linear
     lin = Linear(64, 64).to(dev)
     x = torch.randn(4, 64, device=dev, requires_grad=True)
-    with pytest.raises(NotImplementedError, match="forward pass only"):
-        lin(x)
+    y = lin(x)
+    assert y.grad_fn is not None
+    y.sum().backward()
+    assert torch.allclose(x.grad, lin.weight.sum(0).expand(4, 64), atol=1e-5)
     with torch.no_grad():
         assert not lin(x).requires_grad
-    assert not lin(x.detach()).requires_grad
+        assert torch.allclose(lin(x), y, atol=1e-5)
+    tr = ChunkTransition(128).to(dev)
+    z = torch.randn(1, 8, 8, 128, device=dev, requires_grad=True)
+    with pytest.raises(NotImplementedError, match="forward pass only"):
+        tr.inplace([z])
+    assert tr(z).grad_fn is not None
 
 
 def test_dropout_modules_are_identity_in_eval(dev):
@@ -342,16 +349,13 @@ def test_packed_weights_follow_the_parameters(dev):
         assert lin(x.to(torch.bfloat16)).dtype == torch.bfloat16
 
 
-def test_elementwise_ops_refuse_to_drop_gradients(dev):
+def test_elementwise_ops_keep_the_graph(dev):
     from fastfold_amd.model.fastnn.kernel import bias_dropout_add, bias_ele_dropout_residual, bias_sigmod_ele
     x = torch.randn(1, 4, 6, 32, device=dev, requires_grad=True)
     b = torch.zeros(32, device=dev)
     dm = torch.ones(1, 1, 6, 32, device=dev)
-    with pytest.raises(NotImplementedError):
-        bias_sigmod_ele(x, b, x.detach())
-    with pytest.raises(NotImplementedError):
-        bias_dropout_add(x, b, dm, x.detach(), prob=0.1, training=False)
-    with pytest.raises(NotImplementedError):
-        bias_ele_dropout_residual(x.detach(), b, x, dm, x.detach(), prob=0.1, training=False)
+    assert bias_sigmod_ele(x, b, x.detach()).grad_fn is not None
+    assert bias_dropout_add(x, b, dm, x.detach(), prob=0.1, training=False).grad_fn is not None
+    assert bias_ele_dropout_residual(x.detach(), b, x, dm, x.detach(), prob=0.1, training=False).grad_fn is not None
     with torch.no_grad():
         assert bias_sigmod_ele(x, b, x).shape == x.shape

@@ -1,0 +1,228 @@
+"""The differentiable path of the fastnn modules (what benchmark/perf.py's forward + backward mode and
+tests/test_train.py exercise in the reference): a call that autograd has to see runs the reference's own operator
+sequence, with the HIP LayerNorm / attention-core / elementwise kernels and their backward passes.
+
+Gradients are checked against autograd through the CPU oracle in float64 (oracle.evoformer_ref, whose forward is
+pinned by the reference's golden vectors).  Parameter gradients are carried from the oracle's layout to the fastnn
+layout by the weight re-layout itself: it only copies and concatenates, so applied to a model whose parameters hold
+their gradients it yields the gradients of the re-laid-out parameters.
+
+Tolerances: fp32 relative L2 <= 3e-3 per gradient tensor (1e-6 is what is measured when no ReLU input changes sign
+between the float32 run and the float64 oracle; one such flip among the 2 M hidden activations of the pair
+transition moves every upstream gradient by ~ 1e-3 of its norm, and about one is expected per block at these
+sizes); bf16 relative L2 <= 5e-2 on the input gradients.
+"""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from fastfold_amd.synthetic import synth_inputs, synth_nn_state
+from oracle.evoformer_ref import OracleModel
+
+pytestmark = pytest.mark.gpu
+
+KW = dict(c_m=256, c_z=128, c_hidden_msa_att=32, c_hidden_opm=32, c_hidden_mul=128, c_hidden_pair_att=32, c_s=384,
+          no_heads_msa=8, no_heads_pair=4, transition_n=4, msa_dropout=0.15, pair_dropout=0.25, blocks_per_ckpt=1,
+          inf=1e9, eps=1e-8)
+
+
+def _oracle(seed, nb):
+    model = OracleModel(no_blocks=nb, **KW).eval()
+    sd = synth_nn_state(seed=seed, no_blocks=nb, fan_in_scaled=True, std=0.02)
+    model.evoformer.load_state_dict({k: torch.from_numpy(v) for k, v in sd.items()}, strict=True)
+    return model
+
+
+def _fast(model, dev, dtype):
+    from fastfold_amd.utils.inject_fastnn import inject_fastnn
+    return inject_fastnn(copy.deepcopy(model)).evoformer.to(device=dev, dtype=dtype)
+
+
+def _rel(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+def _oracle_run(model, m, z, mm, pm, cot):
+    """Outputs, input gradients and (in the fastnn layout) parameter gradients of the float64 oracle."""
+    ref = copy.deepcopy(model).double()
+    mi, zi = (torch.from_numpy(t).double().requires_grad_() for t in (m, z))
+    out = ref.evoformer(mi, zi, torch.from_numpy(mm).double(), torch.from_numpy(pm).double(), _mask_trans=False)
+    sum((o * c.double()).sum() for o, c in zip(out, cot)).backward()
+    holder = copy.deepcopy(ref)
+    with torch.no_grad():
+        for p, q in zip(holder.parameters(), ref.parameters()):
+            p.copy_(q.grad if q.grad is not None else torch.zeros_like(q))
+    from fastfold_amd.utils.inject_fastnn import inject_fastnn
+    pgrads = dict(inject_fastnn(holder).evoformer.named_parameters())
+    return [o.detach() for o in out], (mi.grad, zi.grad), pgrads
+
+
+def _mask_cotangents(cot, r, tail):
+    """Zero cotangents at masked residues: what a module leaves there is unspecified (a softmax over keys that are
+    all masked is uniform in the reference's kernel and input-dependent in the oracle), and nothing at a valid
+    residue reads it."""
+    nv = r - int(round(tail * r))
+    cot[0][:, nv:] = 0
+    cot[1][nv:] = 0
+    cot[1][:, nv:] = 0
+    cot[2][nv:] = 0
+    return nv
+
+
+@pytest.mark.parametrize("nb,s,r,tail", [(1, 12, 40, 0.2), (2, 33, 64, 0.0)])
+def test_stack_gradients_fp32(dev, nb, s, r, tail):
+    model = _oracle(31, nb)
+    m, z, mm, pm = synth_inputs(31, s, r, mask_tail_frac=tail)
+    g = torch.Generator().manual_seed(5)
+    cot = [torch.randn(s, r, KW["c_m"], generator=g), torch.randn(r, r, KW["c_z"], generator=g),
+           torch.randn(r, KW["c_s"], generator=g)]
+    nv = _mask_cotangents(cot, r, tail)
+    ref_out, ref_gin, ref_gp = _oracle_run(model, m, z, mm, pm, cot)
+
+    fast = _fast(model, dev, torch.float32).eval()            # eval: no dropout; gradients still flow
+    mi, zi = (torch.from_numpy(t).to(dev).requires_grad_() for t in (m, z))
+    out = fast(mi, zi, torch.from_numpy(mm).to(dev), torch.from_numpy(pm).to(dev), chunk_size=None)
+    assert all(o.grad_fn is not None for o in out)
+    with torch.no_grad():                                       # the fused forward-only launches agree with it
+        fused = fast(mi, zi, torch.from_numpy(mm).to(dev), torch.from_numpy(pm).to(dev), chunk_size=None)
+    for o, f, ref in zip((out[0][:, :nv], out[1][:nv, :nv], out[2][:nv]),
+                         (fused[0][:, :nv], fused[1][:nv, :nv], fused[2][:nv]),
+                         (ref_out[0][:, :nv], ref_out[1][:nv, :nv], ref_out[2][:nv])):
+        assert _rel(o, ref) <= 2e-5, _rel(o, ref)
+        assert _rel(o, f) <= 2e-5, _rel(o, f)
+    sum((o * c.to(dev)).sum() for o, c in zip(out, cot)).backward()
+    assert _rel(mi.grad, ref_gin[0]) <= 3e-3, _rel(mi.grad, ref_gin[0])
+    assert _rel(zi.grad, ref_gin[1]) <= 3e-3, _rel(zi.grad, ref_gin[1])
+    checked = 0
+    for name, p in fast.named_parameters():
+        want = ref_gp[name].detach().double()
+        assert p.grad is not None, name
+        err = float((p.grad.double().cpu() - want).norm())
+        # the absolute term covers gradients that are zero by construction (a LayerNorm bias that shifts every logit
+        # of a softmax row by the same amount): the others have norms of 30 .. 10 000 here
+        assert err <= 3e-3 * float(want.norm()) + 1e-3, (name, err, float(want.norm()))
+        checked += float(want.norm()) > 1.0
+    assert checked >= 70 * nb, checked
+
+
+def test_stack_gradients_bf16_and_checkpointing(dev):
+    """bf16 training step in train() mode with dropout probabilities forced to zero (so that it is comparable):
+    blocks are re-run in the backward pass (blocks_per_ckpt = 1) and give the gradients of the un-checkpointed run."""
+    nb, s, r = 2, 16, 48
+    model = _oracle(32, nb)
+    m, z, mm, pm = synth_inputs(32, s, r, mask_tail_frac=0.1)
+    g = torch.Generator().manual_seed(6)
+    cot = [torch.randn(s, r, KW["c_m"], generator=g), torch.randn(r, r, KW["c_z"], generator=g),
+           torch.randn(r, KW["c_s"], generator=g)]
+    _mask_cotangents(cot, r, 0.1)
+    _, ref_gin, _ = _oracle_run(model, m, z, mm, pm, cot)
+    fast = _fast(model, dev, torch.bfloat16).train()
+    for mod in fast.modules():
+        if hasattr(mod, "p_drop"):
+            mod.p_drop = 0.0
+    grads = []
+    for per in (1, None):
+        fast.blocks_per_ckpt = per
+        mi, zi = (torch.from_numpy(t).to(dev, torch.bfloat16).requires_grad_() for t in (m, z))
+        out = fast(mi, zi, torch.from_numpy(mm).to(dev, torch.bfloat16), torch.from_numpy(pm).to(dev, torch.bfloat16),
+                   chunk_size=None)
+        sum((o.float() * c.to(dev)).sum() for o, c in zip(out, cot)).backward()
+        grads.append((mi.grad.clone(), zi.grad.clone()))
+        fast.zero_grad()
+    # not bit for bit: the pair-bias gradient is accumulated with floating-point atomics, and a last-bit difference
+    # there becomes a bf16 rounding step (4e-3) further up
+    assert _rel(grads[0][0], grads[1][0]) <= 2e-2 and _rel(grads[0][1], grads[1][1]) <= 2e-2
+    assert _rel(grads[0][0], ref_gin[0]) <= 5e-2, _rel(grads[0][0], ref_gin[0])
+    assert _rel(grads[0][1], ref_gin[1]) <= 5e-2, _rel(grads[0][1], ref_gin[1])
+
+
+def test_block_chain_the_benchmark_way(dev):
+    """benchmark/perf.py:141-155: stand-alone first / middle / last blocks in their default (training) mode, inputs
+    that require gradients, ``layer_inputs[1].backward(grads)``.  Dropout is active: every triangle update drops
+    whole rows (columns for the ending node) of channels with one mask, so only shapes, finiteness and the
+    presence of every gradient are checked here."""
+    from fastfold_amd.model.fastnn import Evoformer
+    torch.manual_seed(0)
+    s, r, cm, cz = 16, 40, 256, 128
+    layers = [Evoformer(c_m=cm, c_z=cz, first_block=(i == 0), last_block=(i == 2)).to(dev, torch.bfloat16)
+              for i in range(3)]
+    node = torch.randn(s, r, cm, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    pair = torch.randn(r, r, cz, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    nmask = torch.ones(s, r, device=dev, dtype=torch.bfloat16)
+    pmask = torch.ones(r, r, device=dev, dtype=torch.bfloat16)
+    x = (node, pair)
+    for i, lyr in enumerate(layers):
+        x = lyr.forward(*x, nmask, pmask)
+        if i < 2:
+            assert x[0].shape == (1, s, r + 1, cm) and x[1].shape == (1, r + 1, r + 1, cz)
+    assert x[0].shape == (s, r, cm) and x[1].shape == (r, r, cz)
+    x[1].backward(torch.randn_like(pair))
+    assert node.grad is not None and pair.grad is not None
+    assert torch.isfinite(node.grad.float()).all() and torch.isfinite(pair.grad.float()).all()
+    assert float(pair.grad.float().abs().max()) > 0
+
+
+def test_dropout_masks_are_shared_along_rows_and_columns(dev):
+    """bias_dropout_add / bias_ele_dropout_residual in training mode: one mask per (column, channel) for the row-wise
+    updates, per (row, channel) for the ending node (fastnn/ops.py:405-412, :899-905); kept entries are scaled by
+    1 / (1 - p)."""
+    from fastfold_amd.model.fastnn.ops import ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode
+    torch.manual_seed(1)
+    r, cz = 32, 128
+    z = torch.randn(1, r, r, cz, device=dev)
+    mask = torch.ones(1, r, r, device=dev)
+    for cls, dim in ((ChunkTriangleAttentionStartingNode, 1), (ChunkTriangleAttentionEndingNode, 2)):
+        mod = cls(cz, p_drop=0.25, c=32, n_head=4).to(dev)
+        with torch.no_grad():
+            mod.attention.o_linear.weight.zero_()        # the update is then the bias alone
+            mod.out_bias.fill_(1.0)
+        upd = mod(z, mask) - z                           # parameters require gradients -> differentiable path
+        assert upd.grad_fn is not None
+        vals = torch.unique(upd.detach().round(decimals=4)).tolist()
+        assert len(vals) == 2 and vals[0] == 0.0 and abs(vals[1] - 1 / 0.75) < 1e-4, vals
+        keep = (upd.detach() != 0)
+        assert torch.equal(keep, keep.narrow(dim, 0, 1).expand_as(keep))
+        assert 0.5 < float(keep.float().mean()) < 0.95
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_elementwise_ops_backward(dev, dtype):
+    from fastfold_amd.model.fastnn.kernel import bias_dropout_add, bias_ele_dropout_residual, bias_sigmod_ele
+    g = torch.Generator().manual_seed(3)
+    shape = (1, 5, 7, 64)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+
+    def leaf(*sh):
+        return torch.randn(*sh, generator=g).to(dev, dtype).requires_grad_()
+
+    def f64(t):
+        return t.detach().double().requires_grad_()
+    cot = torch.randn(*shape, generator=g).to(dev)
+    dm = (torch.rand(1, 1, 7, 64, generator=g) > 0.3).to(dev, dtype) / 0.7
+
+    y, b, z = leaf(*shape), leaf(64), leaf(*shape)
+    out = bias_sigmod_ele(y, b, z)
+    (out.float() * cot).sum().backward()
+    y2, b2, z2 = f64(y), f64(b), f64(z)
+    (torch.sigmoid(y2 + b2) * z2 * cot.double()).sum().backward()
+    for a, ref in ((y, y2), (b, b2), (z, z2)):
+        assert _rel(a.grad, ref.grad) <= tol, _rel(a.grad, ref.grad)
+
+    x, b, res = leaf(*shape), leaf(64), leaf(*shape)
+    out = bias_dropout_add(x, b, dm, res, prob=0.3, training=False)
+    (out.float() * cot).sum().backward()
+    x2, b2, r2 = f64(x), f64(b), f64(res)
+    ((r2 + (x2 + b2) * dm.double()) * cot.double()).sum().backward()
+    for a, ref in ((x, x2), (b, b2), (res, r2)):
+        assert _rel(a.grad, ref.grad) <= tol, _rel(a.grad, ref.grad)
+
+    ab, b, gt, zr = leaf(*shape), leaf(64), leaf(*shape), leaf(*shape)
+    out = bias_ele_dropout_residual(ab, b, gt, dm, zr, prob=0.3, training=False)
+    (out.float() * cot).sum().backward()
+    ab2, b2, g2, zr2 = f64(ab), f64(b), f64(gt), f64(zr)
+    ((zr2 + dm.double() * (g2 * (ab2 + b2))) * cot.double()).sum().backward()
+    for a, ref in ((ab, ab2), (b, b2), (gt, g2), (zr, zr2)):
+        assert _rel(a.grad, ref.grad) <= tol, _rel(a.grad, ref.grad)
