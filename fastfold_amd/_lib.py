@@ -273,6 +273,25 @@ def attention_bwd(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, 
          dq_scale, dk_scale, dtype_tag(q_qk.dtype), stream_ptr())
 
 
+SIGNATURES["ffk_tile_pack"] = [_P, _P, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I, _P]
+
+
+def tile_pack(x, kind, scale=1.0):
+    """[B2, H, N, D <= 32] (any strides over the first three dims, channels contiguous) -> [B2, H, ceil(N/32), 1024]
+    operand tiles of the attention kernels in ``kind`` order (``FFK_TILE_QK`` / ``FFK_TILE_V``), times ``scale``."""
+    import torch
+    if x.dim() != 4 or x.shape[-1] > 32:
+        raise RuntimeError("tile_pack: expected [B2, H, N, D <= 32], got %s" % (tuple(x.shape),))
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    B2, H, N, D = x.shape
+    out = torch.empty(B2, H, (N + 31) // 32, 1024, dtype=x.dtype, device=x.device)
+    if out.numel():
+        call("ffk_tile_pack", ptr(out), ptr(x), B2, H, N, D, x.stride(0), x.stride(1), x.stride(2), float(scale), kind,
+             dtype_tag(x.dtype), stream_ptr())
+    return out
+
+
 SIGNATURES["ffk_pair_bias"] = [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _F, _F, _I, _P]
 
 

@@ -424,6 +424,127 @@ __global__ __launch_bounds__(BLOCK) void layernorm_bwd_kernel(T* dx, float* dgam
     }
 }
 
+// Vector form of the backward pass for rows of exactly LPR * VPL vectors (at most LN_BWD_MAXCOLS elements): one pass
+// over x and dy with 16-byte loads, the row sums inside the lane group, and the column sums for dgamma / dbeta kept
+// per lane over the whole grid-stride loop, then folded across the wave's row groups (xor shuffles), across the
+// block's waves (LDS) and into the result with one atomic per column and block.
+constexpr int LN_BWD_MAXCOLS = 1024;
+template <typename T, int LPR, int VPL>
+__global__ __launch_bounds__(BLOCK) void layernorm_bwd_vec_kernel(T* __restrict__ dx, float* dgamma, float* dbeta,
+                                                                 const T* __restrict__ dy, const T* __restrict__ x,
+                                                                 const float* __restrict__ mean,
+                                                                 const float* __restrict__ rstd,
+                                                                 const T* __restrict__ gamma, unsigned rows) {
+    constexpr int VEC = DT<T>::VEC;
+    constexpr int RPW = 64 / LPR;
+    constexpr int ROWLEN = LPR * VPL * VEC;
+    __shared__ float red[WAVES_PER_BLOCK][2][ROWLEN];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int sub = lane / LPR;
+    const int j = lane % LPR;
+    const float inv_n = 1.0f / (float)ROWLEN;
+    float gm[VPL][VEC], pg[VPL][VEC], pb[VPL][VEC];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+        Vec16<T> gv = ld16(gamma + (j + i * LPR) * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            gm[i][e] = DT<T>::to_f(gv.e[e]);
+            pg[i][e] = pb[i][e] = 0.0f;
+        }
+    }
+    const unsigned stride = gridDim.x * WAVES_PER_BLOCK * RPW;
+    for (unsigned base = (blockIdx.x * WAVES_PER_BLOCK + wave) * RPW; base < rows; base += stride) {
+        const unsigned row = base + sub;
+        const bool valid = row < rows;
+        const unsigned rc = valid ? row : rows - 1;              // clamped: neither stored nor accumulated below
+        const T* xr = x + (long)rc * ROWLEN + j * VEC;
+        const T* gr = dy + (long)rc * ROWLEN + j * VEC;
+        Vec16<T> xv[VPL], dv[VPL];
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            xv[i] = ld16_nt(xr + i * LPR * VEC);
+            dv[i] = ld16_nt(gr + i * LPR * VEC);
+        }
+        const float mu = mean[rc], rs = rstd[rc];
+        float xh[VPL][VEC], g[VPL][VEC];
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float d = valid ? DT<T>::to_f(dv[i].e[e]) : 0.0f;
+                xh[i][e] = (DT<T>::to_f(xv[i].e[e]) - mu) * rs;
+                g[i][e] = d * gm[i][e];
+                s1 += g[i][e];
+                s2 += g[i][e] * xh[i][e];
+                pg[i][e] += d * xh[i][e];
+                pb[i][e] += d;
+            }
+        }
+        s1 = group_sum(s1, LPR) * inv_n;
+        s2 = group_sum(s2, LPR) * inv_n;
+        T* orow = dx + (long)rc * ROWLEN + j * VEC;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            Vec16<T> ov;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) ov.e[e] = DT<T>::from_f(rs * (g[i][e] - s1 - xh[i][e] * s2));
+            if (valid) st16_nt(orow + i * LPR * VEC, ov);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+#pragma unroll
+            for (int off = LPR; off < 64; off <<= 1) {
+                pg[i][e] += __shfl_xor(pg[i][e], off, 64);
+                pb[i][e] += __shfl_xor(pb[i][e], off, 64);
+            }
+            if (sub == 0) {
+                red[wave][0][(j + i * LPR) * VEC + e] = pg[i][e];
+                red[wave][1][(j + i * LPR) * VEC + e] = pb[i][e];
+            }
+        }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < ROWLEN; c += BLOCK) {
+        float a = 0.0f, b = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES_PER_BLOCK; ++w) {
+            a += red[w][0][c];
+            b += red[w][1][c];
+        }
+        atomicAdd(dgamma + c, a);
+        atomicAdd(dbeta + c, b);
+    }
+}
+
+template <typename T>
+bool layernorm_bwd_vec_launch(T* dx, float* dgamma, float* dbeta, const T* dy, const T* x, const float* mean,
+                              const float* rstd, const T* gamma, long rows, long cols, hipStream_t st) {
+    constexpr int VEC = DT<T>::VEC;
+    RowGeom g;
+    if (cols % VEC != 0 || cols > LN_BWD_MAXCOLS || !ffk_aligned16(dx) || !ffk_aligned16(dy) || !ffk_aligned16(x) ||
+        !ffk_aligned16(gamma) || rows >= (1L << 31) - (1L << 24) || !row_geom(cols / VEC, &g) ||
+        cols != (long)g.lpr * g.vpl * VEC)
+        return false;
+    const long rows_per_block = (long)WAVES_PER_BLOCK * (64 / g.lpr);
+    const long need = (rows + rows_per_block - 1) / rows_per_block;
+    dim3 grid((unsigned)(need < 256L * 2 ? need : 256L * 2));
+#define FFK_LNB_CASE(L, V)                                                                                            \
+    if (g.lpr == L && g.vpl == V && (long)L * V * VEC <= LN_BWD_MAXCOLS) {                                            \
+        layernorm_bwd_vec_kernel<T, L, (L * V * VEC <= LN_BWD_MAXCOLS ? V : 1)><<<grid, BLOCK, 0, st>>>(             \
+            dx, dgamma, dbeta, dy, x, mean, rstd, gamma, (unsigned)rows);                                             \
+        return true;                                                                                                  \
+    }
+    FFK_ROW_GEOMETRIES(FFK_LNB_CASE)
+#undef FFK_LNB_CASE
+    return false;
+}
+
 template <typename T>
 int layernorm_launch(T* out, float* mean, float* rstd, const T* x, const T* gamma, const T* beta, long rows,
                      long cols, float eps, hipStream_t st) {
@@ -610,6 +731,14 @@ extern "C" int ffk_layernorm_bwd(void* dx, float* dgamma, float* dbeta, const vo
     FFK_REQUIRE(rows > 0 && cols > 0 && cols < (1L << 30), FFK_ERR_SHAPE, "ffk_layernorm_bwd: bad shape [%ld,%ld]",
                 (long)rows, (long)cols);
     hipStream_t st = (hipStream_t)stream;
+    bool done = false;
+    switch (dtype) {
+        case FFK_F32: done = layernorm_bwd_vec_launch<float>((float*)dx, dgamma, dbeta, (const float*)dy, (const float*)x, mean, rstd, (const float*)gamma, rows, cols, st); break;
+        case FFK_BF16: done = layernorm_bwd_vec_launch<bf16_t>((bf16_t*)dx, dgamma, dbeta, (const bf16_t*)dy, (const bf16_t*)x, mean, rstd, (const bf16_t*)gamma, rows, cols, st); break;
+        case FFK_F16: done = layernorm_bwd_vec_launch<f16_t>((f16_t*)dx, dgamma, dbeta, (const f16_t*)dy, (const f16_t*)x, mean, rstd, (const f16_t*)gamma, rows, cols, st); break;
+        default: return ffk_fail(FFK_ERR_DTYPE, "ffk_layernorm_bwd: unsupported dtype tag %d", dtype);
+    }
+    if (done) return ffk_check_launch("ffk_layernorm_bwd");
     const long waves = 256L * 8 * WAVES_PER_BLOCK;
     const long rpw = (rows + waves - 1) / waves;
     const long nw = (rows + rpw - 1) / rpw;

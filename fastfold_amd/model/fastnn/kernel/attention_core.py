@@ -21,7 +21,9 @@ from . import layouts
 
 
 def _attention_core(q, k, v, mask=None, bias=None):
-    _lib.check_device(q, k, v, mask, bias)
+    for t in (q, k, v, mask, bias):          # any strides: the operands are re-tiled as they lie
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("fastfold_amd: tensor must be a CUDA/HIP tensor (got %s)" % t.device)
     if q.dim() != 5 or q.shape != k.shape or q.shape != v.shape:
         raise RuntimeError("fused_attention_core: q, k, v must be [b1, b2, h, n, d] of one shape, got %s %s %s"
                            % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
@@ -29,33 +31,27 @@ def _attention_core(q, k, v, mask=None, bias=None):
     if d not in (8, 16, 32):
         raise RuntimeError("fused_attention_core: head dim %d is not supported: the kernel is built for 32 and takes "
                            "8 and 16 zero-padded; 64 and 128 (accepted by the reference's Triton kernel) are not built" % d)
-    if d != 32:      # zero channels add nothing to q.k and give zero output channels, which are dropped below
-        pad = torch.nn.functional.pad
-        out = _attention_core_d32(pad(q, (0, 32 - d)), pad(k, (0, 32 - d)), pad(v, (0, 32 - d)), mask, bias, d)
-        return out.view(b1, b2, n, h, 32)[..., :d].reshape(b1, b2, n, h * d)
-    return _attention_core_d32(q, k, v, mask, bias, d)
-
-
-def _attention_core_d32(q, k, v, mask, bias, d_scale):
-    b1, b2, h, n, d = q.shape
     if mask is not None and tuple(mask.shape) != (b1, b2, n):
         raise RuntimeError("fused_attention_core: mask must be [b1, b2, n], got %s" % (tuple(mask.shape),))
     if bias is not None and tuple(bias.shape) != (b1, h, n, n):
         raise RuntimeError("fused_attention_core: bias must be [b1, h, n, n], got %s" % (tuple(bias.shape),))
-    out = torch.empty(b1, b2, n, h * d, dtype=q.dtype, device=q.device)
+    # zero channels past d add nothing to q.k and give zero output channels, which are dropped at the end
+    out = torch.empty(b1, b2, n, h * 32, dtype=q.dtype, device=q.device)
     if out.numel() == 0:
-        return out
+        return out.view(b1, b2, n, h, 32)[..., :d].reshape(b1, b2, n, h * d)
     nt = layouts.n_tiles(n)
-    scale = _lib.LOG2E / math.sqrt(d_scale)      # the kernel exponentiates in base 2; the scale is the true head dim's
+    scale = _lib.LOG2E / math.sqrt(d)      # the kernel exponentiates in base 2
     kb = torch.empty(b2, nt * 32, dtype=torch.float32, device=q.device)
     fl = torch.empty(b2, nt, dtype=torch.int32, device=q.device)
     for i in range(b1):
         mk = mask[i].to(q.dtype).contiguous() if mask is not None else torch.ones(b2, n, dtype=q.dtype, device=q.device)
         _lib.key_bias(kb, fl, mk, B=b2, N=n, mask_sb=n, mask_sn=1)
-        qt = layouts.tile_qk((q[i].float() * scale).to(q.dtype))
         bt = layouts.tile_bias((bias[i].float() * _lib.LOG2E).to(q.dtype)) if bias is not None else None
-        _lib.attention_fwd(out[i].view(b2 * n, h * d), qt, layouts.tile_qk(k[i]), layouts.tile_v(v[i]), bt, kb, fl,
+        _lib.attention_fwd(out[i].view(b2 * n, h * 32), _lib.tile_pack(q[i], _lib.FFK_TILE_QK, scale),
+                           _lib.tile_pack(k[i], _lib.FFK_TILE_QK), _lib.tile_pack(v[i], _lib.FFK_TILE_V), bt, kb, fl,
                            None, B2=b2, H=h, Nq=n, Nk=n)
+    if d != 32:
+        return out.view(b1, b2, n, h, 32)[..., :d].reshape(b1, b2, n, h * d)
     return out
 
 
@@ -63,11 +59,7 @@ def _attention_core_backward(q, k, v, mask, bias, out, dout, need_dbias):
     """dq, dk, dv (shapes of q, k, v) and dbias ([b1, h, n, n] or None) through ``ffk_attention_bwd``."""
     b1, b2, h, n, d = q.shape
     dt, dev = q.dtype, q.device
-    if d != 32:
-        pad = torch.nn.functional.pad
-        q, k, v = (pad(t, (0, 32 - d)) for t in (q, k, v))
-        out = pad(out.view(b1, b2, n, h, d), (0, 32 - d)).reshape(b1, b2, n, h * 32)
-        dout = pad(dout.view(b1, b2, n, h, d), (0, 32 - d)).reshape(b1, b2, n, h * 32)
+    QK, ACC = _lib.FFK_TILE_QK, _lib.FFK_TILE_V
     nt = layouts.n_tiles(n)
     scale = _lib.LOG2E / math.sqrt(d)
     dq, dk, dv = (torch.empty(b1, b2, h, n, 32, dtype=dt, device=dev) for _ in range(3))
@@ -79,17 +71,17 @@ def _attention_core_backward(q, k, v, mask, bias, out, dout, need_dbias):
     for i in range(b1):
         mk = mask[i].to(dt).contiguous() if mask is not None else torch.ones(b2, n, dtype=dt, device=dev)
         _lib.key_bias(kb, fl, mk, B=b2, N=n, mask_sb=n, mask_sn=1)
-        q2 = (q[i].float() * scale).to(dt)                       # the operand the forward kernel saw
         b2s = (bias[i].float() * _lib.LOG2E).to(dt).contiguous() if bias is not None else None
-        do_ = dout[i].reshape(b2, n, h, 32).permute(0, 2, 1, 3).contiguous()
-        o_ = out[i].reshape(b2, n, h, 32).permute(0, 2, 1, 3).contiguous()
+        do_ = dout[i].view(b2, n, h, d).permute(0, 2, 1, 3)          # [b2, h, n, d] views: re-tiled as they lie
+        o_ = out[i].view(b2, n, h, d).permute(0, 2, 1, 3)
         _lib.attention_bwd(dq[i], dk[i], dv[i], None if dbias is None else dbias[i], lse, dsum,
-                           layouts.tile_qk(q2), layouts.tile_v(q2), layouts.tile_qk(k[i]), layouts.tile_v(k[i]),
-                           layouts.tile_qk(v[i]), None if b2s is None else layouts.tile_bias(b2s), b2s, kb,
-                           layouts.tile_qk(do_), layouts.tile_v(do_), layouts.tile_qk(o_),
+                           _lib.tile_pack(q[i], QK, scale), _lib.tile_pack(q[i], ACC, scale),     # as the forward saw q
+                           _lib.tile_pack(k[i], QK), _lib.tile_pack(k[i], ACC), _lib.tile_pack(v[i], QK),
+                           None if b2s is None else layouts.tile_bias(b2s), b2s, kb,
+                           _lib.tile_pack(do_, QK), _lib.tile_pack(do_, ACC), _lib.tile_pack(o_, QK),
                            B2=b2, H=h, Nq=n, Nk=n, dq_scale=1.0 / math.sqrt(d), dk_scale=1.0 / _lib.LOG2E)
     if d != 32:
-        dq, dk, dv = (t[..., :d].contiguous() for t in (dq, dk, dv))
+        dq, dk, dv = (t[..., :d] for t in (dq, dk, dv))
     return dq, dk, dv, (None if dbias is None else dbias.to(dt))
 
 
@@ -108,7 +100,7 @@ class FusedAttenionCoreFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout):
         q, k, v, mask, bias, out = ctx.saved_tensors
-        dq, dk, dv, dbias = _attention_core_backward(q, k, v, mask, bias, out, dout.contiguous(),
+        dq, dk, dv, dbias = _attention_core_backward(q, k, v, mask, bias, out.contiguous(), dout.contiguous(),
                                                      bias is not None and ctx.needs_input_grad[4])
         return dq, dk, dv, None, dbias
 

@@ -86,6 +86,46 @@ def _needs_grad(module, *tensors):
     return any(p.requires_grad for p in module.parameters())
 
 
+_WGRAD_SPLIT_ROWS = 4096
+
+
+def _weight_grad(dy2, x2):
+    """dy2^T . x2 for [M, N] and [M, K] activations with M in the hundreds of thousands: one GEMM whose whole
+    parallelism is its N x K output (a few hundred tiles reducing over a million rows each) runs at a few per cent
+    of the matrix pipe, so the rows are cut into slabs that a batched GEMM reduces side by side; the slab results
+    are added in fp32."""
+    M = dy2.shape[0]
+    S = 1
+    while M % (2 * S) == 0 and M // (2 * S) >= _WGRAD_SPLIT_ROWS:
+        S *= 2
+    if S == 1 or dy2.dtype == torch.float32:
+        return dy2.t() @ x2
+    part = torch.bmm(dy2.view(S, M // S, -1).transpose(1, 2), x2.view(S, M // S, -1))
+    return part.sum(0, dtype=torch.float32).to(dy2.dtype)
+
+
+class _LinearFn(torch.autograd.Function):
+    """y = x W^T + b through the library GEMM, with the weight gradient computed by ``_weight_grad``."""
+
+    @staticmethod
+    def forward(ctx, x, w, b):
+        ctx.save_for_backward(x, w)
+        return torch.nn.functional.linear(x, w, b)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = (dy2 @ w).view(x.shape)
+        if ctx.needs_input_grad[1]:
+            dw = _weight_grad(dy2, x.reshape(-1, x.shape[-1]))
+        if ctx.needs_input_grad[2]:
+            db = dy2.sum(0)
+        return dx, dw, db
+
+
 def _check_tail(xtail, x):
     """The int8 tail of ``x`` as an extended residual stream (see include/ffk.h): same shape, bf16 stream only."""
     if xtail is None:
@@ -169,8 +209,8 @@ class Linear(nn.Linear, _PackMixin):
         if _needs_grad(self, input):
             if act != _lib.FFK_ACT_NONE:
                 raise NotImplementedError("Linear: fused activations are forward-only")
-            return torch.nn.functional.linear(input, self.weight.to(input.dtype),
-                                              self.bias.to(input.dtype) if self.use_bias else None)
+            return _LinearFn.apply(input, self.weight.to(input.dtype),
+                                   self.bias.to(input.dtype) if self.use_bias else None)
         w, b = self._pk(input.dtype, input.device)
         x2 = input.reshape(-1, self.in_features)
         kp = self._kpad()
@@ -351,7 +391,8 @@ class SelfAttention(nn.Module, _PackMixin):
                 bias = bias.permute(0, 3, 1, 2)                 # 'b q k h -> b h q k'
             bias = bias.contiguous()
         qkv = self.to_qkv(in_data).chunk(3, dim=-1)
-        q, k, v = (t.unflatten(-1, (self.n_head, self.c)).transpose(-2, -3).contiguous() for t in qkv)
+        # [b1, b2, h, n, d] views of the projection's output: the operator re-tiles them as they lie
+        q, k, v = (t.unflatten(-1, (self.n_head, self.c)).transpose(-2, -3) for t in qkv)
         if mask is not None:
             mask = mask.to(in_data.dtype).contiguous()
         weighted_avg = fused_attention_core(q, k, v, mask, bias)          # [b1, b2, n, h * d]

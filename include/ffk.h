@@ -300,6 +300,15 @@ int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, fl
                       const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, float dq_scale,
                       float dk_scale, int dtype, void* stream);
 
+/* Re-tiles a strided tensor x[b2, h, n, d] (element at src + b2*s_b + h*s_h + n*s_n + d, strides in elements,
+ * d contiguous, D <= 32) into [B2][H][ceil(N/32)][1024] operand tiles of ffk_attention_fwd / ffk_attention_bwd, in
+ * FFK_TILE_QK or FFK_TILE_V order: rows past N and channels past D are zero, and every element is multiplied by
+ * `scale` in fp32 before it is rounded (the log2(e) / sqrt(d) of the q operand; 1 for the others).
+ * Replaces: the rearrange / transpose / contiguous chain in front of the reference's attention kernels
+ * (fastfold/model/fastnn/ops.py:303-306; kernel/attention_core.py:24-31), which here has to end in tile order. */
+int ffk_tile_pack(void* dst, const void* src, int64_t B2, int64_t H, int64_t N, int64_t D, int64_t s_b, int64_t s_h,
+                  int64_t s_n, float scale, int kind, int dtype, void* stream);
+
 /* Pair bias of a biased attention, straight into the operand tiles ffk_attention_fwd reads:
  *     bias_t[h][q/32][k/32][tile(k, q)] = scale * ( LayerNorm(z[q, k, :]; gamma, beta, eps) . w[h, :] )
  * z holds N*N rows of C channels; logical row m = q*N + k lives at (m / a_inner) * a_so + (m % a_inner) * a_si

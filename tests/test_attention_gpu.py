@@ -266,3 +266,22 @@ def test_fused_attention_core_backward_fully_masked_rows(dev):
     for t in (q, k, v):
         assert bool(torch.isfinite(t.grad).all()) and float(t.grad[0, 1].abs().max()) == 0.0
         assert float(t.grad[0, 0].abs().max()) > 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("b2,h,n,d", [(3, 4, 70, 32), (2, 8, 33, 16), (1, 4, 128, 8), (5, 4, 31, 32)])
+def test_tile_pack_matches_the_torch_layout_helpers(dev, dtype, b2, h, n, d):
+    """ffk_tile_pack against the pad / view / permute formulation of the same tiles (layouts.tile_qk / tile_v), bit
+    for bit, on a contiguous tensor and on the strided [b2, h, n, d] view of a fused [b2, n, 3 * h * d] projection."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    g = torch.Generator().manual_seed(n + d)
+    qkv = torch.randn(b2, n, 3 * h * d, generator=g).to(dev, dtype)
+    views = [t.unflatten(-1, (h, d)).transpose(-2, -3) for t in qkv.chunk(3, dim=-1)]     # not contiguous
+    pad = torch.nn.functional.pad
+    for x in views + [views[1].contiguous()]:
+        x32 = pad(x, (0, 32 - d))
+        for scale in (1.0, 0.255):
+            ref = (x32.float() * scale).to(dtype) if scale != 1.0 else x32
+            assert torch.equal(_lib.tile_pack(x, _lib.FFK_TILE_QK, scale).view(-1), layouts.tile_qk(ref).reshape(-1))
+            assert torch.equal(_lib.tile_pack(x, _lib.FFK_TILE_V, scale).view(-1), layouts.tile_v(ref).reshape(-1))
