@@ -213,6 +213,40 @@ def long_sequence(dev):
             "tflops": round(block_gflop(s, r) / ms, 1), "peak_device_GB": round(torch.cuda.max_memory_allocated() / 1e9, 1)}
 
 
+def forward_backward(dev, layers=4, trials=5, warm=2):
+    """The reference's own harness shape (benchmark/perf.py:83-183): stand-alone blocks in training mode (dropout
+    active), bf16, N_seq = 128, N_res = 256, inputs that require gradients, ``layer_inputs[1].backward(grads)``;
+    HIP-event times of the forward and of the backward pass per layer."""
+    import torch
+    from fastfold_amd.model.fastnn import Evoformer
+    s, r = 128, 256
+    torch.manual_seed(0)
+    blocks = [Evoformer(c_m=256, c_z=128, first_block=(i == 0), last_block=(i == layers - 1)).to(dev, torch.bfloat16)
+              for i in range(layers)]
+    node = torch.randn(s, r, 256, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    pair = torch.randn(r, r, 128, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    nm = torch.ones(s, r, device=dev, dtype=torch.bfloat16)
+    pm = torch.ones(r, r, device=dev, dtype=torch.bfloat16)
+    grads = torch.randn_like(pair)
+    fwd = bwd = 0.0
+    for t in range(trials + warm):
+        e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        torch.cuda.synchronize()
+        e0.record()
+        x = (node, pair)
+        for blk in blocks:
+            x = blk(*x, nm, pm)
+        e1.record()
+        x[1].backward(grads)
+        e2.record()
+        torch.cuda.synchronize()
+        if t >= warm:
+            fwd += e0.elapsed_time(e1)
+            bwd += e1.elapsed_time(e2)
+    return {"workload": "benchmark/perf.py shape: %d stand-alone blocks, training mode, bf16, N_seq=128, N_res=256" % layers,
+            "fwd_ms_per_block": round(fwd / trials / layers, 3), "bwd_ms_per_block": round(bwd / trials / layers, 3)}
+
+
 def _cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -399,6 +433,8 @@ def main():
         line["long_sequence"] = long_sequence(dev)
         torch.cuda.empty_cache()
     if not args.no_micro:
+        line["forward_backward"] = forward_backward(dev)
+        torch.cuda.empty_cache()
         line["feeders"] = feeder_stacks(dev, r)
         line["ops"] = micro_ops(dev)
     if not args.no_cpu:

@@ -263,13 +263,13 @@ def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H
          B2, H, Nq, Nk, FFK_ATT_GATE_TILED if gate_tiled else 0, dtype_tag(q_t.dtype), stream_ptr())
 
 
-SIGNATURES["ffk_attention_bwd"] = [_P] * 17 + [_L, _L, _L, _L, _F, _F, _I, _P]
+SIGNATURES["ffk_attention_bwd"] = [_P] * 16 + [_L, _L, _L, _L, _F, _F, _I, _P]
 
 
-def attention_bwd(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, bias_rm, keybias, do_qk, do_acc,
+def attention_bwd(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias, do_qk, do_acc,
                   o_qk, *, B2, H, Nq, Nk, dq_scale, dk_scale):
     call("ffk_attention_bwd", ptr(dq), ptr(dk), ptr(dv), ptr(dbias), ptr(lse), ptr(dsum), ptr(q_qk), ptr(q_acc), ptr(k_qk),
-         ptr(k_acc), ptr(v_qk), ptr(bias_t), ptr(bias_rm), ptr(keybias), ptr(do_qk), ptr(do_acc), ptr(o_qk), B2, H, Nq, Nk,
+         ptr(k_acc), ptr(v_qk), ptr(bias_t), ptr(keybias), ptr(do_qk), ptr(do_acc), ptr(o_qk), B2, H, Nq, Nk,
          dq_scale, dk_scale, dtype_tag(q_qk.dtype), stream_ptr())
 
 

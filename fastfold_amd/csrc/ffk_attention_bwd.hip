@@ -14,8 +14,13 @@
 //                             is the N operand of that product as it stands.
 //   attention_bwd_dkv_kernel  one wave per (b2, head, 32 keys): walks the query tiles with the score tile the other
 //                             way round (queries along the MFMA rows, one key per lane), so that P and dS are the N
-//                             operands of  dv^T = do^T . P  and  dk^T = q^T . dS;  dbias is accumulated with fp32
-//                             atomic adds (consecutive lanes = consecutive keys of one query row).
+//                             operands of  dv^T = do^T . P  and  dk^T = q^T . dS.
+//   attention_bwd_dbias_kernel  one wave per (head, query tile, key tile, slice of the batch rows): recomputes dS of
+//                             its tile for every batch row of the slice, sums in registers and adds the result to
+//                             dbias with one fp32 atomic per element (the slices are what fills the chip when
+//                             H * QT * KT alone is a few hundred tiles).
+// Both take the pair bias from the same operand tiles as the forward kernel: added to the scores by a product with
+// an identity operand, here with the roles of the two operands exchanged (rows = queries).
 // Every operand arrives in the tile order its role needs (the wrapper re-tiles q, k, v, do with the same helpers
 // as the forward pass); waves load their tiles straight from global memory - this pair of kernels serves the
 // autograd path of the stand-alone operator, not the inference block, and is not tuned beyond that.
@@ -179,11 +184,12 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
 // ------------------------------------------------------------------------- dk, dv ----
 template <typename T>
 __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
-    T* __restrict__ dk, T* __restrict__ dv, float* __restrict__ dbias, const T* __restrict__ q_qk,
-    const T* __restrict__ q_acc, const T* __restrict__ k_qk, const T* __restrict__ v_qk, const T* __restrict__ bias_rm,
+    T* __restrict__ dk, T* __restrict__ dv, const T* __restrict__ q_qk,
+    const T* __restrict__ q_acc, const T* __restrict__ k_qk, const T* __restrict__ v_qk, const T* __restrict__ bias_t,
     const float* __restrict__ keybias, const T* __restrict__ do_qk, const T* __restrict__ do_acc,
     const float* __restrict__ lse, const float* __restrict__ dsum, int B2, int H, int Nq, int Nk, float dk_scale) {
     typedef Mma<T> MM;
+    typedef typename MM::Frag Frag;
     constexpr int NF = 16 / MM::KLANE;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
@@ -198,8 +204,12 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
     kf.load(k_qk + ((bh * KT + kt) << 10) + lane * 16);
     vf.load(v_qk + ((bh * KT + kt) << 10) + lane * 16);
     const int key = kt * 32 + l32;
-    const int keyc = key < Nk ? key : Nk - 1;
     const float kb = keybias[(long)b2 * KT * 32 + key];     // 0, masked (-1e9 log2e) or padding (hugely negative)
+    Frag ident[NF];
+    if (bias_t) {
+#pragma unroll
+        for (int i = 0; i < NF; ++i) ident[i] = identity_frag<T>(i, l32, half);
+    }
 
     f32x16 acc_k, acc_v;
 #pragma unroll
@@ -215,6 +225,12 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
         for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.0f;
 #pragma unroll
         for (int i = 0; i < NF; ++i) MM::mma(s, qc.frag(i), kf.frag(i));        // S[q, key], log2 domain
+        if (bias_t) {                                                           // S += I . bias (rows = queries)
+            Tile16<T> bc;
+            bc.load(bias_t + ((((long)h * QT + qt) * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(s, ident[i], bc.frag(i));
+        }
 #pragma unroll
         for (int i = 0; i < NF; ++i) MM::mma(dp, doc.frag(i), vf.frag(i));      // dP[q, key] = do[q] . v[key]
         const float* lp = lse + (bh * QT + qt) * 32 + 4 * half;
@@ -227,15 +243,8 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int v = 4 * g + e;
-                const int qrow = qt * 32 + 8 * g + 4 * half + e;
-                float sv = s[v] + kb;
-                if (bias_rm) {
-                    const int qc_ = qrow < Nq ? qrow : Nq - 1;
-                    sv += DT<T>::to_f(bias_rm[((long)h * Nq + qc_) * Nk + keyc]);
-                }
-                p[v] = fast_exp2(sv - L4[e]);
+                p[v] = fast_exp2(s[v] + kb - L4[e]);
                 ds[v] = p[v] * (dp[v] - D4[e]);
-                if (dbias && qrow < Nq && key < Nk) atomicAdd(dbias + ((long)h * Nq + qrow) * Nk + key, ds[v]);
             }
         }
 #pragma unroll
@@ -256,9 +265,81 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------- dbias ----
+// dbias[h, q, key] += sum over the batch rows b2 = slice, slice + NS, ... of dS[b2, h, q, key].
+template <typename T>
+__global__ __launch_bounds__(256) void attention_bwd_dbias_kernel(
+    float* __restrict__ dbias, const T* __restrict__ q_qk, const T* __restrict__ k_qk, const T* __restrict__ v_qk,
+    const T* __restrict__ bias_t, const float* __restrict__ keybias, const T* __restrict__ do_qk,
+    const float* __restrict__ lse, const float* __restrict__ dsum, int B2, int H, int Nq, int Nk, int NS) {
+    typedef Mma<T> MM;
+    typedef typename MM::Frag Frag;
+    constexpr int NF = 16 / MM::KLANE;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
+    const long item = (long)blockIdx.x * 4 + wave;             // key tile fastest: a block's waves share q and do
+    if (item >= (long)NS * H * QT * KT) return;
+    const int kt = (int)(item % KT);
+    const int qt = (int)((item / KT) % QT);
+    const int h = (int)((item / ((long)KT * QT)) % H);
+    const int slice = (int)(item / ((long)KT * QT * H));
+    const int key = kt * 32 + l32;
+
+    Frag ident[NF];
+#pragma unroll
+    for (int i = 0; i < NF; ++i) ident[i] = identity_frag<T>(i, l32, half);
+    Tile16<T> bc;
+    bc.load(bias_t + ((((long)h * QT + qt) * KT + kt) << 10) + lane * 16);
+    f32x16 sb;                                                  // the bias tile in accumulator order, once
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sb[v] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NF; ++i) MM::mma(sb, ident[i], bc.frag(i));
+
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    for (int b2 = slice; b2 < B2; b2 += NS) {
+        const long bh = (long)b2 * H + h;
+        Tile16<T> qc, doc, kf, vf;
+        qc.load(q_qk + ((bh * QT + qt) << 10) + lane * 16);
+        doc.load(do_qk + ((bh * QT + qt) << 10) + lane * 16);
+        kf.load(k_qk + ((bh * KT + kt) << 10) + lane * 16);
+        vf.load(v_qk + ((bh * KT + kt) << 10) + lane * 16);
+        const float kb = keybias[(long)b2 * KT * 32 + key];
+        f32x16 s = sb, dp;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dp[v] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) MM::mma(s, qc.frag(i), kf.frag(i));
+#pragma unroll
+        for (int i = 0; i < NF; ++i) MM::mma(dp, doc.frag(i), vf.frag(i));
+        const float* lp = lse + (bh * QT + qt) * 32 + 4 * half;
+        const float* dpz = dsum + (bh * QT + qt) * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 L4 = *reinterpret_cast<const f32x4*>(lp + 8 * g);
+            const f32x4 D4 = *reinterpret_cast<const f32x4*>(dpz + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int v = 4 * g + e;
+                acc[v] += fast_exp2(s[v] + kb - L4[e]) * (dp[v] - D4[e]);
+            }
+        }
+    }
+    if (key < Nk) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int qrow = qt * 32 + acc_row(v, lane);
+            if (qrow < Nq) atomicAdd(dbias + ((long)h * Nq + qrow) * Nk + key, acc[v]);
+        }
+    }
+}
+
 template <typename T>
 int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk, const void* q_acc,
-               const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t, const void* bias_rm,
+               const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
                const float* keybias, const void* do_qk, const void* do_acc, const void* o_qk, long B2, long H, long Nq,
                long Nk, float dq_scale, float dk_scale, hipStream_t st) {
     const long QT = (Nq + 31) / 32, KT = (Nk + 31) / 32;
@@ -277,10 +358,22 @@ int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* ds
     }
     int rc = ffk_check_launch("ffk_attention_bwd");
     if (rc != FFK_OK) return rc;
-    attention_bwd_dkv_kernel<T><<<(unsigned)g2, 256, 0, st>>>((T*)dk, (T*)dv, dbias, (const T*)q_qk, (const T*)q_acc,
-                                                            (const T*)k_qk, (const T*)v_qk, (const T*)bias_rm, keybias,
+    attention_bwd_dkv_kernel<T><<<(unsigned)g2, 256, 0, st>>>((T*)dk, (T*)dv, (const T*)q_qk, (const T*)q_acc,
+                                                            (const T*)k_qk, (const T*)v_qk, (const T*)bias_t, keybias,
                                                             (const T*)do_qk, (const T*)do_acc, lse, dsum, (int)B2, (int)H,
                                                             (int)Nq, (int)Nk, dk_scale);
+    rc = ffk_check_launch("ffk_attention_bwd");
+    if (rc != FFK_OK || !dbias) return rc;
+    // enough slices of the batch rows for ~ 8 waves per SIMD, at least 8 rows per slice
+    const long tiles = H * QT * KT;
+    long ns = (8L * 1024 + tiles - 1) / tiles;
+    if (ns > (B2 + 7) / 8) ns = (B2 + 7) / 8;
+    if (ns < 1) ns = 1;
+    const long g3 = (ns * tiles + 3) / 4;
+    FFK_REQUIRE(g3 < (1L << 31), FFK_ERR_SHAPE, "ffk_attention_bwd: too many tiles for one launch");
+    attention_bwd_dbias_kernel<T><<<(unsigned)g3, 256, 0, st>>>(dbias, (const T*)q_qk, (const T*)k_qk, (const T*)v_qk,
+                                                              (const T*)bias_t, keybias, (const T*)do_qk, lse, dsum,
+                                                              (int)B2, (int)H, (int)Nq, (int)Nk, (int)ns);
     return ffk_check_launch("ffk_attention_bwd");
 }
 
@@ -288,13 +381,12 @@ int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* ds
 
 extern "C" int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk,
                                  const void* q_acc, const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
-                                 const void* bias_rm, const float* keybias, const void* do_qk, const void* do_acc,
+                                 const float* keybias, const void* do_qk, const void* do_acc,
                                  const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, float dq_scale,
                                  float dk_scale, int dtype, void* stream) {
     FFK_REQUIRE(dq && dk && dv && lse && dsum && q_qk && q_acc && k_qk && k_acc && v_qk && keybias && do_qk && do_acc && o_qk,
                 FFK_ERR_NULL, "ffk_attention_bwd: null pointer");
-    FFK_REQUIRE((bias_t != nullptr) == (bias_rm != nullptr) && (!dbias || bias_t), FFK_ERR_NULL,
-                "ffk_attention_bwd: bias_t and bias_rm go together, and dbias needs them");
+    FFK_REQUIRE(!dbias || bias_t, FFK_ERR_NULL, "ffk_attention_bwd: dbias needs bias_t");
     FFK_REQUIRE(B2 > 0 && B2 < 131072 && H > 0 && H < 65536 && Nq > 0 && Nk > 0 && Nq < (1 << 24) && Nk < (1 << 24),
                 FFK_ERR_SHAPE, "ffk_attention_bwd: bad shape B2=%ld H=%ld Nq=%ld Nk=%ld", (long)B2, (long)H, (long)Nq, (long)Nk);
     FFK_REQUIRE(ffk_aligned16(dq) && ffk_aligned16(dk) && ffk_aligned16(dv) && ffk_aligned16(lse) && ffk_aligned16(dsum) &&
@@ -305,10 +397,10 @@ extern "C" int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, flo
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
         case FFK_BF16:
-            return launch_bwd<bf16_t>(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, bias_rm, keybias,
+            return launch_bwd<bf16_t>(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias,
                                       do_qk, do_acc, o_qk, B2, H, Nq, Nk, dq_scale, dk_scale, st);
         case FFK_F32:
-            return launch_bwd<float>(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, bias_rm, keybias,
+            return launch_bwd<float>(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias,
                                      do_qk, do_acc, o_qk, B2, H, Nq, Nk, dq_scale, dk_scale, st);
         default: return ffk_fail(FFK_ERR_DTYPE, "ffk_attention_bwd: unsupported dtype tag %d", dtype);
     }

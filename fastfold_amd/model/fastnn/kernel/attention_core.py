@@ -71,13 +71,13 @@ def _attention_core_backward(q, k, v, mask, bias, out, dout, need_dbias):
     for i in range(b1):
         mk = mask[i].to(dt).contiguous() if mask is not None else torch.ones(b2, n, dtype=dt, device=dev)
         _lib.key_bias(kb, fl, mk, B=b2, N=n, mask_sb=n, mask_sn=1)
-        b2s = (bias[i].float() * _lib.LOG2E).to(dt).contiguous() if bias is not None else None
+        bt = layouts.tile_bias((bias[i].float() * _lib.LOG2E).to(dt)) if bias is not None else None
         do_ = dout[i].view(b2, n, h, d).permute(0, 2, 1, 3)          # [b2, h, n, d] views: re-tiled as they lie
         o_ = out[i].view(b2, n, h, d).permute(0, 2, 1, 3)
         _lib.attention_bwd(dq[i], dk[i], dv[i], None if dbias is None else dbias[i], lse, dsum,
                            _lib.tile_pack(q[i], QK, scale), _lib.tile_pack(q[i], ACC, scale),     # as the forward saw q
                            _lib.tile_pack(k[i], QK), _lib.tile_pack(k[i], ACC), _lib.tile_pack(v[i], QK),
-                           None if b2s is None else layouts.tile_bias(b2s), b2s, kb,
+                           bt, kb,
                            _lib.tile_pack(do_, QK), _lib.tile_pack(do_, ACC), _lib.tile_pack(o_, QK),
                            B2=b2, H=h, Nq=n, Nk=n, dq_scale=1.0 / math.sqrt(d), dk_scale=1.0 / _lib.LOG2E)
     if d != 32:

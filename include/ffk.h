@@ -284,19 +284,20 @@ int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v
  *   k_qk, k_acc : k, [B2][H][ceil(Nk/32)][1024] in FFK_TILE_QK and in FFK_TILE_V order
  *   v_qk        : v in FFK_TILE_QK order
  *   do_qk, do_acc, o_qk : do and the forward output, as [B2][H][Nq][32] tensors tiled like q
- *   bias_t      : bias * log2(e) in FFK_TILE_BIAS order, bias_rm : the same values row-major [H][Nq][Nk]; both or neither
+ *   bias_t      : bias * log2(e) in FFK_TILE_BIAS order, or NULL
  *   keybias     : as for ffk_attention_fwd
  *   lse, dsum   : fp32 scratch [B2][H][ceil(Nq/32)*32] (row log-sum-exp in the log2 domain and sum_d do.o; written by
  *                 the first kernel, read by the second)
- *   dq : [B2][H][Nq][32], dk, dv : [B2][H][Nk][32] (operand dtype);  dbias : fp32 [H][Nq][Nk], ZEROED by the caller,
- *                 accumulated over b2 with atomic adds (summation order not fixed), or NULL
+ *   dq : [B2][H][Nq][32], dk, dv : [B2][H][Nk][32] (operand dtype);  dbias : fp32 [H][Nq][Nk], ZEROED by the caller:
+ *                 a third kernel sums dS over slices of the batch rows in registers and adds each slice's sum with
+ *                 one atomic per element (summation order across slices not fixed), or NULL
  *   dq_scale = 1 / sqrt(d), dk_scale = 1 / log2(e): undo the factors folded into the q operand.
  * Rows whose keys are all masked get zero gradients (the forward pass gives them zero output).
  * Replaces: autograd through the matmul / fused_softmax / matmul chain of SelfAttention.forward
  * (fastfold/model/fastnn/ops.py:310-322; softmax backward kernels softmax_cuda_kernel.cu:252-334,524-614). */
 int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk,
                       const void* q_acc, const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
-                      const void* bias_rm, const float* keybias, const void* do_qk, const void* do_acc,
+                      const float* keybias, const void* do_qk, const void* do_acc,
                       const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, float dq_scale,
                       float dk_scale, int dtype, void* stream);
 
