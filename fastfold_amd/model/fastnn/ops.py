@@ -207,10 +207,11 @@ class Linear(nn.Linear, _PackMixin):
     def forward(self, input, act=_lib.FFK_ACT_NONE):
         F_.check_cuda(input)
         if _needs_grad(self, input):
-            if act != _lib.FFK_ACT_NONE:
-                raise NotImplementedError("Linear: fused activations are forward-only")
-            return _LinearFn.apply(input, self.weight.to(input.dtype),
-                                   self.bias.to(input.dtype) if self.use_bias else None)
+            y = _LinearFn.apply(input, self.weight.to(input.dtype),
+                                self.bias.to(input.dtype) if self.use_bias else None)
+            if act == _lib.FFK_ACT_RELU:
+                return torch.relu(y)
+            return torch.sigmoid(y) if act == _lib.FFK_ACT_SIGMOID else y
         w, b = self._pk(input.dtype, input.device)
         x2 = input.reshape(-1, self.in_features)
         kp = self._kpad()

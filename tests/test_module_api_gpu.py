@@ -232,6 +232,8 @@ def test_forward_only_guard(dev):
     assert y.grad_fn is not None
     y.sum().backward()
     assert torch.allclose(x.grad, lin.weight.sum(0).expand(4, 64), atol=1e-5)
+    from fastfold_amd import _lib
+    assert torch.equal(lin(x, act=_lib.FFK_ACT_RELU), torch.relu(y))      # the fused activations, differentiably
     with torch.no_grad():
         assert not lin(x).requires_grad
         assert torch.allclose(lin(x), y, atol=1e-5)
