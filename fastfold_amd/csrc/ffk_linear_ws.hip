@@ -48,6 +48,7 @@ struct WsPlan {
     int row_perm;                // 1: rows of a group are read through tau (launch has channel-major tiles)
     int mask_tile;               // first tile with a row mask (all masked tiles share its mask), -1 = none
     int max_slots;               // largest number of slots any wave holds
+    int resid_a2;                // 1: every residual is the second operand itself (same rows): taken from its LDS slab
 };
 
 struct WsArgs {
@@ -482,14 +483,23 @@ __device__ __forceinline__ void ws_store_cols(const WsSlot& t, const f32x16& acc
 template <bool XT>
 __device__ __forceinline__ void ws_store_rows_folded(const WsSlot& t, const f32x16& acc, const f32x16& accg, const float* sb,
                                                      const float* sc1, float rstd, float nmr, float rstd_g, float nmr_g,
-                                                     bool valid, unsigned hi, unsigned lo, int half) {
+                                                     bool valid, unsigned hi, unsigned lo, int half,
+                                                     const unsigned char* a2row, int a2vec, int a2swz) {
     // rstd_g / nmr_g (the second operand's statistics) arrive multiplied by -log2(e), as the gate's bias table is
+    // a2row: this lane's row of the second operand's LDS slab when that operand is also the residual (the triangle
+    // multiplication's output stage: gate input and residual are both z), else nullptr; a2vec: the 16-byte vector
+    // of the row this lane's 16 channels start at; a2swz: the row's swizzle (vector v lives at v ^ a2swz)
     const int cl = 16 * half;
     const long off = (long)hi * t.s_o + (long)lo * t.s_i + cl;
     u32x4 rv[2];
     if (t.resid) {
-        rv[0] = *reinterpret_cast<const u32x4*>(t.resid + off);
-        rv[1] = *reinterpret_cast<const u32x4*>(t.resid + off + 8);
+        if (a2row) {
+            rv[0] = *reinterpret_cast<const u32x4*>(a2row + ((a2vec ^ a2swz) << 4));
+            rv[1] = *reinterpret_cast<const u32x4*>(a2row + (((a2vec + 1) ^ a2swz) << 4));
+        } else {
+            rv[0] = *reinterpret_cast<const u32x4*>(t.resid + off);
+            rv[1] = *reinterpret_cast<const u32x4*>(t.resid + off + 8);
+        }
     }
     if (XT && t.xtail) {       // extended residual stream: the update is added at 24 bits, eight channels at a time
         const u32x4 tv = *reinterpret_cast<const u32x4*>(t.xtail + off);
@@ -987,8 +997,14 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                             su2 += lane_xor<32>(su2);
                             const float mean_g = su1 * (1.0f / WS_K);
                             const float rstd_g = -1.4426950408889634f * rsqrtf(fmaxf(su2 * (1.0f / WS_K) - mean_g * mean_g, 0.0f) + d.ln_eps);
+                            const unsigned char* a2r = nullptr;
+                            int a2v = 0;
+                            if (args.plan.resid_a2 && t.resid) {
+                                a2r = s_a2 + buf * (WS_BM * 256) + (rg * 32 + n32) * 256;
+                                a2v = (int)(t.resid - (const T*)d.a2) / 8 + 2 * half;
+                            }
                             ws_store_rows_folded<XT>(t, acc, accg, sb, s_c1 + s_wrow[s], rstd, -rstd * mean, rstd_g, -rstd_g * mean_g,
-                                                 valid, c_hi, c_lo, half);
+                                                 valid, c_hi, c_lo, half, a2r, a2v, n32 & 15);
                         } else if (ALLOW_GLU && glu) ws_store_rows_compact<true, XT>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                         else ws_store_rows_compact<false, XT>(t, acc, accg, sb, valid, mc, c_hi, c_lo, rmask, half);
                     } else {
@@ -1160,16 +1176,24 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     }
     args.plan.row_perm = chan_major ? 1 : 0;
     args.plan.mask_tile = mask_tile;
+    args.plan.resid_a2 = 0;
     args.d = *d;
     if (d->a2) {
         // second operand: every unit must be a GLU unit stored [row][channel], first operand channel-major
         if (!d->a_chanmajor || args.plan.max_slots > 2 || mask_tile >= 0 || d->a2_si % 8 || d->a2_so % 8) return 0;
+        bool resid_a2 = true;
         for (int i = 0; i < d->n_tiles; ++i) {
             const ffk_tile& t = d->tiles[i];
             if (!t.glu || !ws_by_rows(t)) return 0;
             // plain residual GLU tiles of 64 channels only
             if (t.kind != FFK_TILE_STRIDED || t.gate || t.rowmask || t.scale != 1.0f || t.ncols != 64) return 0;
+            // the residual is the second operand itself: same rows, channels [c0, c0 + 64) of its 128
+            const long c0 = (const T*)t.resid - (const T*)d->a2;
+            if (!t.resid || c0 < 0 || c0 + t.ncols > 128 || c0 % 32 || t.s_o != d->a2_so || t.s_i != d->a2_si ||
+                t.inner != d->a2_inner || t.s_h != 32 || t.s_d != 1)
+                resid_a2 = false;
         }
+        args.plan.resid_a2 = resid_a2 ? 1 : 0;
         *status = tails ? ws_launch<2, 128, true, true, true>(args, st) : ws_launch<2, 128, true, true>(args, st);
     } else if (tails) {
         // residual tails: built for the output projections of the attentions (one plain tile group, two slots)
