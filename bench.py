@@ -308,6 +308,8 @@ def main():
                     help="time only the extra-MSA and template pair stacks (for profiling them on their own)")
     ap.add_argument("--no-long-sequence", action="store_true",
                     help="skip the block at N_res = 4096 (a few seconds and about 30 GB of device memory)")
+    ap.add_argument("--forward-backward", action="store_true",
+                    help="also time the differentiable path the way benchmark/perf.py does (training-mode blocks, N_res = 256)")
     ap.add_argument("--plain-residual", action="store_true",
                     help="A/B switch: the reference's plain bf16 residual stream instead of the extended one")
     args = ap.parse_args()
@@ -432,9 +434,10 @@ def main():
     if not args.no_long_sequence and args.workload == "cfg4":
         line["long_sequence"] = long_sequence(dev)
         torch.cuda.empty_cache()
-    if not args.no_micro:
+    if args.forward_backward:
         line["forward_backward"] = forward_backward(dev)
         torch.cuda.empty_cache()
+    if not args.no_micro:
         line["feeders"] = feeder_stacks(dev, r)
         line["ops"] = micro_ops(dev)
     if not args.no_cpu:
