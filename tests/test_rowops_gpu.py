@@ -95,6 +95,35 @@ def test_layernorm_backward(dev):
     assert (ln.bias.grad - ref.bias.grad).abs().max().item() < 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(65, 64), (1000, 128), (37, 256), (4096 + 3, 384), (513, 512), (70, 1024),
+                                       (33, 2048), (40, 72)])
+def test_layernorm_backward_shapes(dev, dtype, rows, cols):
+    """Both backward kernels (the vector form for rows of exactly lanes x vectors x 16 bytes up to 1024 elements, the
+    general one otherwise) against float64 autograd of torch's layer_norm on the same rounded inputs; row counts that
+    leave ragged row groups, enough rows for several grid-stride passes."""
+    from fastfold_amd.model.fastnn.kernel import LayerNorm
+    g = torch.Generator().manual_seed(rows + cols)
+    x = torch.randn(rows, cols, generator=g).to(dev, dtype)
+    dy = torch.randn(rows, cols, generator=g).to(dev, dtype)
+    ln = LayerNorm(cols).to(dev, dtype)
+    with torch.no_grad():
+        ln.weight.copy_(1 + 0.2 * torch.randn(cols, generator=g))
+        ln.bias.copy_(0.1 * torch.randn(cols, generator=g))
+    xa = x.clone().requires_grad_(True)
+    ln(xa).backward(dy)
+    xr = x.double().cpu().requires_grad_(True)
+    wr, br = ln.weight.detach().double().cpu().requires_grad_(True), ln.bias.detach().double().cpu().requires_grad_(True)
+    torch.nn.functional.layer_norm(xr, (cols,), wr, br, ln.eps).backward(dy.double().cpu())
+    tol = 1e-5 if dtype == torch.float32 else (1.5e-2 if dtype == torch.bfloat16 else 2e-3)
+
+    def rel(a, b):
+        return float((a.double().cpu() - b).abs().max() / b.abs().max())
+    assert rel(xa.grad, xr.grad) <= tol, rel(xa.grad, xr.grad)
+    assert rel(ln.weight.grad, wr.grad) <= tol, rel(ln.weight.grad, wr.grad)
+    assert rel(ln.bias.grad, br.grad) <= tol, rel(ln.bias.grad, br.grad)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("C", [128, 36, 7])
 def test_elementwise_fusions(dev, dtype, C):
