@@ -225,7 +225,8 @@ def _torch_attention_core(q, k, v, mask, bias):
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
 @pytest.mark.parametrize("b1,b2,h,n,d,use_bias", [(1, 3, 4, 77, 32, True), (2, 2, 8, 64, 32, True), (1, 2, 4, 130, 32, False),
-                                                  (1, 2, 4, 50, 16, True), (1, 3, 8, 40, 8, True)])
+                                                  (1, 2, 4, 50, 16, True), (1, 3, 8, 40, 8, True),
+                                                  (1, 43, 4, 70, 32, True)])      # several batch-row slices in the dbias kernel
 def test_fused_attention_core_backward(dev, dtype, tol, b1, b2, h, n, d, use_bias):
     """dq, dk, dv, dbias of the exported op (``ffk_attention_bwd``: logits recomputed tile by tile) against torch
     autograd of the reference's formula in float64, with masked keys, a ragged last tile and the narrow heads."""
