@@ -49,6 +49,8 @@ struct WsPlan {
     int mask_tile;               // first tile with a row mask (all masked tiles share its mask), -1 = none
     int max_slots;               // largest number of slots any wave holds
     int resid_a2;                // 1: every residual is the second operand itself (same rows): taken from its LDS slab
+    int bias_tile;               // index of a trailing FFK_TILE_BIAS tile (<= 4 heads, K = 128), -1 = none: it takes no
+                                 // weight slot - its few dot products per row run on the vector pipe from the slab in LDS
 };
 
 struct WsArgs {
@@ -583,6 +585,8 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     T* s_ln2 = reinterpret_cast<T*>(s_cmln + (CM ? 256 : 0));                               // DUAL: gamma2[128], beta2[128]
     T* s_ln1 = s_ln2 + (DUAL ? 256 : 0);                                                    // !CM: gamma[K], beta[K]
     float* s_c1 = reinterpret_cast<float*>(s_ln1 + (CM ? 0 : 2 * WS_K));                    // DUAL: folded LayerNorm row sums
+    constexpr bool PB = !CM && !DUAL && !XT && WS_K == 128;    // variants that take a trailing pair-bias tile
+    T* s_wb = reinterpret_cast<T*>(s_c1);                                                   // PB: [4][WS_K] head weights
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
@@ -804,6 +808,12 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         }
     };
 
+    const int pb_tile = PB ? args.plan.bias_tile : -1;
+    if (PB && pb_tile >= 0) {
+        const int heads = d.tiles[pb_tile].ncols;
+        for (int i = tid; i < 4 * WS_K; i += WS_THREADS)
+            s_wb[i] = (i / WS_K) < heads ? W[(long)(pb_tile * 128 + i / WS_K) * WS_K + (i % WS_K)] : (T)0.0f;
+    }
     const int nslabs = (M + WS_BM - 1) / WS_BM;
     int slab = blockIdx.x;                               // grid <= nslabs
     fetch(slab, 0);
@@ -814,6 +824,32 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         const int nxt = slab + (int)gridDim.x < nslabs ? slab + (int)gridDim.x : slab;
         fetch(nxt, buf ^ 1);                             // in flight during the products below
         const unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
+        if (PB && pb_tile >= 0) {
+            // pair bias of this slab: thread -> (row tid / 4, head tid % 4); the row is the operand as the products
+            // see it (normalised, rounded to bf16), so the value equals a fifth output column group of four channels
+            const ffk_tile& tb = d.tiles[pb_tile];
+            const int prow = tid >> 2, hd = tid & 3;
+            const long pm = (long)slab * WS_BM + prow;
+            if (pm < M && hd < tb.ncols) {
+                typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                const unsigned char* xr = sa + prow * WS_AP;
+                const T* wr = s_wb + hd * WS_K;
+                float acc = 0.0f;
+#pragma unroll
+                for (int c8 = 0; c8 < WS_K / 8; ++c8) {
+                    const bf16x8 xv = *reinterpret_cast<const bf16x8*>(xr + c8 * 16);
+                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(wr + c8 * 8);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const bf16x2 xp = {xv[2 * e], xv[2 * e + 1]}, wp = {wv[2 * e], wv[2 * e + 1]};
+                        acc = __builtin_amdgcn_fdot2_f32_bf16(xp, wp, acc, false);
+                    }
+                }
+                const unsigned hi = (unsigned)pm / (unsigned)tb.inner, lo = (unsigned)pm - hi * (unsigned)tb.inner;
+                ((T*)tb.out)[(long)hd * tb.s_h + (long)(hi >> 5) * tb.s_o + (long)(lo >> 5) * 1024 +
+                             qk_tile_off((int)(lo & 31), (int)(hi & 31))] = (T)(acc * tb.scale);
+            }
+        }
         for (int rg = rg_first; rg < WS_RG; rg += rg_step) {
             const long m0g = (long)slab * WS_BM + rg * 32;
             if (m0g >= M) break;
@@ -1124,7 +1160,8 @@ int ws_launch(const WsArgs& args, hipStream_t st) {
     constexpr int WS_BM = WsGeo<K>::BM;
     const size_t smem = 2 * (size_t)WS_BM * WsGeo<K>::AP + 2 * WS_BM * sizeof(float) + FFK_MAX_TILES * 128 * sizeof(float) +
                         (DUAL ? 2 * (size_t)WS_BM * 256 + 256 * sizeof(T) + FFK_MAX_TILES * 128 * sizeof(float) : 0) +
-                        (CM ? 256 * sizeof(float) : 2 * K * sizeof(T));
+                        (CM ? 256 * sizeof(float) : 2 * K * sizeof(T)) +
+                        (!CM && !DUAL && !XT && K == 128 ? 4 * K * sizeof(T) : 0);      // head weights of a pair-bias tile
     static FfkLdsReservation lds_reserved;
     {
         const int rc_lds = ffk_reserve_lds(lds_reserved, (const void*)linear_ws_kernel<NS, K, CM, DUAL, XT>, smem, "ffk_fused_linear");
@@ -1149,8 +1186,20 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (d->variant == FFK_LINEAR_STAGED) return 0;
     bool chan_major = false, v_tiles = false, tails = false;
     int mask_tile = -1;
-    for (int i = 0; i < d->n_tiles; ++i) {
+    // a trailing pair-bias tile (score-operand tiles of <= 4 heads) rides on the launch without a weight slot
+    int n_slot_tiles = d->n_tiles, bias_tile = -1;
+    if (d->n_tiles >= 2 && d->tiles[d->n_tiles - 1].kind == FFK_TILE_BIAS) {
+        const ffk_tile& t = d->tiles[d->n_tiles - 1];
+        auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+        if (d->K != 128 || d->a_chanmajor || d->a2 || t.ncols < 1 || t.ncols > 4 || t.bias || t.resid || t.gate || t.rowmask ||
+            t.xtail || t.glu || t.act != FFK_ACT_NONE || t.inner <= 0 || !t.out || !al16(t.out))
+            return 0;
+        bias_tile = d->n_tiles - 1;
+        n_slot_tiles = d->n_tiles - 1;
+    }
+    for (int i = 0; i < n_slot_tiles; ++i) {
         const ffk_tile& t = d->tiles[i];
+        if (t.kind == FFK_TILE_BIAS) return 0;
         if (!ws_tile_ok(*d, t)) return 0;
         tails = tails || t.xtail != nullptr;
         chan_major = chan_major || (!ws_by_rows(t) && t.kind == FFK_TILE_STRIDED);
@@ -1167,9 +1216,14 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     if (chan_major && v_tiles) return 0;          // they need different row orders within a group
     WsArgs args;
     const bool k64 = d->K == 64;
-    if (!ws_make_plan(*d, args.plan, k256 ? WsGeo<256>::RG : (k64 ? WsGeo<64>::RG : WsGeo<128>::RG),
-                      k256 ? 2 : (k64 ? 4 : 3)))
-        return 0;
+    {
+        ffk_linear_desc slots = *d;                   // the plan covers the tiles that take weight slots
+        slots.n_tiles = n_slot_tiles;
+        if (!ws_make_plan(slots, args.plan, k256 ? WsGeo<256>::RG : (k64 ? WsGeo<64>::RG : WsGeo<128>::RG),
+                          k256 ? 2 : (k64 ? 4 : 3)))
+            return 0;
+    }
+    if (bias_tile >= 0 && (tails || chan_major)) return 0;   // built into the plain K = 128 variants only
     if (k256) {
         for (int i = 0; i < d->n_tiles; ++i)
             if (d->tiles[i].glu) return 0;                   // GLU units are only built for K = 128
@@ -1177,6 +1231,7 @@ int ffk_linear_ws_try(const ffk_linear_desc* d, hipStream_t st, int* status) {
     args.plan.row_perm = chan_major ? 1 : 0;
     args.plan.mask_tile = mask_tile;
     args.plan.resid_a2 = 0;
+    args.plan.bias_tile = bias_tile;
     args.d = *d;
     if (d->a2) {
         // second operand: every unit must be a GLU unit stored [row][channel], first operand channel-major

@@ -231,15 +231,21 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     if bias_in_launch:
         bias_tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H,
                               scale=LOG2E)
-    # The skinny bias projection has its own pass over x.  It goes first: x was written by the launch before
+    # With 128 input channels, at most four heads and all rows in one slab the bias rides on the projection launch:
+    # the weights-stationary kernel computes its four dot products per row on the vector pipe from the rows it
+    # has in LDS anyway (one read of x less than a pass of its own; -0.05 ms per triangle attention at N = 1024).
+    rides = bias_tile is not None and acc_order and C == 128 and H <= 4 and slab >= B2 and _PAIR_BIAS_RIDES
+    # Otherwise the skinny bias projection has its own pass over x.  It goes first: x was written by the launch before
     # this call and is still (partly) cache-resident, and the bias pass writes little, so the projection after
     # it finds x as warm as before - the other way round the projection's output (four times the size of x)
     # has pushed x out by the time the bias pass reads it (measured: -0.65 % block time at N = 1024).
-    if bias_tile is not None and acc_order and C in (64, 128):
+    if rides:
+        pass
+    elif bias_tile is not None and acc_order and C in (64, 128):
         _pair_bias_launch(bias_t, x, ln, w_pk[4 * tpg * 128:], pb_scratch, N=N, C=C, H=H, a_inner=a_inner,
                           a_so=a_so, a_si=a_si, scale=LOG2E)
         bias_tile = None
-    if bias_tile is not None and (acc_order or slab < B2):     # its own launch over all rows, before x changes
+    if bias_tile is not None and not rides and (acc_order or slab < B2):     # its own launch over all rows, before x changes
         _lib.fused_linear(x, w_pk, [bias_tile], M=M, K=C, a_inner=a_inner, a_so=a_so, a_si=a_si, ln=ln,
                           w_row_off=4 * tpg * 128)
         bias_tile = None
@@ -353,6 +359,7 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
 # the projection kernel - one channel each - all land in the same memory channel; 128 bytes of padding spread them
 # (block 6.97 -> 6.885 ms in a same-box A/B at N_res = 1024; 64, 192 and 1088 elements measure the same).
 _TRIMUL_CHAN_PAD = 64
+_PAIR_BIAS_RIDES = True      # see attention(): switch for same-box comparisons
 
 
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,

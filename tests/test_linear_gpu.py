@@ -183,6 +183,46 @@ def test_bias_tiles(dev, dtype, r, H):
         assert _rel(_np(layouts.untile_bias(bt, r, r)), ref) < TOL[dtype]
 
 
+@pytest.mark.parametrize("r,H", [(45, 4), (64, 3), (33, 1)])
+def test_bias_tile_rides_on_a_projection_launch(dev, r, H):
+    """A trailing FFK_TILE_BIAS tile in a launch of the weights-stationary kernel (bf16, K = 128, <= 4 heads): computed
+    on the vector pipe from the slab rows, no weight slot.  Checked against numpy, against the staged kernels on the
+    same descriptor, in both traversal orders; the other tile of the launch is unaffected and the padding of ragged
+    bias tiles stays zero."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    dtype, C = torch.bfloat16, 128
+    g = torch.Generator().manual_seed(r * 7 + H)
+    z = (torch.randn(r, r, C, generator=g) * 1.3 + 0.2).to(dev, dtype)
+    w = (torch.randn(128, C, generator=g) / C ** 0.5).to(dev, dtype)
+    wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dev, dtype)
+    gam = (1 + 0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    bet = (0.1 * torch.randn(C, generator=g)).to(dev, dtype)
+    wpk = torch.cat([_pack(w, 1), _pack(wb, 1)]).contiguous()
+    T = layouts.n_tiles(r)
+    for transposed in (False, True):
+        res = []
+        for staged in (False, True):
+            y = torch.zeros(r * r, 128, dtype=dtype, device=dev)
+            bt = torch.zeros(H, T, T, 2, 32, 16, dtype=dtype, device=dev)
+            tiles = [_lib.make_tile(y, inner=r * r, s_i=128),
+                     _lib.make_tile(bt, kind=_lib.FFK_TILE_BIAS, inner=r, s_o=T * 1024, s_h=T * T * 1024, ncols=H,
+                                    scale=_lib.LOG2E)]
+            kw = dict(a_inner=r, a_so=C, a_si=r * C) if transposed else {}
+            _lib.fused_linear(z, wpk, tiles, M=r * r, K=C, ln=(gam, bet), staged=staged, **kw)
+            res.append((y, bt))
+        zz = _np(z).transpose(1, 0, 2) if transposed else _np(z)
+        x = _np(torch.from_numpy(ops_np.layer_norm(zz, _np(gam), _np(bet))).to(dtype))
+        ref = (ops_np.linear(x, _np(wb)) * _lib.LOG2E).transpose(2, 0, 1)       # [h, q, k]
+        for y, bt in res:
+            assert _rel(_np(layouts.untile_bias(bt, r, r)), ref) < 1e-2
+            assert _rel(_np(y), ops_np.linear(x, _np(w)).reshape(r * r, 128)) < TOL[dtype]
+            full = _np(layouts.untile_bias(bt, T * 32, T * 32))
+            assert np.abs(full[:, r:, :]).max(initial=0.0) == 0.0 and np.abs(full[:, :, r:]).max(initial=0.0) == 0.0
+        assert _rel(_np(res[0][1]), _np(res[1][1])) < 1e-2
+        assert torch.equal(res[0][0], res[1][0]) or _rel(_np(res[0][0]), _np(res[1][0])) < 1e-2
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("C,with_ln", [(128, True), (64, True), (64, False)])
 @pytest.mark.parametrize("r", [40, 27, 104])
