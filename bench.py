@@ -33,7 +33,7 @@ WORKLOADS = {
                  attn_traffic=None),
     "cfg4": dict(n_seq=128, n_res=1024, tail=0.05,
                  name="configs[3]: 48-block stack bf16 N_seq=128 N_res=1024, last 5% of residues masked",
-                 attn_traffic=1.568e9),
+                 attn_traffic=1.642e9),
 }
 
 
