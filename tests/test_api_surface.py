@@ -54,3 +54,26 @@ def test_fastfold_alias_is_opt_in():
         "print('ok')\n")
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.strip() == "ok", out.stderr
+
+
+def test_slab_weight_gradient_on_cpu():
+    """``_weight_grad`` (the differentiable Linear's dW): bf16 activations with many rows are reduced slab by slab through
+    a batched GEMM and summed in fp32; other inputs take the plain product.  Both against float64."""
+    from fastfold_amd.model.fastnn.ops import _LinearFn, _weight_grad
+    g = torch.Generator().manual_seed(0)
+    dy = torch.randn(32768, 24, generator=g)
+    x = torch.randn(32768, 40, generator=g)
+    ref = dy.double().t() @ x.double()
+    assert torch.allclose(_weight_grad(dy, x).double(), ref, rtol=1e-4, atol=1e-2)            # fp32: plain product
+    got = _weight_grad(dy.bfloat16(), x.bfloat16())                                            # 8 slabs of 4096 rows
+    assert got.dtype == torch.bfloat16
+    ref16 = dy.bfloat16().double().t() @ x.bfloat16().double()
+    assert float((got.double() - ref16).norm() / ref16.norm()) < 1e-2
+    odd = _weight_grad(dy[:4099].bfloat16(), x[:4099].bfloat16())                              # no even split: plain
+    assert float((odd.double() - dy[:4099].bfloat16().double().t() @ x[:4099].bfloat16().double()).norm()) < 5.0
+    # the autograd function against float64 autograd of F.linear
+    xi = torch.randn(3, 7, 10, generator=g, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(5, 10, generator=g, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(5, generator=g, dtype=torch.float64, requires_grad=True)
+    assert torch.autograd.gradcheck(_LinearFn.apply, (xi, w, b))
+    assert torch.autograd.gradcheck(lambda a, c: _LinearFn.apply(a, c, None), (xi, w))
