@@ -145,9 +145,14 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
 
     f32x16 acc2[G::CT];                                    // out^T tiles: channels 32 ct + 16 half + v, row l32
 #pragma unroll
-    for (int c = 0; c < G::CT; ++c)
+    for (int c = 0; c < G::CT; ++c) {                      // start from b2: the epilogue has no bias to add
+        const Vec16<T> b0 = ld16(b2 + c * 32 + 16 * half), b1v = ld16(b2 + c * 32 + 16 * half + 8);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc2[c][v] = 0.0f;
+        for (int v = 0; v < 8; ++v) {
+            acc2[c][v] = (float)b0.e[v];
+            acc2[c][8 + v] = (float)b1v.e[v];
+        }
+    }
 
     // W1 fragment of hidden tile 0: row l32, column 2 ks + half.  The swizzle touches the low four column bits only,
     // so K steps 8 .. 15 (C = 256) are the first eight plus 256 bytes.
@@ -186,13 +191,18 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
             // one packed integer max per pair replaces one clamp per value (rounding is monotonic: same bits)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                bf16x8 r;
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                typedef short s16x2 __attribute__((ext_vector_type(2)));
+                const s16x2 zero = {0, 0};
+                u32x4 w;
 #pragma unroll
-                for (int t = 0; t < 8; ++t) r[t] = (T)h[8 * j + t];
-                typedef short s16x8 __attribute__((ext_vector_type(8)));
-                const s16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-                const s16x8 c = __builtin_elementwise_max(__builtin_bit_cast(s16x8, r), zero);
-                hf[ht][j] = __builtin_bit_cast(bf16x8, c);
+                for (int t = 0; t < 4; ++t) {              // one packed conversion and one packed max per pair
+                    const f32x2 pr = {h[8 * j + 2 * t], h[8 * j + 2 * t + 1]};
+                    const bf16x2 r = __builtin_convertvector(pr, bf16x2);
+                    w[t] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2, r), zero));
+                }
+                hf[ht][j] = __builtin_bit_cast(bf16x8, w);
             }
         }
 #pragma unroll
@@ -212,16 +222,14 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
     for (int c = 0; c < G::CT; ++c) {
         const int ch = c * 32 + 16 * half;
         const long o = rc * TR_C + ch;
-        u32x4 bv[2], rv[2];
-        bv[0] = *reinterpret_cast<const u32x4*>(b2 + ch);
-        bv[1] = *reinterpret_cast<const u32x4*>(b2 + ch + 8);
+        u32x4 rv[2];
         rv[0] = *reinterpret_cast<const u32x4*>(x + o);
         rv[1] = *reinterpret_cast<const u32x4*>(x + o + 8);
         if (xtail) {           // extended residual stream: the update is added at 24 bits
             const u32x4 tv = *reinterpret_cast<const u32x4*>(xtail + o);
             float upd[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) upd[v] = (float)(T)(acc2[c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7]);
+            for (int v = 0; v < 16; ++v) upd[v] = (float)(T)acc2[c][v];
             u32x4 h0, h1, tn;
             xs_update16(upd, rv[0], rv[1], tv, h0, h1, tn);
             if (ok) {
@@ -234,8 +242,7 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
         T y[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const float u = acc2[c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7];
-            y[v] = (T)((float)(T)u + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7]);
+            y[v] = (T)((float)(T)acc2[c][v] + (float)reinterpret_cast<const T*>(&rv[v >> 3])[v & 7]);
         }
         if (ok) {
             *reinterpret_cast<u32x4*>(out + o) = *reinterpret_cast<const u32x4*>(&y[0]);
