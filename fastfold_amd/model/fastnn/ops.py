@@ -100,7 +100,7 @@ def _weight_grad(dy2, x2):
         S *= 2
     if S == 1 or dy2.dtype == torch.float32:
         return dy2.t() @ x2
-    part = torch.bmm(dy2.view(S, M // S, -1).transpose(1, 2), x2.view(S, M // S, -1))
+    part = torch.bmm(dy2.reshape(S, M // S, -1).transpose(1, 2), x2.reshape(S, M // S, -1))
     return part.sum(0, dtype=torch.float32).to(dy2.dtype)
 
 
