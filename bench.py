@@ -24,17 +24,39 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
 
-# "attn_traffic": HBM bytes per launch of the biased attention kernel, averaged over the launches the
-# roofline object covers (2 triangle : 1 MSA-row per block).  It comes from rocprofv3 --pmc FETCH_SIZE
-# and WRITE_SIZE runs of this script (profiles/evoformer_blocks_cfg4_hbm_traffic.txt: counters scaled by
-# 2.0 / 1.0 after calibration on a plain streaming kernel); counters cannot be read inside a timed run.
 WORKLOADS = {
     "cfg3": dict(n_seq=128, n_res=256, tail=0.0, name="configs[2]: 48-block stack bf16 N_seq=128 N_res=256",
-                 attn_traffic=None),
+                 traffic_profile=None),
     "cfg4": dict(n_seq=128, n_res=1024, tail=0.05,
                  name="configs[3]: 48-block stack bf16 N_seq=128 N_res=1024, last 5% of residues masked",
-                 attn_traffic=1.642e9),
+                 traffic_profile="profiles/evoformer_blocks_cfg4_hbm_traffic.txt"),
 }
+
+
+def attention_traffic(profile):
+    """HBM bytes per launch of the biased attention kernel, averaged over the launches the roofline object covers
+    (triangle and MSA-row attention, weighted by their launch counts).  Hardware counters cannot be read inside a
+    timed run: the figure is taken from the committed summary of the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+    of this script (rows ``attention_kernel<bf16, true>  workgroups  n  read MB  written MB`` of its table, already
+    scaled by the calibration the file states); None when the file or its rows are missing."""
+    if profile is None:
+        return None
+    try:
+        lines = open(os.path.join(ROOT, profile)).read().splitlines()
+    except OSError:
+        return None
+    tot, n = 0.0, 0
+    for ln in lines:
+        if not ln.startswith("attention_kernel<bf16, true>"):
+            continue
+        f = ln.split(">", 1)[1].split()
+        try:
+            launches, rd, wr = int(f[1]), float(f[2]), float(f[3])
+        except (IndexError, ValueError):
+            continue
+        tot += launches * (rd + wr) * 1e6
+        n += launches
+    return round(tot / n) if n else None
 
 
 def block_gflop(s, r, c_m=256, c_z=128, hm=8, hz=4, d=32, c_opm=32, c_mul=128, n=4):
@@ -308,8 +330,8 @@ def main():
                     help="time only the extra-MSA and template pair stacks (for profiling them on their own)")
     ap.add_argument("--no-long-sequence", action="store_true",
                     help="skip the block at N_res = 4096 (a few seconds and about 30 GB of device memory)")
-    ap.add_argument("--forward-backward", action="store_true",
-                    help="also time the differentiable path the way benchmark/perf.py does (training-mode blocks, N_res = 256)")
+    ap.add_argument("--no-forward-backward", action="store_true",
+                    help="skip the differentiable path timed the way benchmark/perf.py does (training-mode blocks, N_res = 256)")
     ap.add_argument("--plain-residual", action="store_true",
                     help="A/B switch: the reference's plain bf16 residual stream instead of the extended one")
     args = ap.parse_args()
@@ -370,7 +392,7 @@ def main():
     ach = flops / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
     roofline = {"bound": "mfma", "kernel": "attention_kernel<bf16, bias> (ffk_attention_fwd)",
                 "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": wl["attn_traffic"],
+                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": attention_traffic(wl["traffic_profile"]),
                 "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, see profiles/)",
                 "launches": n, "avg_launch_ms": round(ms / max(n, 1), 4),
                 "flops_per_launch_avg": round(flops / max(n, 1) / 1e9, 2)}
@@ -434,7 +456,7 @@ def main():
     if not args.no_long_sequence and args.workload == "cfg4":
         line["long_sequence"] = long_sequence(dev)
         torch.cuda.empty_cache()
-    if args.forward_backward:
+    if not args.no_forward_backward and not args.no_micro:
         line["forward_backward"] = forward_backward(dev)
         torch.cuda.empty_cache()
     if not args.no_micro:

@@ -231,7 +231,7 @@ class BgemmDesc(ctypes.Structure):
 
 
 SIGNATURES["ffk_bgemm_nt"] = [ctypes.POINTER(BgemmDesc), _P]
-SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P]
+SIGNATURES["ffk_attention_fwd"] = [_P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _I, _I, _P]
 SIGNATURES["ffk_key_bias"] = [_P, _P, _P, _L, _L, _L, _L, _I, _P]
 
 
@@ -257,19 +257,19 @@ def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, i
 FFK_ATT_GATE_TILED = 1
 
 
-def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H, Nq, Nk, gate_tiled=False):
+def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H, Nq, Nk, D=32, gate_tiled=False):
     call("ffk_attention_fwd", ptr(out), ptr(q_t), ptr(k_t), ptr(v_t), ptr(bias_t), ptr(keybias), ptr(tileflags),
          ptr(gate),
-         B2, H, Nq, Nk, FFK_ATT_GATE_TILED if gate_tiled else 0, dtype_tag(q_t.dtype), stream_ptr())
+         B2, H, Nq, Nk, D, FFK_ATT_GATE_TILED if gate_tiled else 0, dtype_tag(q_t.dtype), stream_ptr())
 
 
-SIGNATURES["ffk_attention_bwd"] = [_P] * 16 + [_L, _L, _L, _L, _F, _F, _I, _P]
+SIGNATURES["ffk_attention_bwd"] = [_P] * 16 + [_L, _L, _L, _L, _L, _F, _F, _I, _P]
 
 
 def attention_bwd(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias, do_qk, do_acc,
-                  o_qk, *, B2, H, Nq, Nk, dq_scale, dk_scale):
+                  o_qk, *, B2, H, Nq, Nk, dq_scale, dk_scale, D=32):
     call("ffk_attention_bwd", ptr(dq), ptr(dk), ptr(dv), ptr(dbias), ptr(lse), ptr(dsum), ptr(q_qk), ptr(q_acc), ptr(k_qk),
-         ptr(k_acc), ptr(v_qk), ptr(bias_t), ptr(keybias), ptr(do_qk), ptr(do_acc), ptr(o_qk), B2, H, Nq, Nk,
+         ptr(k_acc), ptr(v_qk), ptr(bias_t), ptr(keybias), ptr(do_qk), ptr(do_acc), ptr(o_qk), B2, H, Nq, Nk, D,
          dq_scale, dk_scale, dtype_tag(q_qk.dtype), stream_ptr())
 
 
@@ -277,19 +277,23 @@ SIGNATURES["ffk_tile_pack"] = [_P, _P, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I, _
 
 
 def tile_pack(x, kind, scale=1.0):
-    """[B2, H, N, D <= 32] (any strides over the first three dims, channels contiguous) -> [B2, H, ceil(N/32), 1024]
-    operand tiles of the attention kernels in ``kind`` order (``FFK_TILE_QK`` / ``FFK_TILE_V``), times ``scale``."""
+    """[B2, H, N, D] (any strides over the first three dims, channels contiguous) -> operand tiles of the attention
+    kernels in ``kind`` order (``FFK_TILE_QK`` / ``FFK_TILE_V``), times ``scale``: [B2, H, ceil(N/32), 1024] for
+    D <= 32 (channels past D zero), [D/32, B2, H, ceil(N/32), 1024] - one block per 32-channel part of the head - for
+    D = 64 or 128."""
     import torch
-    if x.dim() != 4 or x.shape[-1] > 32:
-        raise RuntimeError("tile_pack: expected [B2, H, N, D <= 32], got %s" % (tuple(x.shape),))
+    if x.dim() != 4 or (x.shape[-1] > 32 and x.shape[-1] not in (64, 128)):
+        raise RuntimeError("tile_pack: expected [B2, H, N, D] with D <= 32, 64 or 128, got %s" % (tuple(x.shape),))
     if x.stride(-1) != 1:
         x = x.contiguous()
     B2, H, N, D = x.shape
-    out = torch.empty(B2, H, (N + 31) // 32, 1024, dtype=x.dtype, device=x.device)
+    parts = max(1, D // 32)
+    out = torch.empty(parts, B2, H, (N + 31) // 32, 1024, dtype=x.dtype, device=x.device)
     if out.numel():
-        call("ffk_tile_pack", ptr(out), ptr(x), B2, H, N, D, x.stride(0), x.stride(1), x.stride(2), float(scale), kind,
-             dtype_tag(x.dtype), stream_ptr())
-    return out
+        for p in range(parts):
+            call("ffk_tile_pack", ptr(out[p]), x.data_ptr() + p * 32 * x.element_size(), B2, H, N, min(D, 32),
+                 x.stride(0), x.stride(1), x.stride(2), float(scale), kind, dtype_tag(x.dtype), stream_ptr())
+    return out[0] if D <= 32 else out
 
 
 SIGNATURES["ffk_pair_bias"] = [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _F, _F, _I, _P]

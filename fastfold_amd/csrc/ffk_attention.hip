@@ -402,6 +402,130 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
     }
 }
 
+// Head dimensions 64 and 128 (the widths the reference's attention core also accepts; no module of the Evoformer
+// uses them): the head is cut into DP = D / 32 parts of 32 channels, each part an operand tile of its own
+// (part-major: part p of every tensor lies p * part elements behind part 0), so a score tile is the sum of DP
+// products and the output DP accumulator tiles.  One wave per (batch row, head, 32 queries), operands straight
+// from global memory, the classic running-maximum walk: this instantiation serves the stand-alone operator, not
+// the inference block, and is not tuned beyond that.
+template <typename T, int DP, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void attention_wide_kernel(
+    T* __restrict__ out, const T* __restrict__ q_t, const T* __restrict__ k_t, const T* __restrict__ v_t,
+    const T* __restrict__ bias_t, const float* __restrict__ keybias, const int* __restrict__ tileflags,
+    int B2, int H, int Nq, int Nk, long part_q, long part_k) {
+    typedef Mma<T> MM;
+    typedef typename MM::Frag Frag;
+    constexpr int NF = 16 / MM::KLANE;
+    constexpr float REF_FLOOR = -1.0e4f;          // rows whose every score lies below are all-masked: they give zeros
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
+    const long item = (long)blockIdx.x * 4 + wave;
+    if (item >= (long)B2 * H * QT) return;
+    const int qt = (int)(item % QT);
+    const long bh = item / QT;
+    const int h = (int)(bh % H), b2 = (int)(bh / H);
+
+    Ops16<T> qf[DP];
+#pragma unroll
+    for (int p = 0; p < DP; ++p) qf[p].load(q_t + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+    const float* mp = keybias + (long)b2 * KT * 32 + 4 * half;
+    const int* fl = tileflags + (long)b2 * KT;
+    Frag ident[NF];
+    if (HAS_BIAS) {
+#pragma unroll
+        for (int i = 0; i < NF; ++i) ident[i] = identity_frag<T>(i, l32, half);
+    }
+    f32x16 o_acc[DP];
+#pragma unroll
+    for (int p = 0; p < DP; ++p)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o_acc[p][v] = 0.0f;
+    float m_run = REF_FLOOR, l_run = 0.0f;
+    for (int kt = 0; kt < KT; ++kt) {
+        if (fl[kt] == 2) continue;                 // every key masked or padding: contributes exactly zero
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.0f;
+#pragma unroll
+        for (int p = 0; p < DP; ++p) {
+            Ops16<T> kc;
+            kc.load(k_t + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf[p].frag(i));
+        }
+        if (HAS_BIAS) {
+            Ops16<T> bc;
+            bc.load(bias_t + ((((long)h * QT + qt) * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(s, bc.frag(i), ident[i]);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 mk = *reinterpret_cast<const f32x4*>(mp + kt * 32 + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[4 * g + e] += mk[e];
+        }
+        float mt = fmaxf(s[0], s[1]);
+#pragma unroll
+        for (int v = 2; v < 16; ++v) mt = fmaxf(mt, s[v]);
+        mt = fmaxf(mt, lane_xor<32>(mt));
+        const float m_new = fmaxf(m_run, mt);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        float pr[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) pr[v] = fast_exp2(s[v] - m_new);
+        Frag pf[NF];
+        float tsum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+            pf[i] = PFrag<T>::make(pr + i * MM::KLANE);
+            tsum = PFrag<T>::add_sum(pf[i], tsum);
+        }
+        l_run = l_run * alpha + tsum;
+#pragma unroll
+        for (int p = 0; p < DP; ++p) {
+            Ops16<T> vc;
+            vc.load(v_t + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o_acc[p][v] *= alpha;
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(o_acc[p], vc.frag(i), pf[i]);
+        }
+    }
+    const float l_tot = l_run + lane_xor<32>(l_run);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    const int q = qt * 32 + l32;
+    if (q < Nq) {
+        T* o = out + ((long)b2 * Nq + q) * ((long)H * DP * 32) + (long)h * DP * 32 + 4 * half;
+#pragma unroll
+        for (int p = 0; p < DP; ++p)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[p * 32 + 8 * g + e] = DT<T>::from_f(o_acc[p][4 * g + e] * inv);
+    }
+}
+
+template <typename T, int DP>
+int launch_attention_wide(void* out, const void* q, const void* k, const void* v, const void* bias, const float* kb,
+                          const int* flags, long B2, long H, long Nq, long Nk, hipStream_t st) {
+    const long QT = (Nq + 31) / 32, KT = (Nk + 31) / 32;
+    const long grid = (B2 * H * QT + 3) / 4;
+    FFK_REQUIRE(grid < (1L << 31), FFK_ERR_SHAPE, "ffk_attention_fwd: too many tiles for one launch");
+    const long part_q = B2 * H * QT * 1024, part_k = B2 * H * KT * 1024;
+    if (bias)
+        attention_wide_kernel<T, DP, true><<<(unsigned)grid, 256, 0, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
+                                                                         (const T*)bias, kb, flags, (int)B2, (int)H,
+                                                                         (int)Nq, (int)Nk, part_q, part_k);
+    else
+        attention_wide_kernel<T, DP, false><<<(unsigned)grid, 256, 0, st>>>((T*)out, (const T*)q, (const T*)k, (const T*)v,
+                                                                          nullptr, kb, flags, (int)B2, (int)H, (int)Nq,
+                                                                          (int)Nk, part_q, part_k);
+    return ffk_check_launch("ffk_attention_fwd");
+}
+
 // One thread block per batch row: writes the additive key bias and, per 32-key tile, a flag
 // (0: all keys valid, 1: some masked / padding, 2: every key masked or padding).
 template <typename T>
@@ -451,7 +575,7 @@ int launch_attention(void* out, const void* q, const void* k, const void* v, con
 
 extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t, const void* bias_t,
                                  const float* keybias, const int32_t* tileflags, const void* gate, int64_t B2, int64_t H, int64_t Nq,
-                                 int64_t Nk, int flags, int dtype, void* stream) {
+                                 int64_t Nk, int64_t D, int flags, int dtype, void* stream) {
     FFK_REQUIRE(out && q_t && k_t && v_t && keybias && tileflags, FFK_ERR_NULL, "ffk_attention_fwd: null pointer");
     FFK_REQUIRE(B2 > 0 && B2 < 131072 && H > 0 && H < 65536 && Nq > 0 && Nk > 0 && Nq < (1 << 24) && Nk < (1 << 24),
                 FFK_ERR_SHAPE, "ffk_attention_fwd: bad shape B2=%ld H=%ld Nq=%ld Nk=%ld", (long)B2, (long)H, (long)Nq,
@@ -459,7 +583,19 @@ extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, co
     FFK_REQUIRE(ffk_aligned16(out) && ffk_aligned16(q_t) && ffk_aligned16(k_t) && ffk_aligned16(v_t) &&
                     ffk_aligned16(keybias) && (!bias_t || ffk_aligned16(bias_t)) && (!gate || ffk_aligned16(gate)),
                 FFK_ERR_ALIGN, "ffk_attention_fwd: buffers must be 16-byte aligned");
+    FFK_REQUIRE(D == 32 || D == 64 || D == 128, FFK_ERR_SHAPE,
+                "ffk_attention_fwd: head dimension %ld (32, 64 or 128; narrower heads arrive zero-padded to 32)", (long)D);
     hipStream_t st = (hipStream_t)stream;
+    if (D != 32) {
+        FFK_REQUIRE(!gate, FFK_ERR_UNSUPPORTED, "ffk_attention_fwd: the gate is built for head dimension 32 only");
+        if (dtype == FFK_BF16)
+            return D == 64 ? launch_attention_wide<bf16_t, 2>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st)
+                           : launch_attention_wide<bf16_t, 4>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st);
+        if (dtype == FFK_F32)
+            return D == 64 ? launch_attention_wide<float, 2>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st)
+                           : launch_attention_wide<float, 4>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st);
+        return ffk_fail(FFK_ERR_DTYPE, "ffk_attention_fwd: unsupported dtype tag %d", dtype);
+    }
     switch (dtype) {
         case FFK_BF16: return launch_attention<bf16_t>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, B2, H, Nq, Nk, flags, st);
         case FFK_F32: return launch_attention<float>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, B2, H, Nq, Nk, flags, st);

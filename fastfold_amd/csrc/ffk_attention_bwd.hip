@@ -1,4 +1,7 @@
-// Backward of the attention core for head dimension 32 (see ffk_attention_bwd in include/ffk.h).
+// Backward of the attention core for head dimensions 32, 64 and 128 (see ffk_attention_bwd in include/ffk.h).
+// A head wider than 32 is cut into DP = D / 32 parts of 32 channels, each with operand tiles of its own (part-major:
+// part p of a tensor lies p * part elements behind part 0): scores and dP are sums over the parts, dq / dk / dv have one
+// accumulator tile per part.
 //
 // Like the forward kernel it never forms the [B2, H, Nq, Nk] logits in memory: both kernels recompute the
 // 32 x 32 score tiles from q and k on the matrix pipe.  With  s = q.k / sqrt(d) + bias  (masked keys very
@@ -73,12 +76,12 @@ __device__ __forceinline__ typename Mma<T>::Frag identity_frag(int i, int l32, i
 }
 
 // ------------------------------------------------------------------------------ dq ----
-template <typename T, bool HAS_BIAS>
+template <typename T, int DP, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
     T* __restrict__ dq, float* __restrict__ lse, float* __restrict__ dsum, const T* __restrict__ q_qk,
     const T* __restrict__ k_qk, const T* __restrict__ k_acc, const T* __restrict__ v_qk, const T* __restrict__ bias_t,
     const float* __restrict__ keybias, const T* __restrict__ do_qk, const T* __restrict__ o_qk, int B2, int H, int Nq,
-    int Nk, float dq_scale) {
+    int Nk, float dq_scale, long part_q, long part_k) {
     typedef Mma<T> MM;
     typedef typename MM::Frag Frag;
     constexpr int NF = 16 / MM::KLANE;
@@ -91,13 +94,17 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
     const long bh = item / QT;
     const int h = (int)(bh % H), b2 = (int)(bh / H);
 
-    Tile16<T> qf, dof, of;
-    qf.load(q_qk + ((bh * QT + qt) << 10) + lane * 16);
-    dof.load(do_qk + ((bh * QT + qt) << 10) + lane * 16);
-    of.load(o_qk + ((bh * QT + qt) << 10) + lane * 16);
+    Tile16<T> qf[DP], dof[DP];
     float dpart = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) dpart += dof.f(j) * of.f(j);
+    for (int p = 0; p < DP; ++p) {
+        Tile16<T> of;
+        qf[p].load(q_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+        dof[p].load(do_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+        of.load(o_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) dpart += dof[p].f(j) * of.f(j);
+    }
     const float D = dpart + lane_xor<32>(dpart);             // this lane's query: sum_d do o
     const float* mp = keybias + (long)b2 * KT * 32 + 4 * half;
 
@@ -108,12 +115,15 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
     }
     // S^T tile kt (rows: keys, columns: queries), log2 domain, key bias included
     auto score = [&](int kt, f32x16& s) {
-        Tile16<T> kc;
-        kc.load(k_qk + ((bh * KT + kt) << 10) + lane * 16);
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
+        for (int p = 0; p < DP; ++p) {
+            Tile16<T> kc;
+            kc.load(k_qk + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf[p].frag(i));
+        }
         if (HAS_BIAS) {
             Tile16<T> bc;
             bc.load(bias_t + ((((long)h * QT + qt) * KT + kt) << 10) + lane * 16);
@@ -152,42 +162,57 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
     }
 
     // second walk: dq^T += k^T . dS^T
-    f32x16 acc;
+    f32x16 acc[DP];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    for (int p = 0; p < DP; ++p)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[p][v] = 0.0f;
     for (int kt = 0; kt < KT; ++kt) {
         f32x16 s, dp;
         score(kt, s);
-        Tile16<T> vq, ka;
-        vq.load(v_qk + ((bh * KT + kt) << 10) + lane * 16);
-        ka.load(k_acc + ((bh * KT + kt) << 10) + lane * 16);
 #pragma unroll
         for (int v = 0; v < 16; ++v) dp[v] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(dp, vq.frag(i), dof.frag(i));      // dP^T[key, q] = v[key] . do[q]
+        for (int p = 0; p < DP; ++p) {
+            Tile16<T> vq;
+            vq.load(v_qk + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(dp, vq.frag(i), dof[p].frag(i));      // dP^T[key, q] = v[key] . do[q]
+        }
         float ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) ds[v] = fast_exp2(s[v] - L) * (dp[v] - D);
+        Frag dsf[NF];
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(acc, ka.frag(i), NFrag<T>::make(ds + i * MM::KLANE));
+        for (int i = 0; i < NF; ++i) dsf[i] = NFrag<T>::make(ds + i * MM::KLANE);
+#pragma unroll
+        for (int p = 0; p < DP; ++p) {
+            Tile16<T> ka;
+            ka.load(k_acc + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(acc[p], ka.frag(i), dsf[i]);
+        }
     }
     const int q = qt * 32 + l32;
     if (q < Nq) {
-        T* o = dq + ((bh * Nq + q) << 5) + 4 * half;
+        T* o = dq + (bh * Nq + q) * (32 * DP) + 4 * half;
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int p = 0; p < DP; ++p)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[8 * g + e] = DT<T>::from_f(acc[4 * g + e] * dq_scale);
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[32 * p + 8 * g + e] = DT<T>::from_f(acc[p][4 * g + e] * dq_scale);
     }
 }
 
 // ------------------------------------------------------------------------- dk, dv ----
-template <typename T>
+template <typename T, int DP>
 __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
     T* __restrict__ dk, T* __restrict__ dv, const T* __restrict__ q_qk,
     const T* __restrict__ q_acc, const T* __restrict__ k_qk, const T* __restrict__ v_qk, const T* __restrict__ bias_t,
     const float* __restrict__ keybias, const T* __restrict__ do_qk, const T* __restrict__ do_acc,
-    const float* __restrict__ lse, const float* __restrict__ dsum, int B2, int H, int Nq, int Nk, float dk_scale) {
+    const float* __restrict__ lse, const float* __restrict__ dsum, int B2, int H, int Nq, int Nk, float dk_scale,
+    long part_q, long part_k) {
     typedef Mma<T> MM;
     typedef typename MM::Frag Frag;
     constexpr int NF = 16 / MM::KLANE;
@@ -200,9 +225,12 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
     const long bh = item / KT;
     const int h = (int)(bh % H), b2 = (int)(bh / H);
 
-    Tile16<T> kf, vf;                              // this lane's key (column l32): k and v rows as N operands
-    kf.load(k_qk + ((bh * KT + kt) << 10) + lane * 16);
-    vf.load(v_qk + ((bh * KT + kt) << 10) + lane * 16);
+    Tile16<T> kf[DP], vf[DP];                      // this lane's key (column l32): k and v rows as N operands
+#pragma unroll
+    for (int p = 0; p < DP; ++p) {
+        kf[p].load(k_qk + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+        vf[p].load(v_qk + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+    }
     const int key = kt * 32 + l32;
     const float kb = keybias[(long)b2 * KT * 32 + key];     // 0, masked (-1e9 log2e) or padding (hugely negative)
     Frag ident[NF];
@@ -211,28 +239,31 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
         for (int i = 0; i < NF; ++i) ident[i] = identity_frag<T>(i, l32, half);
     }
 
-    f32x16 acc_k, acc_v;
+    f32x16 acc_k[DP], acc_v[DP];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc_k[v] = acc_v[v] = 0.0f;
+    for (int p = 0; p < DP; ++p)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_k[p][v] = acc_v[p][v] = 0.0f;
     for (int qt = 0; qt < QT; ++qt) {
-        Tile16<T> qc, doc, qa, doa;
-        qc.load(q_qk + ((bh * QT + qt) << 10) + lane * 16);
-        doc.load(do_qk + ((bh * QT + qt) << 10) + lane * 16);
-        qa.load(q_acc + ((bh * QT + qt) << 10) + lane * 16);
-        doa.load(do_acc + ((bh * QT + qt) << 10) + lane * 16);
         f32x16 s, dp;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(s, qc.frag(i), kf.frag(i));        // S[q, key], log2 domain
+        for (int p = 0; p < DP; ++p) {
+            Tile16<T> qc, doc;
+            qc.load(q_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+            doc.load(do_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(s, qc.frag(i), kf[p].frag(i));       // S[q, key], log2 domain
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(dp, doc.frag(i), vf[p].frag(i));     // dP[q, key] = do[q] . v[key]
+        }
         if (bias_t) {                                                           // S += I . bias (rows = queries)
             Tile16<T> bc;
             bc.load(bias_t + ((((long)h * QT + qt) * KT + kt) << 10) + lane * 16);
 #pragma unroll
             for (int i = 0; i < NF; ++i) MM::mma(s, ident[i], bc.frag(i));
         }
-#pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(dp, doc.frag(i), vf.frag(i));      // dP[q, key] = do[q] . v[key]
         const float* lp = lse + (bh * QT + qt) * 32 + 4 * half;
         const float* dpz = dsum + (bh * QT + qt) * 32 + 4 * half;
         float p[16], ds[16];
@@ -247,31 +278,46 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
                 ds[v] = p[v] * (dp[v] - D4[e]);
             }
         }
+        Frag pfr[NF], dsf[NF];
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(acc_v, doa.frag(i), NFrag<T>::make(p + i * MM::KLANE));   // dv^T += do^T . P
+        for (int i = 0; i < NF; ++i) {
+            pfr[i] = NFrag<T>::make(p + i * MM::KLANE);
+            dsf[i] = NFrag<T>::make(ds + i * MM::KLANE);
+        }
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(acc_k, qa.frag(i), NFrag<T>::make(ds + i * MM::KLANE));   // dk^T += q^T . dS
+        for (int pp = 0; pp < DP; ++pp) {
+            Tile16<T> qa, doa;
+            qa.load(q_acc + pp * part_q + ((bh * QT + qt) << 10) + lane * 16);
+            doa.load(do_acc + pp * part_q + ((bh * QT + qt) << 10) + lane * 16);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(acc_v[pp], doa.frag(i), pfr[i]);   // dv^T += do^T . P
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(acc_k[pp], qa.frag(i), dsf[i]);    // dk^T += q^T . dS
+        }
     }
     if (key < Nk) {
-        T* ok = dk + ((bh * Nk + key) << 5) + 4 * half;
-        T* ov = dv + ((bh * Nk + key) << 5) + 4 * half;
+        T* ok = dk + (bh * Nk + key) * (32 * DP) + 4 * half;
+        T* ov = dv + (bh * Nk + key) * (32 * DP) + 4 * half;
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int pp = 0; pp < DP; ++pp)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                ok[8 * g + e] = DT<T>::from_f(acc_k[4 * g + e] * dk_scale);
-                ov[8 * g + e] = DT<T>::from_f(acc_v[4 * g + e]);
-            }
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ok[32 * pp + 8 * g + e] = DT<T>::from_f(acc_k[pp][4 * g + e] * dk_scale);
+                    ov[32 * pp + 8 * g + e] = DT<T>::from_f(acc_v[pp][4 * g + e]);
+                }
     }
 }
 
 // ---------------------------------------------------------------------------- dbias ----
 // dbias[h, q, key] += sum over the batch rows b2 = slice, slice + NS, ... of dS[b2, h, q, key].
-template <typename T>
+template <typename T, int DP>
 __global__ __launch_bounds__(256) void attention_bwd_dbias_kernel(
     float* __restrict__ dbias, const T* __restrict__ q_qk, const T* __restrict__ k_qk, const T* __restrict__ v_qk,
     const T* __restrict__ bias_t, const float* __restrict__ keybias, const T* __restrict__ do_qk,
-    const float* __restrict__ lse, const float* __restrict__ dsum, int B2, int H, int Nq, int Nk, int NS) {
+    const float* __restrict__ lse, const float* __restrict__ dsum, int B2, int H, int Nq, int Nk, int NS,
+    long part_q, long part_k) {
     typedef Mma<T> MM;
     typedef typename MM::Frag Frag;
     constexpr int NF = 16 / MM::KLANE;
@@ -302,19 +348,22 @@ __global__ __launch_bounds__(256) void attention_bwd_dbias_kernel(
     for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
     for (int b2 = slice; b2 < B2; b2 += NS) {
         const long bh = (long)b2 * H + h;
-        Tile16<T> qc, doc, kf, vf;
-        qc.load(q_qk + ((bh * QT + qt) << 10) + lane * 16);
-        doc.load(do_qk + ((bh * QT + qt) << 10) + lane * 16);
-        kf.load(k_qk + ((bh * KT + kt) << 10) + lane * 16);
-        vf.load(v_qk + ((bh * KT + kt) << 10) + lane * 16);
         const float kb = keybias[(long)b2 * KT * 32 + key];
         f32x16 s = sb, dp;
 #pragma unroll
         for (int v = 0; v < 16; ++v) dp[v] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(s, qc.frag(i), kf.frag(i));
+        for (int p = 0; p < DP; ++p) {
+            Tile16<T> qc, doc, kf, vf;
+            qc.load(q_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+            doc.load(do_qk + p * part_q + ((bh * QT + qt) << 10) + lane * 16);
+            kf.load(k_qk + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
+            vf.load(v_qk + p * part_k + ((bh * KT + kt) << 10) + lane * 16);
 #pragma unroll
-        for (int i = 0; i < NF; ++i) MM::mma(dp, doc.frag(i), vf.frag(i));
+            for (int i = 0; i < NF; ++i) MM::mma(s, qc.frag(i), kf.frag(i));
+#pragma unroll
+            for (int i = 0; i < NF; ++i) MM::mma(dp, doc.frag(i), vf.frag(i));
+        }
         const float* lp = lse + (bh * QT + qt) * 32 + 4 * half;
         const float* dpz = dsum + (bh * QT + qt) * 32 + 4 * half;
 #pragma unroll
@@ -337,31 +386,32 @@ __global__ __launch_bounds__(256) void attention_bwd_dbias_kernel(
     }
 }
 
-template <typename T>
+template <typename T, int DP>
 int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk, const void* q_acc,
                const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
                const float* keybias, const void* do_qk, const void* do_acc, const void* o_qk, long B2, long H, long Nq,
                long Nk, float dq_scale, float dk_scale, hipStream_t st) {
     const long QT = (Nq + 31) / 32, KT = (Nk + 31) / 32;
+    const long part_q = B2 * H * QT * 1024, part_k = B2 * H * KT * 1024;
     const long g1 = (B2 * H * QT + 3) / 4, g2 = (B2 * H * KT + 3) / 4;
     FFK_REQUIRE(g1 < (1L << 31) && g2 < (1L << 31), FFK_ERR_SHAPE, "ffk_attention_bwd: too many tiles for one launch");
     if (bias_t) {
-        attention_bwd_dq_kernel<T, true><<<(unsigned)g1, 256, 0, st>>>((T*)dq, lse, dsum, (const T*)q_qk, (const T*)k_qk,
-                                                                     (const T*)k_acc, (const T*)v_qk, (const T*)bias_t, keybias,
-                                                                     (const T*)do_qk, (const T*)o_qk, (int)B2, (int)H, (int)Nq,
-                                                                     (int)Nk, dq_scale);
+        attention_bwd_dq_kernel<T, DP, true><<<(unsigned)g1, 256, 0, st>>>((T*)dq, lse, dsum, (const T*)q_qk, (const T*)k_qk,
+                                                                         (const T*)k_acc, (const T*)v_qk, (const T*)bias_t, keybias,
+                                                                         (const T*)do_qk, (const T*)o_qk, (int)B2, (int)H, (int)Nq,
+                                                                         (int)Nk, dq_scale, part_q, part_k);
     } else {
-        attention_bwd_dq_kernel<T, false><<<(unsigned)g1, 256, 0, st>>>((T*)dq, lse, dsum, (const T*)q_qk, (const T*)k_qk,
-                                                                      (const T*)k_acc, (const T*)v_qk, nullptr, keybias,
-                                                                      (const T*)do_qk, (const T*)o_qk, (int)B2, (int)H, (int)Nq,
-                                                                      (int)Nk, dq_scale);
+        attention_bwd_dq_kernel<T, DP, false><<<(unsigned)g1, 256, 0, st>>>((T*)dq, lse, dsum, (const T*)q_qk, (const T*)k_qk,
+                                                                          (const T*)k_acc, (const T*)v_qk, nullptr, keybias,
+                                                                          (const T*)do_qk, (const T*)o_qk, (int)B2, (int)H, (int)Nq,
+                                                                          (int)Nk, dq_scale, part_q, part_k);
     }
     int rc = ffk_check_launch("ffk_attention_bwd");
     if (rc != FFK_OK) return rc;
-    attention_bwd_dkv_kernel<T><<<(unsigned)g2, 256, 0, st>>>((T*)dk, (T*)dv, (const T*)q_qk, (const T*)q_acc,
-                                                            (const T*)k_qk, (const T*)v_qk, (const T*)bias_t, keybias,
-                                                            (const T*)do_qk, (const T*)do_acc, lse, dsum, (int)B2, (int)H,
-                                                            (int)Nq, (int)Nk, dk_scale);
+    attention_bwd_dkv_kernel<T, DP><<<(unsigned)g2, 256, 0, st>>>((T*)dk, (T*)dv, (const T*)q_qk, (const T*)q_acc,
+                                                                (const T*)k_qk, (const T*)v_qk, (const T*)bias_t, keybias,
+                                                                (const T*)do_qk, (const T*)do_acc, lse, dsum, (int)B2, (int)H,
+                                                                (int)Nq, (int)Nk, dk_scale, part_q, part_k);
     rc = ffk_check_launch("ffk_attention_bwd");
     if (rc != FFK_OK || !dbias) return rc;
     // enough slices of the batch rows for ~ 8 waves per SIMD, at least 8 rows per slice
@@ -371,9 +421,9 @@ int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* ds
     if (ns < 1) ns = 1;
     const long g3 = (ns * tiles + 3) / 4;
     FFK_REQUIRE(g3 < (1L << 31), FFK_ERR_SHAPE, "ffk_attention_bwd: too many tiles for one launch");
-    attention_bwd_dbias_kernel<T><<<(unsigned)g3, 256, 0, st>>>(dbias, (const T*)q_qk, (const T*)k_qk, (const T*)v_qk,
-                                                              (const T*)bias_t, keybias, (const T*)do_qk, lse, dsum,
-                                                              (int)B2, (int)H, (int)Nq, (int)Nk, (int)ns);
+    attention_bwd_dbias_kernel<T, DP><<<(unsigned)g3, 256, 0, st>>>(dbias, (const T*)q_qk, (const T*)k_qk, (const T*)v_qk,
+                                                                  (const T*)bias_t, keybias, (const T*)do_qk, lse, dsum,
+                                                                  (int)B2, (int)H, (int)Nq, (int)Nk, (int)ns, part_q, part_k);
     return ffk_check_launch("ffk_attention_bwd");
 }
 
@@ -382,8 +432,10 @@ int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* ds
 extern "C" int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk,
                                  const void* q_acc, const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
                                  const float* keybias, const void* do_qk, const void* do_acc,
-                                 const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, float dq_scale,
+                                 const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int64_t D, float dq_scale,
                                  float dk_scale, int dtype, void* stream) {
+    FFK_REQUIRE(D == 32 || D == 64 || D == 128, FFK_ERR_SHAPE,
+                "ffk_attention_bwd: head dimension %ld (32, 64 or 128; narrower heads arrive zero-padded to 32)", (long)D);
     FFK_REQUIRE(dq && dk && dv && lse && dsum && q_qk && q_acc && k_qk && k_acc && v_qk && keybias && do_qk && do_acc && o_qk,
                 FFK_ERR_NULL, "ffk_attention_bwd: null pointer");
     FFK_REQUIRE(!dbias || bias_t, FFK_ERR_NULL, "ffk_attention_bwd: dbias needs bias_t");
@@ -395,13 +447,16 @@ extern "C" int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, flo
                     ffk_aligned16(o_qk) && (!bias_t || ffk_aligned16(bias_t)),
                 FFK_ERR_ALIGN, "ffk_attention_bwd: buffers must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
+#define FFK_BWD_ARGS dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias, do_qk, do_acc, o_qk, \
+                     B2, H, Nq, Nk, dq_scale, dk_scale, st
     switch (dtype) {
         case FFK_BF16:
-            return launch_bwd<bf16_t>(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias,
-                                      do_qk, do_acc, o_qk, B2, H, Nq, Nk, dq_scale, dk_scale, st);
+            return D == 32 ? launch_bwd<bf16_t, 1>(FFK_BWD_ARGS)
+                           : (D == 64 ? launch_bwd<bf16_t, 2>(FFK_BWD_ARGS) : launch_bwd<bf16_t, 4>(FFK_BWD_ARGS));
         case FFK_F32:
-            return launch_bwd<float>(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, bias_t, keybias,
-                                     do_qk, do_acc, o_qk, B2, H, Nq, Nk, dq_scale, dk_scale, st);
+            return D == 32 ? launch_bwd<float, 1>(FFK_BWD_ARGS)
+                           : (D == 64 ? launch_bwd<float, 2>(FFK_BWD_ARGS) : launch_bwd<float, 4>(FFK_BWD_ARGS));
         default: return ffk_fail(FFK_ERR_DTYPE, "ffk_attention_bwd: unsupported dtype tag %d", dtype);
     }
+#undef FFK_BWD_ARGS
 }

@@ -6,11 +6,11 @@
 for q, k, v ``[b1, b2, h, n, d]``, mask ``[b1, b2, n]`` (0/1, over keys) and bias ``[b1, h, n, n]``.
 The logits are never materialised: the operands are re-tiled into the 32x32 MFMA order and handed to
 the flash attention kernel (``ffk_attention_fwd``); the backward pass (``ffk_attention_bwd``) recomputes them the
-same way.  The kernel is
-specialised for the Evoformer's head dim (32); narrower heads (8 and 16, the extra-MSA and template stacks)
-are zero-padded to 32 channels, which changes neither the scores nor the used output channels; the
-reference's Triton kernel also takes 64 and 128 (triton/attention_core.py:143), which no module of the
-path uses and which raise ``RuntimeError`` here.
+same way.  The tuned kernel is the Evoformer's head dim (32); narrower heads (8 and 16, the extra-MSA and template
+stacks) are zero-padded to 32 channels, which changes neither the scores nor the used output channels; the other
+widths the reference's Triton kernel takes (64 and 128, triton/attention_core.py:142), which no module of the path
+uses, run on a plain one-wave-per-query-tile instantiation that cuts the head into 32-channel parts.
+Dtypes: bf16 and fp32 (forward and backward); fp16 raises here, before anything is launched.
 """
 import math
 
@@ -28,17 +28,20 @@ def _attention_core(q, k, v, mask=None, bias=None):
         raise RuntimeError("fused_attention_core: q, k, v must be [b1, b2, h, n, d] of one shape, got %s %s %s"
                            % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
     b1, b2, h, n, d = q.shape
-    if d not in (8, 16, 32):
-        raise RuntimeError("fused_attention_core: head dim %d is not supported: the kernel is built for 32 and takes "
-                           "8 and 16 zero-padded; 64 and 128 (accepted by the reference's Triton kernel) are not built" % d)
+    if d not in (8, 16, 32, 64, 128):
+        raise RuntimeError("fused_attention_core: head dim %d is not supported (8, 16, 32, 64 or 128)" % d)
+    if q.dtype not in (torch.bfloat16, torch.float32) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("fused_attention_core: q, k, v must share one dtype, bfloat16 or float32 (got %s, %s, %s)"
+                           % (q.dtype, k.dtype, v.dtype))
     if mask is not None and tuple(mask.shape) != (b1, b2, n):
         raise RuntimeError("fused_attention_core: mask must be [b1, b2, n], got %s" % (tuple(mask.shape),))
     if bias is not None and tuple(bias.shape) != (b1, h, n, n):
         raise RuntimeError("fused_attention_core: bias must be [b1, h, n, n], got %s" % (tuple(bias.shape),))
     # zero channels past d add nothing to q.k and give zero output channels, which are dropped at the end
-    out = torch.empty(b1, b2, n, h * 32, dtype=q.dtype, device=q.device)
+    dk = max(d, 32)                        # head width the kernel sees
+    out = torch.empty(b1, b2, n, h * dk, dtype=q.dtype, device=q.device)
     if out.numel() == 0:
-        return out.view(b1, b2, n, h, 32)[..., :d].reshape(b1, b2, n, h * d)
+        return out.view(b1, b2, n, h, dk)[..., :d].reshape(b1, b2, n, h * d)
     nt = layouts.n_tiles(n)
     scale = _lib.LOG2E / math.sqrt(d)      # the kernel exponentiates in base 2
     kb = torch.empty(b2, nt * 32, dtype=torch.float32, device=q.device)
@@ -47,10 +50,10 @@ def _attention_core(q, k, v, mask=None, bias=None):
         mk = mask[i].to(q.dtype).contiguous() if mask is not None else torch.ones(b2, n, dtype=q.dtype, device=q.device)
         _lib.key_bias(kb, fl, mk, B=b2, N=n, mask_sb=n, mask_sn=1)
         bt = layouts.tile_bias((bias[i].float() * _lib.LOG2E).to(q.dtype)) if bias is not None else None
-        _lib.attention_fwd(out[i].view(b2 * n, h * 32), _lib.tile_pack(q[i], _lib.FFK_TILE_QK, scale),
+        _lib.attention_fwd(out[i].view(b2 * n, h * dk), _lib.tile_pack(q[i], _lib.FFK_TILE_QK, scale),
                            _lib.tile_pack(k[i], _lib.FFK_TILE_QK), _lib.tile_pack(v[i], _lib.FFK_TILE_V), bt, kb, fl,
-                           None, B2=b2, H=h, Nq=n, Nk=n)
-    if d != 32:
+                           None, B2=b2, H=h, Nq=n, Nk=n, D=dk)
+    if d < 32:
         return out.view(b1, b2, n, h, 32)[..., :d].reshape(b1, b2, n, h * d)
     return out
 
@@ -61,8 +64,9 @@ def _attention_core_backward(q, k, v, mask, bias, out, dout, need_dbias):
     dt, dev = q.dtype, q.device
     QK, ACC = _lib.FFK_TILE_QK, _lib.FFK_TILE_V
     nt = layouts.n_tiles(n)
+    dk_ = max(d, 32)
     scale = _lib.LOG2E / math.sqrt(d)
-    dq, dk, dv = (torch.empty(b1, b2, h, n, 32, dtype=dt, device=dev) for _ in range(3))
+    dq, dk, dv = (torch.empty(b1, b2, h, n, dk_, dtype=dt, device=dev) for _ in range(3))
     dbias = torch.zeros(b1, h, n, n, dtype=torch.float32, device=dev) if (need_dbias and bias is not None) else None
     kb = torch.empty(b2, nt * 32, dtype=torch.float32, device=dev)
     fl = torch.empty(b2, nt, dtype=torch.int32, device=dev)
@@ -79,8 +83,8 @@ def _attention_core_backward(q, k, v, mask, bias, out, dout, need_dbias):
                            _lib.tile_pack(k[i], QK), _lib.tile_pack(k[i], ACC), _lib.tile_pack(v[i], QK),
                            bt, kb,
                            _lib.tile_pack(do_, QK), _lib.tile_pack(do_, ACC), _lib.tile_pack(o_, QK),
-                           B2=b2, H=h, Nq=n, Nk=n, dq_scale=1.0 / math.sqrt(d), dk_scale=1.0 / _lib.LOG2E)
-    if d != 32:
+                           B2=b2, H=h, Nq=n, Nk=n, D=dk_, dq_scale=1.0 / math.sqrt(d), dk_scale=1.0 / _lib.LOG2E)
+    if d < 32:
         dq, dk, dv = (t[..., :d] for t in (dq, dk, dv))
     return dq, dk, dv, (None if dbias is None else dbias.to(dt))
 

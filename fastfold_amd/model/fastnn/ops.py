@@ -74,19 +74,55 @@ def _no_grad_guard(module, *tensors):
             % type(module).__name__)
 
 
+_WARNED_EVAL_GRAD = False
+
+
 def _needs_grad(module, *tensors):
     """True when autograd has to see this call: gradients are enabled and an input or a parameter of ``module``
-    requires one.  Such calls take the differentiable composition (``_train`` methods: the reference's own sequence
-    of operators - HIP LayerNorm / attention-core / elementwise kernels with backward passes, library GEMMs for the
-    ``Linear`` layers); everything else takes the fused forward-only launches."""
+    requires one.  Such calls take the differentiable composition (``_train`` methods); everything else takes the
+    fused forward-only launches.  A module in ``eval()`` mode whose parameters still require gradients, called
+    outside ``torch.no_grad()`` with inputs that need none, is almost always an inference call that forgot the
+    ``no_grad``: it is honoured (autograd semantics), but a warning is raised once, because the differentiable
+    composition is several times slower and carries the plain bf16 residual stream."""
+    global _WARNED_EVAL_GRAD
     if not torch.is_grad_enabled():
         return False
     if any(t is not None and t.requires_grad for t in tensors):
         return True
-    return any(p.requires_grad for p in module.parameters())
+    if any(p.requires_grad for p in module.parameters()):
+        if not module.training and not _WARNED_EVAL_GRAD:
+            _WARNED_EVAL_GRAD = True
+            import warnings
+            warnings.warn("fastfold_amd: %s is in eval() mode but was called with gradients enabled and parameters that "
+                          "require them: taking the differentiable (slower, plain-residual) path.  Wrap inference calls in "
+                          "torch.no_grad() to run the fused kernels." % type(module).__name__, RuntimeWarning, stacklevel=3)
+        return True
+    return False
 
 
 _WGRAD_SPLIT_ROWS = 4096
+
+
+def _storage_span(t):
+    """(first byte, one past the last byte) that a view addresses inside its storage."""
+    if t.numel() == 0:
+        return (0, 0)
+    last = t.storage_offset() + sum((n - 1) * st for n, st in zip(t.shape, t.stride()))
+    return (t.storage_offset() * t.element_size(), (last + 1) * t.element_size())
+
+
+def _check_library_gemm_operands(a, b, who):
+    """Host-side guard in front of every *library* batched GEMM of the differentiable path: each operand view must lie
+    inside its allocation, and the two operands must not be views of one allocation (two GPU memory faults at
+    128 x 1024^3, bf16, were reported from inside the library's batched NT GEMM when its operands were the two halves
+    of one buffer; the callers' views were in bounds).  Raises instead of launching."""
+    for t in (a, b):
+        lo, hi = _storage_span(t)
+        if hi > t.untyped_storage().nbytes():
+            raise RuntimeError("%s: an operand view addresses %d bytes of a %d-byte allocation"
+                               % (who, hi, t.untyped_storage().nbytes()))
+    if a.numel() and b.numel() and a.untyped_storage().data_ptr() == b.untyped_storage().data_ptr():
+        raise RuntimeError("%s: both operands of a library batched GEMM are views of one allocation" % who)
 
 
 def _weight_grad(dy2, x2):
@@ -100,8 +136,66 @@ def _weight_grad(dy2, x2):
         S *= 2
     if S == 1 or dy2.dtype == torch.float32:
         return dy2.t() @ x2
-    part = torch.bmm(dy2.reshape(S, M // S, -1).transpose(1, 2), x2.reshape(S, M // S, -1))
+    a = dy2.reshape(S, M // S, -1).transpose(1, 2)
+    b = x2.reshape(S, M // S, -1)
+    if a.untyped_storage().data_ptr() == b.untyped_storage().data_ptr():
+        b = b.clone()                      # e.g. dy2 and x2 sliced from one tensor: give the library two allocations
+    _check_library_gemm_operands(a, b, "_weight_grad")
+    part = torch.bmm(a, b)
     return part.sum(0, dtype=torch.float32).to(dy2.dtype)
+
+
+def _padded_copy(x):
+    """[c, m, k] view (any strides) -> a freshly allocated contiguous [c, m, kpad] tensor, the last axis zero-padded
+    to the GEMM kernels' 16-byte K step."""
+    kpad = F_.round_up(x.shape[-1], F_.vec_of(x.dtype))
+    out = (torch.zeros if kpad != x.shape[-1] else torch.empty)(x.shape[0], x.shape[1], kpad, dtype=x.dtype,
+                                                                 device=x.device)
+    out[..., :x.shape[-1]].copy_(x)
+    return out
+
+
+def _chan_major(t, perm):
+    """[1, a, b, c] -> [c, x, kpad] with (c, x, k) the last three axes in the order ``perm`` names
+    (permute_final_dims indices), in an allocation of its own."""
+    return _padded_copy(permute_final_dims(t, perm)[0])
+
+
+def _bgemm_cm(a, b, n_valid):
+    """out[c, i, j] = sum_k a[c, i, k] b[c, j, k] for j < n_valid (rows of b past n_valid are padding) through
+    ``ffk_bgemm_nt`` (the library's own batched NT GEMM, the kernel the fused path's contraction runs on); the
+    output's last axis is padded like the operands' and the padding zero."""
+    c, M, K = a.shape
+    N = b.shape[1]
+    npad = F_.round_up(n_valid, F_.vec_of(a.dtype))
+    out = (torch.zeros if npad != n_valid else torch.empty)(c, M, npad, dtype=a.dtype, device=a.device)
+    _lib.bgemm_nt(a, b, out, M=M, N=n_valid, K=K, lda=K, ldb=K, batch=c, a_bs=M * K, b_bs=N * K, o_bs=M * npad,
+                  s_i=npad)
+    return out
+
+
+class _TriContractFn(torch.autograd.Function):
+    """p[c, i, j] = sum_k L[c, i, k] R[c, j, k], forward and both backward products on ``ffk_bgemm_nt``
+    (reference: the permuted ``torch.matmul`` of fastnn/ops.py:400-403,529-532).  L, R: separately allocated
+    [c, r, kpad] tensors (``_chan_major``); returns [c, r, kpad] with zero padding columns."""
+
+    @staticmethod
+    def forward(ctx, L, R, r):
+        ctx.save_for_backward(L, R)
+        ctx.r = r
+        return _bgemm_cm(L, R, r)
+
+    @staticmethod
+    def backward(ctx, dp):
+        L, R = ctx.saved_tensors
+        r = ctx.r
+        dp = dp.contiguous()
+        dL = dR = None
+        if ctx.needs_input_grad[0]:      # dL[c, i, k] = sum_j dp[c, i, j] R[c, j, k]: K runs over j
+            dL = _bgemm_cm(dp, _padded_copy(R.transpose(1, 2)[:, :r]), r)
+        if ctx.needs_input_grad[1]:      # dR[c, j, k] = sum_i dp[c, i, j] L[c, i, k]: K runs over i
+            dR = _bgemm_cm(_padded_copy(dp[:, :, :r].transpose(1, 2)), _padded_copy(L.transpose(1, 2)[:, :r]), r)
+        return dL, dR, None
 
 
 class _LinearFn(torch.autograd.Function):
@@ -148,30 +242,29 @@ def _mask_like(mask, x):
     return F_._mask_derived(mask, ("cast", x.dtype), lambda: mask.to(dtype=x.dtype).contiguous())
 
 
-class DropoutRowwise(nn.Module):
+class _SharedAxisDropout(nn.Module):
+    """Dropout whose keep / drop decision is drawn once per slice and shared along one axis of a
+    [b, i, j, c] tensor (reference: ops.py:45-68): the decision tensor has extent 1 on ``_shared_axis``."""
+    _shared_axis = 1
 
     def __init__(self, p):
-        super(DropoutRowwise, self).__init__()
+        super().__init__()
         self.p = p
         self.dropout = nn.Dropout(p=p)
 
     def forward(self, x):
-        dropout_mask = torch.ones_like(x[:, 0:1, :, :])
-        dropout_mask = self.dropout(dropout_mask)
-        return dropout_mask * x
+        keep = self.dropout(torch.ones_like(x.narrow(self._shared_axis, 0, 1)))
+        return x * keep
 
 
-class DropoutColumnwise(nn.Module):
+class DropoutRowwise(_SharedAxisDropout):
+    """One decision per (b, j, c), shared by all rows i."""
+    _shared_axis = 1
 
-    def __init__(self, p):
-        super(DropoutColumnwise, self).__init__()
-        self.p = p
-        self.dropout = nn.Dropout(p=p)
 
-    def forward(self, x):
-        dropout_mask = torch.ones_like(x[:, :, 0:1, :])
-        dropout_mask = self.dropout(dropout_mask)
-        return dropout_mask * x
+class DropoutColumnwise(_SharedAxisDropout):
+    """One decision per (b, i, c), shared by all columns j."""
+    _shared_axis = 2
 
 
 class Linear(nn.Linear, _PackMixin):
@@ -526,9 +619,10 @@ class ChunkMSAColumnGlobalAttention(nn.Module):
 
 
 def permute_final_dims(tensor, inds):
-    zero_index = -1 * len(inds)
-    first_inds = list(range(len(tensor.shape[:zero_index])))
-    return tensor.permute(first_inds + [zero_index + i for i in inds])
+    """Permutes the last ``len(inds)`` axes of ``tensor`` by ``inds`` (reference: ops.py:366-369)."""
+    n = len(inds)
+    lead = tensor.dim() - n
+    return tensor.permute(*range(lead), *(lead + i for i in inds))
 
 
 class _TriangleMultiplication(nn.Module, _PackMixin):
@@ -588,10 +682,11 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         lr = lr * torch.sigmoid(self.left_right_gate(Z))
         left, right = lr.chunk(2, dim=-1)
         g = torch.sigmoid(self.output_gate(Z))
-        if self._incoming:      # p[c, i, j] = sum_k left[k, i, c] right[k, j, c]
-            p = torch.matmul(permute_final_dims(left, (2, 1, 0)), permute_final_dims(right, (2, 0, 1)))
-        else:                   # p[c, i, j] = sum_k left[i, k, c] right[j, k, c]
-            p = torch.matmul(permute_final_dims(left, (2, 0, 1)), permute_final_dims(right, (2, 1, 0)))
+        # channel-major operands [c, i, k] / [c, j, k] in two allocations of their own, the contraction and its two
+        # backward products on the library's own batched GEMM kernel
+        r = Z_raw.shape[1]
+        perm = (2, 1, 0) if self._incoming else (2, 0, 1)      # incoming: L[c, i, k] = left[k, i, c]
+        p = _TriContractFn.apply(_chan_major(left, perm), _chan_major(right, perm), r)[None, :, :, :r]
         ab = self.output_projection(self.layernorm2(permute_final_dims(p, (1, 2, 0))))
         dropout_mask = torch.ones_like(Z[:, 0:1, :, :])
         return bias_ele_dropout_residual(ab, self.output_bias, g, dropout_mask, Z_raw, prob=self.p_drop,

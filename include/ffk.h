@@ -252,7 +252,8 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
 
 
 /* ------------------------------------------------------------------------------------
- * Flash-style attention core for head dimension 32 (logits never reach HBM):
+ * Flash-style attention core (logits never reach HBM) for head dimension D = 32 - the Evoformer's, and the tuned
+ * path - and D = 64 / 128, the other widths the reference's kernel accepts (kernel/triton/attention_core.py:142):
  *     o[b2, q, h, :] = softmax_k( q.k^T + bias[h, q, k] + keybias[b2, k] ) . v   (* gate)
  * in the exp2 domain: q must already carry the factor  d^-1/2 * log2(e)  and bias the
  * factor log2(e); keybias is fp32 (0 for a valid key, -1e9*log2e for a masked key and a
@@ -267,7 +268,10 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  *   tileflags: [B2][ceil(Nk/32)] int32 per 32-key tile: 0 all keys valid, 1 mixed, 2 all masked
  *   gate     : multiplicative gate (already sigmoid-ed) or NULL: [B2*Nq, H*32] row-major, or with
  *              FFK_ATT_GATE_TILED in flags [B2][H][ceil(Nq/32)][1024] in FFK_TILE_ACC order
- *   out      : [B2*Nq, H*32] row-major
+ *   out      : [B2*Nq, H*D] row-major
+ * D = 64 / 128: the head is cut into D / 32 parts of 32 channels; q_t, k_t (FFK_TILE_QK order) and v_t hold one
+ * [B2][H][ceil(N/32)][1024] block per part, part-major ([D/32][B2][H][...]: part p = channels 32p .. 32p+31 of
+ * every head), q still carries d^-1/2 * log2(e) with d = D; gate must be NULL.
  * Replaces: the matmul / fused_softmax / matmul (+ bias_sigmod_ele) chain of
  * SelfAttention.forward (fastfold/model/fastnn/ops.py:310-322) and
  * fused_attention_core (kernel/attention_core.py:17-52, kernel/triton/attention_core.py:12-190).
@@ -275,7 +279,7 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
 enum { FFK_ATT_GATE_TILED = 1 };
 int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t,
                       const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
-                      int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int flags, int dtype, void* stream);
+                      int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int64_t D, int flags, int dtype, void* stream);
 
 /* Backward of ffk_attention_fwd without a gate (the autograd path of fused_attention_core):
  *     given do = d loss / d out, computes dq, dk, dv and (optionally) dbias of
@@ -290,7 +294,8 @@ int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v
  *   keybias     : as for ffk_attention_fwd
  *   lse, dsum   : fp32 scratch [B2][H][ceil(Nq/32)*32] (row log-sum-exp in the log2 domain and sum_d do.o; written by
  *                 the first kernel, read by the second)
- *   dq : [B2][H][Nq][32], dk, dv : [B2][H][Nk][32] (operand dtype);  dbias : fp32 [H][Nq][Nk], ZEROED by the caller:
+ *   D = 64 / 128: every tiled operand part-major as for ffk_attention_fwd ([D/32] blocks of the D = 32 layout)
+ *   dq : [B2][H][Nq][D], dk, dv : [B2][H][Nk][D] (operand dtype);  dbias : fp32 [H][Nq][Nk], ZEROED by the caller:
  *                 a third kernel sums dS over slices of the batch rows in registers and adds each slice's sum with
  *                 one atomic per element (summation order across slices not fixed), or NULL
  *   dq_scale = 1 / sqrt(d), dk_scale = 1 / log2(e): undo the factors folded into the q operand.
@@ -300,7 +305,7 @@ int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v
 int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* dsum, const void* q_qk,
                       const void* q_acc, const void* k_qk, const void* k_acc, const void* v_qk, const void* bias_t,
                       const float* keybias, const void* do_qk, const void* do_acc,
-                      const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, float dq_scale,
+                      const void* o_qk, int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int64_t D, float dq_scale,
                       float dk_scale, int dtype, void* stream);
 
 /* Re-tiles a strided tensor x[b2, h, n, d] (element at src + b2*s_b + h*s_h + n*s_n + d, strides in elements,

@@ -205,11 +205,42 @@ def test_fused_attention_core_op(dev, dtype, tol, b1, b2, h, n):
         outd = fused_attention_core(qd, kd, vd, mask, bias)
         assert outd.shape == (b1, b2, n, h * d)
         assert _rel(_np(outd), ops_np.attention_core(_np(qd), _np(kd), _np(vd), _np(mask), _np(bias))) < tol
-    # 64 / 128 (taken by the reference's Triton kernel, used by no module of the path) are refused by name
-    with pytest.raises(RuntimeError, match="64 and 128"):
-        fused_attention_core(torch.cat([q, q], -1), torch.cat([k, k], -1), torch.cat([v, v], -1), mask, bias)
+    # 64 / 128: the other widths the reference's Triton kernel takes (kernel/triton/attention_core.py:142)
+    for d in (64, 128):
+        qd, kd, vd = (torch.randn(b1, b2, h, n, d, generator=g).to(dev, dtype) for _ in range(3))
+        outd = fused_attention_core(qd, kd, vd, mask, bias)
+        assert outd.shape == (b1, b2, n, h * d) and outd.dtype == dtype
+        assert _rel(_np(outd), ops_np.attention_core(_np(qd), _np(kd), _np(vd), _np(mask), _np(bias))) < tol, d
+        # without bias, and as strided views of a fused projection
+        qkv = torch.randn(b1, b2, n, 3 * h * d, generator=g).to(dev, dtype)
+        qs, ks, vs = (t.unflatten(-1, (h, d)).transpose(-2, -3) for t in qkv.chunk(3, dim=-1))
+        outs = fused_attention_core(qs, ks, vs, mask, None)
+        zero_bias = torch.zeros(b1, h, n, n)
+        assert _rel(_np(outs), ops_np.attention_core(_np(qs), _np(ks), _np(vs), _np(mask), zero_bias.numpy())) < tol, d
+    with pytest.raises(RuntimeError, match="not supported"):
+        fused_attention_core(q[..., :24], k[..., :24], v[..., :24], mask, bias)
+    with pytest.raises(RuntimeError, match="bfloat16 or float32"):       # fp16 is refused before anything is launched
+        fused_attention_core(q.half(), k.half(), v.half(), mask.half(), bias.half())
     with pytest.raises(RuntimeError):
         fused_attention_core(q.cpu(), k.cpu(), v.cpu(), mask.cpu(), bias.cpu())
+
+
+@pytest.mark.parametrize("n", [32, 256, 370, 512])
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_fused_attention_core_reference_shapes(dev, n, d):
+    """Shapes of the reference's own test of the operator (tests/test_fastnn/test_attention_core.py:36-44: batch 1,
+    chunk 8, 4 heads, std-0.5 operands, a random 0/1 key mask, sequence lengths from its list), bf16, against the
+    float64 formula."""
+    from fastfold_amd.model.fastnn.kernel import fused_attention_core
+    g = torch.Generator().manual_seed(n + d)
+    q, k, v = (0.5 * torch.randn(1, 8, 4, n, d, generator=g) for _ in range(3))
+    q, k, v = (t.to(dev, torch.bfloat16) for t in (q, k, v))
+    mask = (torch.randn(1, 8, n, generator=g) > 0).to(dev, torch.bfloat16)
+    mask[..., 0] = 1
+    bias = torch.randn(1, 4, n, n, generator=g).to(dev, torch.bfloat16)
+    out = fused_attention_core(q, k, v, mask, bias)
+    ref = ops_np.attention_core(_np(q), _np(k), _np(v), _np(mask), _np(bias))
+    assert _rel(_np(out), ref) < 2e-2
 
 
 def _torch_attention_core(q, k, v, mask, bias):
@@ -226,7 +257,9 @@ def _torch_attention_core(q, k, v, mask, bias):
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
 @pytest.mark.parametrize("b1,b2,h,n,d,use_bias", [(1, 3, 4, 77, 32, True), (2, 2, 8, 64, 32, True), (1, 2, 4, 130, 32, False),
                                                   (1, 2, 4, 50, 16, True), (1, 3, 8, 40, 8, True),
-                                                  (1, 43, 4, 70, 32, True)])      # several batch-row slices in the dbias kernel
+                                                  (1, 43, 4, 70, 32, True),       # several batch-row slices in the dbias kernel
+                                                  (1, 3, 4, 77, 64, True), (2, 2, 4, 64, 128, True), (1, 2, 4, 45, 128, False),
+                                                  (1, 19, 4, 70, 64, True)])
 def test_fused_attention_core_backward(dev, dtype, tol, b1, b2, h, n, d, use_bias):
     """dq, dk, dv, dbias of the exported op (``ffk_attention_bwd``: logits recomputed tile by tile) against torch
     autograd of the reference's formula in float64, with masked keys, a ragged last tile and the narrow heads."""

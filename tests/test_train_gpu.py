@@ -230,3 +230,47 @@ def test_elementwise_ops_backward(dev, dtype):
     ((zr2 + dm.double() * (g2 * (ab2 + b2))) * cot.double()).sum().backward()
     for a, ref in ((ab, ab2), (b, b2), (gt, g2), (zr, zr2)):
         assert _rel(a.grad, ref.grad) <= tol, _rel(a.grad, ref.grad)
+
+
+def test_block_forward_backward_at_headline_size(dev):
+    """The differentiable block at the headline shape (N_seq = 128, N_res = 1024, last 5 % of the residues masked), bf16:
+    outputs against the fused forward-only launches, every gradient finite, and the two input gradients against the
+    same path run in fp32 (which the small-shape tests above pin to the float64 oracle) at the bf16 bound.  The
+    triangle contraction and its two backward products run on ffk_bgemm_nt at this size (128 x 1024^3), the weight
+    gradients of the million-row activations through the guarded slab GEMM."""
+    import sys
+    print("test_block_forward_backward_at_headline_size: s=128 r=1024 bf16 + fp32", flush=True)
+    sys.stdout.flush()
+    s, r, tail = 128, 1024, 0.05
+    model = _oracle(33, 1)
+    m, z, mm, pm = synth_inputs(33, s, r, mask_tail_frac=tail)
+    nv = r - int(round(tail * r))
+    g = torch.Generator().manual_seed(7)
+    cot_z = torch.randn(r, r, KW["c_z"], generator=g)
+    cot_z[nv:] = 0
+    cot_z[:, nv:] = 0
+    grads, outs = {}, {}
+    for dtype in (torch.bfloat16, torch.float32):
+        fast = _fast(model, dev, dtype).eval()
+        mi, zi = (torch.from_numpy(t).to(dev, dtype).requires_grad_() for t in (m, z))
+        mk, pk = torch.from_numpy(mm).to(dev, dtype), torch.from_numpy(pm).to(dev, dtype)
+        out = fast(mi, zi, mk, pk, chunk_size=None)
+        assert out[1].grad_fn is not None
+        if dtype == torch.bfloat16:
+            with torch.no_grad():
+                fused = fast(mi, zi, mk, pk, chunk_size=None)
+            assert _rel(out[0][:, :nv], fused[0][:, :nv]) <= 2e-2
+            assert _rel(out[1][:nv, :nv], fused[1][:nv, :nv]) <= 2e-2
+            del fused
+        (out[1].float() * cot_z.to(dev)).sum().backward()
+        torch.cuda.synchronize()
+        for name, p in fast.named_parameters():
+            assert p.grad is not None and bool(torch.isfinite(p.grad.float()).all()), name
+        assert bool(torch.isfinite(mi.grad.float()).all()) and bool(torch.isfinite(zi.grad.float()).all())
+        grads[dtype] = (mi.grad.float().cpu(), zi.grad.float().cpu())
+        outs[dtype] = out[1].detach().float().cpu()
+        del fast, out, mi, zi
+        torch.cuda.empty_cache()
+    assert _rel(outs[torch.bfloat16][:nv, :nv], outs[torch.float32][:nv, :nv]) <= 2e-2
+    assert _rel(grads[torch.bfloat16][0], grads[torch.float32][0]) <= 5e-2, _rel(grads[torch.bfloat16][0], grads[torch.float32][0])
+    assert _rel(grads[torch.bfloat16][1], grads[torch.float32][1]) <= 5e-2, _rel(grads[torch.bfloat16][1], grads[torch.float32][1])

@@ -34,13 +34,20 @@ def test_pair_bias_static_matches_pair_bias(dev):
                                scratch.data_ptr(), r, C, H, amap[0], amap[1], amap[2], _lib.LOG2E, 1e-5, _lib.FFK_BF16, st)
         assert rc == 0, lib.ffk_last_error_string()
         got = torch.zeros_like(want)
+        args = (got.data_ptr(), z.data_ptr(), gam.data_ptr(), bet.data_ptr(), wb.data_ptr(),
+                r, C, H, amap[0], amap[1], amap[2], _lib.LOG2E, 1e-5, _lib.FFK_BF16, st)
+        if i == 0:
+            # one untimed call first: the code object load and the one-time symbol lookup of a device are not
+            # what "allocates nothing" is about
+            assert lib.ffk_pair_bias_static(*args) == 0, lib.ffk_last_error_string()
         torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
-        rc = lib.ffk_pair_bias_static(got.data_ptr(), z.data_ptr(), gam.data_ptr(), bet.data_ptr(), wb.data_ptr(),
-                                      r, C, H, amap[0], amap[1], amap[2], _lib.LOG2E, 1e-5, _lib.FFK_BF16, st)
+        free_before = torch.cuda.mem_get_info()[0]        # the driver's view: sees a hipMalloc made by the library too
+        rc = lib.ffk_pair_bias_static(*args)
         assert rc == 0, lib.ffk_last_error_string()
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before, "free device memory changed across the call"
         assert float(want.float().abs().max()) > 0.5
         assert torch.equal(got, want), "case %d: static-scratch result differs" % i
 
