@@ -265,6 +265,8 @@ def test_block_forward_backward_at_headline_size(dev):
         (out[1].float() * cot_z.to(dev)).sum().backward()
         torch.cuda.synchronize()
         for name, p in fast.named_parameters():
+            if name.startswith("linear."):        # the single-representation projection: not on the path to z
+                continue
             assert p.grad is not None and bool(torch.isfinite(p.grad.float()).all()), name
         assert bool(torch.isfinite(mi.grad.float()).all()) and bool(torch.isfinite(zi.grad.float()).all())
         grads[dtype] = (mi.grad.float().cpu(), zi.grad.float().cpu())
