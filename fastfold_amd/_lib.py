@@ -73,8 +73,8 @@ def stream_ptr() -> int:
 
 
 def ptr(t):
-    """Device address of a tensor (None -> NULL)."""
-    return None if t is None else t.data_ptr()
+    """Device address of a tensor (None -> NULL; an address given as an int is passed through)."""
+    return None if t is None else (t if isinstance(t, int) else t.data_ptr())
 
 
 def check_device(*tensors):
@@ -327,6 +327,15 @@ SIGNATURES["ffk_transition_fused"] = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L
 def transition_fused(out, x, gamma, beta, w1, b1, w2, b2, *, M, C, hidden, eps=1e-5, xtail=None):
     call("ffk_transition_fused", ptr(out), ptr(x), ptr(xtail), ptr(gamma), ptr(beta), ptr(w1), ptr(b1), ptr(w2), ptr(b2), M, C,
          hidden, eps, dtype_tag(x.dtype), stream_ptr())
+
+
+SIGNATURES["ffk_gated_out_fused"] = [_P] * 10 + [_L, _L, _L, _L, _L, _F, _I, _P]
+
+
+def gated_out_fused(out, x, gamma, beta, wg, bg, o, wo, bo, *, M, C, inner, s_o, s_i, eps=1e-5, xtail=None):
+    """out = x + Wo (sigmoid(Wg LN(x) + bg) * o) + bo over logical rows (see include/ffk.h)."""
+    call("ffk_gated_out_fused", ptr(out), ptr(x), ptr(xtail), ptr(gamma), ptr(beta), ptr(wg), ptr(bg), ptr(o), ptr(wo), ptr(bo),
+         M, C, inner, s_o, s_i, eps, dtype_tag(o.dtype), stream_ptr())
 
 
 def key_bias(keybias, tileflags, mask, *, B, N, mask_sb=0, mask_sn=1):

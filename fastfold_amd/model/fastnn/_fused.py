@@ -222,7 +222,19 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     # kernel, which writes q, k and the gate in accumulator order straight from its registers.
     acc_order = dt == torch.bfloat16 and C in (64, 128, 256) and N % 32 == 0
     qk_kind = FFK_TILE_ACC if acc_order else FFK_TILE_QK
-    gate = torch.empty((slab, H, NT, 1024) if acc_order else (slab * N, HC), dtype=dt, device=dev)
+    # Where the update goes back into the tensor the gate is computed from (every attention of the Evoformer block),
+    # the gate is not a tensor at all: the output stage computes sigmoid(Wg LN(x) + bg) from the rows of x it reads as
+    # residual anyway and multiplies the heads' outputs by it on their way into the output projection
+    # (ffk_gated_out_fused).  The projection launch then writes q, k, v only and the core reads no gate.
+    # Measured at N_seq = 128: with a million rows (N_res = 1024) the projection and the core each get ~ 3 % faster and
+    # the output stage as much slower - 1.3 GB less memory traffic per block at the same block time -; with 65 536 rows
+    # (N_res = 256) the non-persistent output stage loses 1.3 % of a block, so small launches keep the gate tensor.
+    gate_in_out = (_GATE_IN_OUT_STAGE and M >= _GATE_IN_OUT_MIN_ROWS and acc_order and ln is not None and C in (128, 256)
+                   and HC == C and c_out == C and resid is not None and o_map is None
+                   and resid.data_ptr() == x.data_ptr() and a_so % 16 == 0 and a_si % 16 == 0)
+    gate = None
+    if not gate_in_out:
+        gate = torch.empty((slab, H, NT, 1024) if acc_order else (slab * N, HC), dtype=dt, device=dev)
     o = torch.empty(slab * N, HC, dtype=dt, device=dev)
     tpg = HC // 128
     qscale = LOG2E / math.sqrt(float(head_dim))
@@ -234,7 +246,8 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     # With 128 input channels, at most four heads and all rows in one slab the bias rides on the projection launch:
     # the weights-stationary kernel computes its four dot products per row on the vector pipe from the rows it
     # has in LDS anyway (one read of x less than a pass of its own; -0.05 ms per triangle attention at N = 1024).
-    rides = bias_tile is not None and acc_order and C == 128 and H <= 4 and slab >= B2 and _PAIR_BIAS_RIDES
+    rides = (bias_tile is not None and acc_order and C == 128 and H <= 4 and slab >= B2 and _PAIR_BIAS_RIDES
+             and (not gate_in_out or hasattr(w_pk, "without_gate")))
     # Otherwise the skinny bias projection has its own pass over x.  It goes first: x was written by the launch before
     # this call and is still (partly) cache-resident, and the bias pass writes little, so the projection after
     # it finds x as warm as before - the other way round the projection's output (four times the size of x)
@@ -265,7 +278,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         for buf, kind, scale in ((q_t, qk_kind, qscale), (k_t, qk_kind, 1.0), (v_t, FFK_TILE_V, 1.0)):
             for t in range(tpg):
                 tiles.append(make_tile(buf.data_ptr() + t * 4 * NT * 1024 * es, kind=kind, scale=scale, **tkw))
-        for t in range(tpg):
+        for t in range(0 if gate_in_out else tpg):
             if acc_order:
                 tiles.append(make_tile(gate.data_ptr() + t * 4 * NT * 1024 * es, kind=FFK_TILE_ACC,
                                        bias=gate_bias_pk.data_ptr() + t * 128 * es, act=FFK_ACT_SIGMOID, **tkw))
@@ -275,12 +288,21 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         if bias_tile is not None:      # single slab: the bias rides on the projection launch
             tiles.append(bias_tile)
         # the weights-stationary kernel holds at most 16 (K = 256) or 24 (K = 128) 32-channel units per launch
-        per = 4 if (acc_order and C == 256) else len(tiles)
+        per = (3 if gate_in_out else 4) if (acc_order and C == 256) else len(tiles)
         for t0 in range(0, len(tiles), per):
-            _lib.fused_linear(x, w_pk, tiles[t0:t0 + per], M=Ms, K=C, a_inner=inner, a_so=a_so, a_si=a_si, ln=ln,
+            # a bias tile riding behind q, k, v (no gate tiles) takes its weight rows from the gate-less packing
+            wp = w_pk.without_gate if (gate_in_out and bias_tile is not None) else w_pk
+            _lib.fused_linear(x, wp, tiles[t0:t0 + per], M=Ms, K=C, a_inner=inner, a_so=a_so, a_si=a_si, ln=ln,
                               w_row_off=t0 * 128, a_off=off)
         _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb[b0:b0 + nb], flags[b0:b0 + nb], gate, B2=nb, H=H, Nq=N, Nk=N,
                            gate_tiled=acc_order)
+        if gate_in_out:
+            # packed rows of w_pk: q, k, v, gate blocks of HC rows each; o holds the slab's rows in logical order
+            _lib.gated_out_fused(out.data_ptr() + o_off * es, x.data_ptr() + off * es, ln[0], ln[1],
+                                 w_pk.data_ptr() + 3 * HC * C * es, gate_bias_pk, o, wo_pk, out_bias_pk, M=Ms, C=C,
+                                 inner=inner, s_o=a_so, s_i=a_si,
+                                 xtail=None if xtail is None else xtail.data_ptr() + o_off)
+            continue
         tiles = []
         for t in range((c_out + 127) // 128):
             tiles.append(make_tile(out.data_ptr() + (o_off + t * 128) * es,
@@ -360,6 +382,8 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
 # (block 6.97 -> 6.885 ms in a same-box A/B at N_res = 1024; 64, 192 and 1088 elements measure the same).
 _TRIMUL_CHAN_PAD = 64
 _PAIR_BIAS_RIDES = True      # see attention(): switch for same-box comparisons
+_GATE_IN_OUT_STAGE = True    # see attention(): False keeps the gate a tensor (written by the projection, read by the core)
+_GATE_IN_OUT_MIN_ROWS = 131072
 
 
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,

@@ -469,7 +469,12 @@ class SelfAttention(nn.Module, _PackMixin):
                     _pad_heads(self.gating_linear.weight, H, c, 0)]
             w = F_.pack_rows(mats, dtype, device)
             if extra_rows is not None:
-                w = torch.cat([w, F_.pack_rows([extra_rows()], dtype, device)], 0).contiguous()
+                hc = H * 32
+                extra = F_.pack_rows([extra_rows()], dtype, device)
+                w = torch.cat([w, extra], 0).contiguous()
+                # the same without the gate block ([q; k; v; extra]): the projection launch of an attention whose gate
+                # is computed in the output stage finds the extra (pair-bias) rows right behind v
+                w.without_gate = torch.cat([w[:3 * hc], extra], 0).contiguous()
             return (w, F_.pack_vec([_pad_heads(self.gating_bias, H, c, 0)], dtype, device),
                     F_.pack_rows([_pad_heads(self.o_linear.weight, H, c, 1)], dtype, device))
         return self._packed(key, params, build)

@@ -366,6 +366,19 @@ int ffk_transition_fused(void* out, const void* x, void* xtail, const void* gamm
                          const void* b1, const void* w2, const void* b2, int64_t M, int64_t C,
                          int64_t hidden, float eps, int dtype, void* stream);
 
+/* Gated output stage of a gated attention (bf16; C = 128 or 256 channels, H * 32 = C gate channels):
+ *     out[row m] = x[row m] + Wo . ( sigmoid( Wg . LayerNorm(x[row m]; gamma, beta, eps) + bg ) * o[m] ) + bo
+ * x, out : the tensor the attention updates, logical row m at (m / inner) * s_o + (m % inner) * s_i (elements, C
+ * contiguous channels; may alias); o : [M, C] the heads' weighted averages in logical row order (ffk_attention_fwd
+ * called without a gate); wg : [C, C] gate projection, bg : [C]; wo : [C, C] output projection, bo : [C] or NULL;
+ * xtail : NULL or the tail bytes of x / out as an extended residual stream (addressed like x).
+ * The gate is computed where it is used: it is neither written by the projection launch nor read by the attention
+ * core.  Replaces: gating_linear + bias_sigmod_ele + o_linear (+ bias_dropout_add in eval mode) of
+ * SelfAttention.forward and its callers (fastfold/model/fastnn/ops.py:320-324, 666-670; msa.py:66-72,96-100). */
+int ffk_gated_out_fused(void* out, const void* x, void* xtail, const void* gamma, const void* beta, const void* wg,
+                        const void* bg, const void* o, const void* wo, const void* bo, int64_t M, int64_t C,
+                        int64_t inner, int64_t s_o, int64_t s_i, float eps, int dtype, void* stream);
+
 /* Global column attention core of the extra-MSA stack: one query per residue column (the masked mean
  * of the normalised rows), one key / value head of width D shared by the H query heads.
  *     x_s = LayerNorm(m[s, j, :]; gamma, beta, ln_eps)
