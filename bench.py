@@ -85,8 +85,9 @@ def build_stack(no_blocks, dev, dtype, seed=0):
 
 def micro_ops(dev):
     """benchmark configuration 2: fused softmax [1,128,8,256,256] bf16 with pair bias and 10% masked keys;
-    LayerNorm over [65536,128] and [32768,256] bf16; plus a plain device copy of the softmax's
-    bytes as the practical HBM ceiling of this box.  Each op runs over rotating buffers (> 512 MB in
+    LayerNorm over [65536,128] and [32768,256] bf16; plus two plain copies of the same bytes as the practical
+    HBM ceiling of this box: torch's copy_ and the library's streaming copy (ffk_stream_copy: the row kernels' own
+    access pattern without their arithmetic).  Each op runs over rotating buffers (> 512 MB in
     total, so nothing is served from cache) as N launches recorded into one HIP graph; the time is
     the graph replay divided by N (no host launch overhead, no per-launch events)."""
     import torch
@@ -131,6 +132,9 @@ def micro_ops(dev):
     res["softmax_bf16_1x128x8x256x256"] = run(
         lambda i: _softmax_forward(xs[i % nb], mask, bias, out=outs[i % nb]), 20, nbytes)
     res["device_copy_same_bytes_as_softmax"] = run(lambda i: outs[i % nb].copy_(xs[i % nb]), 20, nbytes)
+    res["stream_copy_same_bytes_as_softmax"] = run(
+        lambda i: _lib.call("ffk_stream_copy", outs[i % nb].data_ptr(), xs[i % nb].data_ptr(), nbytes // 2, _lib.stream_ptr()),
+        20, nbytes)
     del xs, outs
     for rows, cols in ((65536, 128), (32768, 256)):
         nb = 20
@@ -145,6 +149,9 @@ def micro_ops(dev):
         res["layernorm_bf16_%dx%d" % (rows, cols)] = run(f, 60, 2 * rows * cols * 2)
         if cols == 128:
             res["device_copy_same_bytes_as_layernorm"] = run(lambda i: os_[i % nb].copy_(xs[i % nb]), 60, 2 * rows * cols * 2)
+            res["stream_copy_same_bytes_as_layernorm"] = run(
+                lambda i: _lib.call("ffk_stream_copy", os_[i % nb].data_ptr(), xs[i % nb].data_ptr(), rows * cols * 2,
+                                    _lib.stream_ptr()), 60, 2 * rows * cols * 2)
         del xs, os_
     return res
 

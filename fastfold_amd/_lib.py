@@ -29,6 +29,7 @@ SIGNATURES = {
     "ffk_bias_sigmoid_mul": [_P, _P, _P, _P, _L, _L, _I, _P],
     "ffk_bias_dropout_add": [_P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P],
     "ffk_bias_ele_dropout_res": [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P],
+    "ffk_stream_copy": [_P, _P, _L, _P],
 }
 
 _lib = None

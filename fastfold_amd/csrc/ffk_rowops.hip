@@ -662,6 +662,39 @@ int eltwise_dispatch(int dtype, void* out, const void* a, const void* bias, cons
 }  // namespace
 
 // -------------------------------------------------------------------- C ABI ----
+// Plain streaming copy with the access pattern of the row kernels (16-byte non-temporal loads and stores, four
+// vectors in flight per lane): what a read-once / write-once stream of a given size reaches on this GPU.
+namespace {
+__global__ __launch_bounds__(BLOCK) void stream_copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, long n) {
+    constexpr int U = 4;
+    const long stride = (long)gridDim.x * BLOCK * U;
+    for (long i = (long)blockIdx.x * BLOCK * U + threadIdx.x; i < n; i += stride) {
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const long k = i + u * BLOCK;
+            if (k < n) v[u] = __builtin_nontemporal_load(src + k);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const long k = i + u * BLOCK;
+            if (k < n) __builtin_nontemporal_store(v[u], dst + k);
+        }
+    }
+}
+}  // namespace
+
+extern "C" int ffk_stream_copy(void* dst, const void* src, int64_t bytes, void* stream) {
+    FFK_REQUIRE(dst && src, FFK_ERR_NULL, "ffk_stream_copy: null pointer");
+    FFK_REQUIRE(bytes > 0 && bytes % 16 == 0, FFK_ERR_SHAPE, "ffk_stream_copy: size %ld is not a positive multiple of 16", (long)bytes);
+    FFK_REQUIRE(ffk_aligned16(dst) && ffk_aligned16(src), FFK_ERR_ALIGN, "ffk_stream_copy: buffers must be 16-byte aligned");
+    const long n = bytes / 16;
+    long blocks = (n + BLOCK * 4 - 1) / (BLOCK * 4);
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    stream_copy_kernel<<<dim3((unsigned)blocks), BLOCK, 0, (hipStream_t)stream>>>((u32x4*)dst, (const u32x4*)src, n);
+    return ffk_check_launch("ffk_stream_copy");
+}
+
 extern "C" int ffk_softmax_fwd(void* out, const void* x, const void* mask, const void* bias, int64_t B1,
                                int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int dtype, void* stream) {
     FFK_REQUIRE(out && x, FFK_ERR_NULL, "ffk_softmax_fwd: null pointer");

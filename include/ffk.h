@@ -60,6 +60,12 @@ int ffk_softmax_fwd(void* out, const void* x, const void* mask, const void* bias
 int ffk_softmax_bwd(void* dx, const void* dy, const void* y, int64_t rows, int64_t cols,
                     int dtype, void* stream);
 
+/* Measurement aid with no counterpart in the reference: a plain streaming copy of `bytes` (a multiple of 16) with the
+ * access pattern of the row kernels (16-byte non-temporal loads and stores, a grid like theirs).  bench.py times it
+ * beside the fused softmax and LayerNorm: it is what a read-once / write-once stream of the same size reaches on the
+ * GPU at hand, the practical ceiling of an HBM-bound row kernel. */
+int ffk_stream_copy(void* dst, const void* src, int64_t bytes, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * LayerNorm over the last dimension, affine:  out = (x - mean) * rsqrt(var + eps) * gamma + beta
  *   x, out : [rows, cols] contiguous;  gamma, beta : [cols] of the same dtype
