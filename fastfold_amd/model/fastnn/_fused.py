@@ -185,7 +185,8 @@ def transition(x, out, *, ln, w1_pk, b1_pk, w2, b2, hidden, budget, xtail=None):
 
 # ---------------------------------------------------------------------- attention ----
 def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_pk, out_bias_pk, c_out,
-              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None, head_dim=32, budget=None, o_map=None, xtail=None):
+              mask, mask_sb, mask_sn, bias_t=None, bias_in_launch=False, pb_scratch=None, head_dim=32, budget=None, o_map=None, xtail=None,
+              drop=None):
     """Gated multi-head attention over N tokens for each of B2 batch rows.  The kernels work on 32-wide
     heads; a narrower head (``head_dim`` < 32) arrives zero-padded to 32 channels in ``w_pk`` / ``wo_pk``,
     which changes neither the scores nor the used output channels - only the score scale is its own.
@@ -200,6 +201,10 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     elements per batch row): the batch rows are then processed in slabs - projection, core, output projection per
     slab.  Batch rows are independent and a slab's outputs overwrite only the rows it read, so this also holds
     when ``out`` aliases ``x``; the additive bias, which reads all of x, is computed before the first slab.
+
+    ``drop``: None, or a [period, c_out] tensor of dropout multipliers (0 or 1 / (1 - p)) that scales the update of logical
+    row m by its row ``m % period`` before the residual is added (the shared-axis dropout of the training mode:
+    ``bias_dropout_add`` with a mask drawn by the caller).
     """
     dt, dev = x.dtype, x.device
     es = es_of(dt)
@@ -229,7 +234,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     # Measured at N_seq = 128: with a million rows (N_res = 1024) the projection and the core each get ~ 3 % faster and
     # the output stage as much slower - 1.3 GB less memory traffic per block at the same block time -; with 65 536 rows
     # (N_res = 256) the non-persistent output stage loses 1.3 % of a block, so small launches keep the gate tensor.
-    gate_in_out = (_GATE_IN_OUT_STAGE and M >= _GATE_IN_OUT_MIN_ROWS and acc_order and ln is not None and C in (128, 256)
+    gate_in_out = (_GATE_IN_OUT_STAGE and drop is None and M >= _GATE_IN_OUT_MIN_ROWS and acc_order and ln is not None and C in (128, 256)
                    and HC == C and c_out == C and resid is not None and o_map is None
                    and resid.data_ptr() == x.data_ptr() and a_so % 16 == 0 and a_si % 16 == 0)
     gate = None
@@ -309,6 +314,8 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
                                    bias=None if out_bias_pk is None else out_bias_pk.data_ptr() + t * 128 * es,
                                    resid=None if resid is None else resid.data_ptr() + (o_off + t * 128) * es,
                                    xtail=xtail_ptr(xtail, o_off + t * 128),
+                                   gate=None if drop is None else drop.data_ptr() + t * 128 * es,
+                                   gate_ld=0 if drop is None else c_out, gate_rows=0 if drop is None else drop.shape[0],
                                    inner=inner, s_o=o_so, s_i=o_si, ncols=min(128, c_out - t * 128)))
         _lib.fused_linear(o, wo_pk, tiles, M=Ms, K=HC)
     return out
@@ -387,10 +394,12 @@ _GATE_IN_OUT_MIN_ROWS = 131072
 
 
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,
-                            dual_pk=None, xtail=None):
+                            dual_pk=None, xtail=None, drop=None):
     """out = z + sigmoid(Wg LN(z) + bg) * (Wout LN2(p) + b_out),  p[i,j,:] = sum_k a[i,k,:] b[j,k,:]
     (outgoing) or sum_k a[k,i,:] b[k,j,:] (incoming), a/b the masked gated projections.
-    ``dual_pk`` = (weights, biases) of pack_trimul_out: the gate is then computed in the output stage."""
+    ``dual_pk`` = (weights, biases) of pack_trimul_out: the gate is then computed in the output stage.
+    ``drop``: None, or [r, C] dropout multipliers shared by all rows i (the update of (i, j) is scaled by drop[j]): the
+    gate tensor is multiplied by it, so the output stage is the one with a gate tensor."""
     dt, dev = z.dtype, z.device
     es = es_of(dt)
     M = r * r
@@ -399,7 +408,7 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
     # channel planes of the operands and of the contraction result are cs elements apart (_TRIMUL_CHAN_PAD beyond r * kpad)
     cs = r * kpad + _TRIMUL_CHAN_PAD
     lr = alloc((2, c, cs), dt, dev, zero)
-    dual = dual_pk is not None and trimul_gate_in_output_stage(dt, r, C, c)
+    dual = dual_pk is not None and drop is None and trimul_gate_in_output_stage(dt, r, C, c)
     g = None if dual else torch.empty(M, C, dtype=dt, device=dev)
     tiles = []
     if incoming:      # logical row (a, b) reads z[b, a]
@@ -417,6 +426,8 @@ def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu
         tiles.append(make_tile(g.data_ptr() + t * 128 * es, bias=b_pk.data_ptr() + (n_glu + t) * 128 * es,
                                act=FFK_ACT_SIGMOID, ncols=min(128, C - t * 128), **kw))
     _lib.fused_linear(z, w_pk, tiles, M=M, K=C, a_inner=a_map[0], a_so=a_map[1], a_si=a_map[2], ln=ln1)
+    if drop is not None:
+        g.view(r, r, C).mul_(drop[None])
     p = torch.empty(c, cs, dtype=dt, device=dev)
     _lib.bgemm_nt(lr[0], lr[1], p, M=r, N=r, K=kpad, lda=kpad, ldb=kpad, batch=c, a_bs=cs, b_bs=cs,
                   o_bs=cs, s_i=kpad)

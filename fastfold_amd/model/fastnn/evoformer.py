@@ -26,7 +26,34 @@ def _private_copy(view, owner):
     return out.clone() if out.data_ptr() == owner.data_ptr() else out
 
 
+class _BlockRecompute(torch.autograd.Function):
+    """One Evoformer block as its own checkpoint: the forward pass runs the fused launches (nothing of it is kept but
+    the two inputs and the dropout multipliers, which are drawn here so that both passes see the same ones); the
+    backward pass re-runs the block operator by operator with autograd on, the way block checkpointing re-runs it
+    (fastfold/utils/checkpointing.py:55-73; evoformer.py:262-266), and back-propagates through that."""
+
+    @staticmethod
+    def forward(ctx, block, msa_mask, pair_mask, drops, _grad_anchor, m, z):
+        ctx.block, ctx.masks, ctx.drops = block, (msa_mask, pair_mask), drops
+        ctx.save_for_backward(m, z)
+        return block._core(m.contiguous(), z.contiguous(), msa_mask, pair_mask, inplace=False, drops=drops)
+
+    @staticmethod
+    def backward(ctx, dm, dz):
+        m, z = ctx.saved_tensors
+        with torch.enable_grad():
+            m_, z_ = m.detach().requires_grad_(True), z.detach().requires_grad_(True)
+            mo, zo = ctx.block._core_train(m_, z_, *ctx.masks, drops=ctx.drops if ctx.drops is not None else {})
+        torch.autograd.backward((mo, zo), (dm, dz))        # parameter gradients accumulate here, as under checkpointing
+        return None, None, None, None, None, m_.grad, z_.grad
+
+
 class Evoformer(nn.Module):
+
+    # A call that autograd has to see runs the fused forward and re-runs the block in the backward pass
+    # (_BlockRecompute).  False: the forward itself is the operator-by-operator composition, every intermediate is
+    # kept, and the backward pass re-runs nothing.
+    recompute_in_backward = True
 
     def __init__(self, c_m: int, c_z: int, first_block: bool, last_block: bool, is_multimer: bool = False):
         super(Evoformer, self).__init__()
@@ -38,9 +65,10 @@ class Evoformer(nn.Module):
         self.is_multimer = is_multimer
 
     # -- un-padded core on [1, s, r, c_m] / [1, r, r, c_z] / [1, s, r] / [1, r, r] ----------
-    def _core(self, m, z, msa_mask, pair_mask, inplace: bool, tails=(None, None)):
+    def _core(self, m, z, msa_mask, pair_mask, inplace: bool, tails=(None, None), drops=None):
         """``tails = (m_tail, z_tail)``: int8 tails of m / z as extended residual streams (the stack's bf16 mode),
-        or None for the plain stream of the reference."""
+        or None for the plain stream of the reference.  ``drops``: None, or the dropout multipliers of a training-mode
+        pass (``_draw_drops``; out-of-place only)."""
         F_.check_nonempty("Evoformer", m, z)
         mt, zt = tails
         if self.is_multimer:
@@ -48,31 +76,57 @@ class Evoformer(nn.Module):
             # pair tensor it leaves, the pair stack runs last
             z_new = z if inplace else torch.empty_like(z)
             self.communication._run(m, msa_mask, z, z_new, zt)
-            m = self.msa.inplace(m, z_new, msa_mask, mt) if inplace else self.msa.forward(m, z_new, msa_mask, mt)
-            self.pair.inplace([z_new], pair_mask, zt)
+            m = self.msa.inplace(m, z_new, msa_mask, mt) if inplace else self.msa.forward(m, z_new, msa_mask, mt, drops=drops)
+            self.pair.inplace([z_new], pair_mask, zt, drops=drops)
             return m, z_new
         if inplace:
             m = self.msa.inplace(m, z, msa_mask, mt)
             self.communication._run(m, msa_mask, z, z, zt)
             self.pair.inplace([z], pair_mask, zt)
             return m, z
-        m = self.msa.forward(m, z, msa_mask, mt)
+        m = self.msa.forward(m, z, msa_mask, mt, drops=drops)
         z_new = torch.empty_like(z)
         self.communication._run(m, msa_mask, z, z_new, zt)
-        self.pair.inplace([z_new], pair_mask, zt)
+        self.pair.inplace([z_new], pair_mask, zt, drops=drops)
         return m, z_new
 
-    def _core_train(self, m, z, msa_mask, pair_mask):
+    def _core_train(self, m, z, msa_mask, pair_mask, drops=None):
         """The differentiable block (evoformer.py:64-76) on the un-padded tensors: every update is out of place and
-        made of operators with a backward pass."""
+        made of operators with a backward pass.  ``drops``: None (every module draws its own dropout mask in training
+        mode) or the multipliers drawn by the caller (a dict, possibly empty: no dropout)."""
         F_.check_nonempty("Evoformer", m, z)
         if self.is_multimer:
             z_ori = self.communication(m, msa_mask, z)
-            z = self.pair(z_ori, pair_mask)
-            return self.msa(m, z_ori, msa_mask), z
-        m = self.msa(m, z, msa_mask)
+            z = self.pair(z_ori, pair_mask, drops=drops)
+            return self.msa(m, z_ori, msa_mask, drops=drops), z
+        m = self.msa(m, z, msa_mask, drops=drops)
         z = self.communication(m, msa_mask, z)
-        return m, self.pair(z, pair_mask)
+        return m, self.pair(z, pair_mask, drops=drops)
+
+    def _draw_drops(self, m, z):
+        """Dropout multipliers (0 or 1 / (1 - p)) of one training-mode pass of this block, one tensor per update that
+        the reference drops (msa.py:70-73; triangle.py:66-75,122-131,168-173,215-222): shared along the rows, except for
+        the ending-node attention, which shares them along the columns.  None in eval mode."""
+        if not self.training:
+            return None
+        r = z.shape[-2]
+
+        def draw(p, shape):
+            return F.dropout(torch.ones(shape, dtype=z.dtype, device=z.device), p=p, training=True) if p > 0 else None
+        pair = self.pair
+        d = {"row": draw(self.msa.MSARowAttentionWithPairBias.p_drop, (1, 1, r, m.shape[-1])),
+             "tmo": draw(pair.TriangleMultiplicationOutgoing.p_drop, (1, 1, r, z.shape[-1])),
+             "tmi": draw(pair.TriangleMultiplicationIncoming.p_drop, (1, 1, r, z.shape[-1])),
+             "tas": draw(pair.TriangleAttentionStartingNode.p_drop, (1, 1, r, z.shape[-1])),
+             "tae": draw(pair.TriangleAttentionEndingNode.p_drop, (1, r, 1, z.shape[-1]))}
+        return {k: v for k, v in d.items() if v is not None}
+
+    def _run_grad(self, m, z, msa_mask, pair_mask):
+        """The block under autograd, on the un-padded [1, ...] tensors."""
+        if not self.recompute_in_backward:
+            return self._core_train(m, z, msa_mask, pair_mask)
+        anchor = torch.empty(0, device=m.device, requires_grad=True)     # outputs need a gradient even when m and z do not
+        return _BlockRecompute.apply(self, msa_mask, pair_mask, self._draw_drops(m, z), anchor, m, z)
 
     def _enter(self, m, z, r):
         if self.first_block:
@@ -100,7 +154,7 @@ class Evoformer(nn.Module):
                 m, z = m.unsqueeze(0), z.unsqueeze(0)
             else:
                 m, z = m[:, :, :r, :], z[:, :r, :r, :]
-            return self._leave(*self._core_train(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)))
+            return self._leave(*self._run_grad(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0)))
         m, z = self._enter(m, z, r)
         m, z = self._core(m, z, msa_mask.unsqueeze(0), pair_mask.unsqueeze(0), inplace=not self.first_block)
         return self._leave(m, z)
@@ -173,6 +227,12 @@ class EvoformerStack(nn.Module):
             return a, b
         if per is None:
             mm, zz = run(blocks, mm, zz)
+        elif all(blk.recompute_in_backward for blk in blocks):
+            # every block its own checkpoint, with a fused forward (at least as fine as groups of blocks_per_ckpt)
+            for blk in blocks:
+                if self.clear_cache_between_blocks:
+                    torch.cuda.empty_cache()
+                mm, zz = blk._run_grad(mm, zz, mk, pk)
         else:
             for i in range(0, len(blocks), per):
                 mm, zz = checkpoint(run, blocks[i:i + per], mm, zz, use_reentrant=False)

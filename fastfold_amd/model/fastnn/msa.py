@@ -40,7 +40,8 @@ class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
                                        last_bias_fuse=True)
         self.out_bias = nn.parameter.Parameter(data=torch.zeros((d_node,)), requires_grad=True)
 
-    def _run(self, M_raw, Z, M_mask, out, xtail=None):
+    def _run(self, M_raw, Z, M_mask, out, xtail=None, drop=None):
+        """``drop``: None or the [1, 1, r, C] dropout multipliers of a training-mode call (drawn by the caller)."""
         F_.check_cuda(M_raw, Z, M_mask)
         _no_grad_guard(self, M_raw, Z)
         dt, dev = M_raw.dtype, M_raw.device
@@ -63,15 +64,17 @@ class MSARowAttentionWithPairBias(nn.Module, _PackMixin):
         F_.attention(M_raw, out, M_raw, B2=s, N=r, C=C, H=self.n_head, a_map=(s * r, 0, C),
                      ln=_ln_pair(self.layernormM, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
                      c_out=C, mask=mask, mask_sb=r, mask_sn=1, bias_t=bias_t, head_dim=self.c, budget=_budget(),
-                     xtail=_check_tail(xtail, M_raw))
+                     xtail=_check_tail(xtail, M_raw), drop=None if drop is None else drop.reshape(r, C).contiguous())
         return out
 
-    def _train(self, M_raw, Z, M_mask):
-        """msa.py:60-74, operator by operator."""
+    def _train(self, M_raw, Z, M_mask, drop=None):
+        """msa.py:60-74, operator by operator.  ``drop``: dropout multipliers drawn by the caller; None = drawn here."""
         from .kernel import bias_dropout_add
         M = self.layernormM(M_raw)
         b = F.linear(self.layernormZ(Z), self.linear_b_weights.to(Z.dtype))
         M = self.attention(M, M_mask, (b, None))
+        if drop is not None:
+            return bias_dropout_add(M, self.out_bias, drop, M_raw, prob=0.0, training=False)
         dropout_mask = torch.ones_like(M[:, 0:1, :, :])
         return bias_dropout_add(M, self.out_bias, dropout_mask, M_raw, prob=self.p_drop, training=self.training)
 
@@ -143,20 +146,25 @@ class MSACore(nn.Module):
         self.MSAColumnAttention = MSAColumnAttention(d_node=d_node)
         self.MSATransition = Transition(d=d_node)
 
-    def forward(self, node, pair, node_mask, xtail=None):
+    def forward(self, node, pair, node_mask, xtail=None, drops=None):
         """node [1, s, r, d_node], pair [1, r, r, d_pair], node_mask [1, s, r] -> new node
         (the input tensor is left untouched; the two later updates run in place on the copy).
         ``xtail``: int8 tail of the *new* node tensor as an extended residual stream (zero on entry when the input
-        is a plain bf16 tensor)."""
+        is a plain bf16 tensor).  ``drops``: None, or a dict with the dropout multipliers of a training-mode call
+        drawn by the caller (key "row": [1, 1, r, d_node])."""
+        drop = None if drops is None else drops.get("row")
         if _needs_grad(self, node, pair):
             if xtail is not None:
                 raise RuntimeError("MSACore: the extended residual stream is forward-only")
-            node = self.MSARowAttentionWithPairBias(node, pair, node_mask)
+            if drop is not None:
+                node = self.MSARowAttentionWithPairBias._train(node, pair, node_mask, drop=drop)
+            else:
+                node = self.MSARowAttentionWithPairBias(node, pair, node_mask)
             node = self.MSAColumnAttention(node, node_mask)
             return self.MSATransition(node)
         node = node.contiguous()
         out = torch.empty_like(node)
-        self.MSARowAttentionWithPairBias._run(node, pair, node_mask, out, xtail)
+        self.MSARowAttentionWithPairBias._run(node, pair, node_mask, out, xtail, drop=drop)
         self.MSAColumnAttention._run(out, node_mask, out, xtail)
         self.MSATransition._run(out, out, xtail)
         return out

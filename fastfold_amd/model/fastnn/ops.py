@@ -646,7 +646,8 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         self.output_bias = nn.parameter.Parameter(data=torch.zeros((d_pair,)), requires_grad=True)
         self.p_drop = p_drop
 
-    def _run(self, Z_raw, Z_mask, out, xtail=None):
+    def _run(self, Z_raw, Z_mask, out, xtail=None, drop=None):
+        """``drop``: None or the [1, 1, r, C] dropout multipliers of a training-mode call (drawn by the caller)."""
         F_.check_cuda(Z_raw, Z_mask)
         _no_grad_guard(self, Z_raw)
         dt, dev = Z_raw.dtype, Z_raw.device
@@ -676,11 +677,13 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         F_.triangle_multiplication(Z_raw, out, r=r, C=C, c=self.c, incoming=self._incoming,
                                    ln1=_ln_pair(self.layernorm1, dt), w_pk=w, b_pk=b, n_glu=n_glu,
                                    ln2=_ln_pair(self.layernorm2, dt), wout_pk=wout, out_bias_pk=bout,
-                                   mask=_mask_like(Z_mask, Z_raw), dual_pk=dual, xtail=_check_tail(xtail, Z_raw))
+                                   mask=_mask_like(Z_mask, Z_raw), dual_pk=dual, xtail=_check_tail(xtail, Z_raw),
+                                   drop=None if drop is None else drop.reshape(r, C).contiguous())
         return out
 
-    def _train(self, Z_raw, Z_mask):
-        """triangle.py:41-75 / :97-131, operator by operator."""
+    def _train(self, Z_raw, Z_mask, drop=None):
+        """triangle.py:41-75 / :97-131, operator by operator.  ``drop``: dropout multipliers drawn by the caller
+        ([1, 1, r, C]); None = drawn here in training mode."""
         from .kernel import bias_ele_dropout_residual
         Z = self.layernorm1(Z_raw)
         lr = Z_mask.unsqueeze(-1).to(Z.dtype) * self.left_right_projection(Z)
@@ -693,6 +696,8 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         perm = (2, 1, 0) if self._incoming else (2, 0, 1)      # incoming: L[c, i, k] = left[k, i, c]
         p = _TriContractFn.apply(_chan_major(left, perm), _chan_major(right, perm), r)[None, :, :, :r]
         ab = self.output_projection(self.layernorm2(permute_final_dims(p, (1, 2, 0))))
+        if drop is not None:
+            return bias_ele_dropout_residual(ab, self.output_bias, g, drop, Z_raw, prob=0.0, training=False)
         dropout_mask = torch.ones_like(Z[:, 0:1, :, :])
         return bias_ele_dropout_residual(ab, self.output_bias, g, dropout_mask, Z_raw, prob=self.p_drop,
                                          training=self.training)
@@ -734,7 +739,9 @@ class _TriangleAttention(nn.Module, _PackMixin):
                                        last_bias_fuse=True)
         self.out_bias = nn.parameter.Parameter(data=torch.zeros((d_pair,)), requires_grad=True)
 
-    def _run(self, Z_raw, Z_mask, out, xtail=None):
+    def _run(self, Z_raw, Z_mask, out, xtail=None, drop=None):
+        """``drop``: None or the dropout multipliers of a training-mode call, [1, 1, r, C] (starting node) or
+        [1, r, 1, C] (ending node)."""
         F_.check_cuda(Z_raw, Z_mask)
         _no_grad_guard(self, Z_raw)
         dt, dev = Z_raw.dtype, Z_raw.device
@@ -757,10 +764,11 @@ class _TriangleAttention(nn.Module, _PackMixin):
         F_.attention(Z_raw, out, Z_raw, B2=r, N=r, C=C, H=self.n_head, a_map=a_map,
                      ln=_ln_pair(self.layernorm1, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
                      c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=bias_t, bias_in_launch=True, pb_scratch=pbs,
-                     head_dim=self.c, budget=_budget(), xtail=_check_tail(xtail, Z_raw))
+                     head_dim=self.c, budget=_budget(), xtail=_check_tail(xtail, Z_raw),
+                     drop=None if drop is None else drop.reshape(r, C).contiguous())     # logical row m: key index m % r
         return out
 
-    def _train(self, Z_raw, Z_mask):
+    def _train(self, Z_raw, Z_mask, drop=None):
         """triangle.py:156-173 (starting node) / :202-222 (ending node: the same on the transposed pair tensor, with
         the dropout mask shared along the other axis)."""
         from .kernel import bias_dropout_add
@@ -774,6 +782,8 @@ class _TriangleAttention(nn.Module, _PackMixin):
             dropout_mask = torch.ones_like(Z[:, :, 0:1, :])
         else:
             dropout_mask = torch.ones_like(Z[:, 0:1, :, :])
+        if drop is not None:
+            return bias_dropout_add(Z, self.out_bias, drop, Z_raw, prob=0.0, training=False)
         return bias_dropout_add(Z, self.out_bias, dropout_mask, Z_raw, prob=self.p_drop, training=self.training)
 
     def forward(self, Z_raw, Z_mask):

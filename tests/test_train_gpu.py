@@ -276,3 +276,58 @@ def test_block_forward_backward_at_headline_size(dev):
     assert _rel(outs[torch.bfloat16][:nv, :nv], outs[torch.float32][:nv, :nv]) <= 2e-2
     assert _rel(grads[torch.bfloat16][0], grads[torch.float32][0]) <= 5e-2, _rel(grads[torch.bfloat16][0], grads[torch.float32][0])
     assert _rel(grads[torch.bfloat16][1], grads[torch.float32][1]) <= 5e-2, _rel(grads[torch.bfloat16][1], grads[torch.float32][1])
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-5), (torch.bfloat16, 2e-2)])
+def test_block_recompute_same_dropout_in_both_passes(dev, dtype, tol):
+    """A training-mode block under autograd runs the fused launches forward and re-runs itself operator by operator
+    in the backward pass (``_BlockRecompute``): with dropout active both passes must apply the SAME multipliers.  The
+    multipliers of one call are captured, and the fused forward is compared with the operator-by-operator block run
+    on them; the gradients of the call are those of that run."""
+    from fastfold_amd.model.fastnn import Evoformer
+    torch.manual_seed(4)
+    s, r = 12, 40
+    blk = Evoformer(c_m=256, c_z=128, first_block=True, last_block=True).to(dev, dtype).train()
+    with torch.no_grad():
+        for n, p in blk.named_parameters():        # the zero-initialised output layers would hide every update
+            if p.dim() >= 2:
+                p.copy_(torch.randn_like(p) * p.shape[-1] ** -0.5)
+    m = torch.randn(s, r, 256, device=dev).to(dtype).requires_grad_()
+    z = torch.randn(r, r, 128, device=dev).to(dtype).requires_grad_()
+    mm = torch.ones(s, r, device=dev, dtype=dtype)
+    pm = torch.ones(r, r, device=dev, dtype=dtype)
+    seen = {}
+    draw = blk._draw_drops
+
+    def capture(a, b):
+        seen["d"] = draw(a, b)
+        return seen["d"]
+    blk._draw_drops = capture
+    mo, zo = blk(m, z, mm, pm)
+    d = seen["d"]
+    assert set(d) == {"row", "tmo", "tmi", "tas", "tae"}
+    for k, v in d.items():
+        assert v.shape == ((1, r, 1, 128) if k == "tae" else (1, 1, r, 256 if k == "row" else 128))
+        assert 0.4 < float((v != 0).float().mean()) < 0.99 and float(v.max()) > 1.0
+    cot = torch.randn_like(zo)
+    (zo.float() * cot.float()).sum().backward()
+    got = (m.grad.clone(), z.grad.clone())
+    pg = {n: p.grad.clone() for n, p in blk.named_parameters() if p.grad is not None}
+    blk.zero_grad()
+    m2, z2 = m.detach().clone().requires_grad_(), z.detach().clone().requires_grad_()
+    mo2, zo2 = blk._core_train(m2.unsqueeze(0), z2.unsqueeze(0), mm.unsqueeze(0), pm.unsqueeze(0), drops=d)
+    assert _rel(mo, mo2.squeeze(0)) <= tol and _rel(zo, zo2.squeeze(0)) <= tol, (_rel(mo, mo2.squeeze(0)), _rel(zo, zo2.squeeze(0)))
+    (zo2.squeeze(0).float() * cot.float()).sum().backward()
+    gtol = 1e-4 if dtype == torch.float32 else 5e-2      # atomics in the parameter gradients; bf16: one rounding step
+    assert _rel(got[0], m2.grad) <= gtol and _rel(got[1], z2.grad) <= gtol
+    assert len(pg) >= 70
+    for n, p in blk.named_parameters():
+        if n in pg and float(p.grad.float().norm()) > 1e-3:
+            assert _rel(pg[n], p.grad) <= gtol, n
+    # dropped updates really are dropped: with every multiplier zero the pair stack's dropped updates vanish
+    zero = {k: torch.zeros_like(v) for k, v in d.items()}
+    blk._draw_drops = lambda a, b: zero
+    with torch.enable_grad():
+        mo3, zo3 = blk(m.detach().requires_grad_(), z.detach().requires_grad_(), mm, pm)
+    mo4, zo4 = blk._core_train(m.detach().unsqueeze(0), z.detach().unsqueeze(0), mm.unsqueeze(0), pm.unsqueeze(0), drops=zero)
+    assert _rel(zo3, zo4.squeeze(0)) <= tol and _rel(mo3, mo4.squeeze(0)) <= tol
