@@ -231,11 +231,13 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     # the gate is not a tensor at all: the output stage computes sigmoid(Wg LN(x) + bg) from the rows of x it reads as
     # residual anyway and multiplies the heads' outputs by it on their way into the output projection
     # (ffk_gated_out_fused).  The projection launch then writes q, k, v only and the core reads no gate.
-    # Measured at N_seq = 128: with a million rows (N_res = 1024) the projection and the core each get ~ 3 % faster and
-    # the output stage as much slower - 1.3 GB less memory traffic per block at the same block time -; with 65 536 rows
-    # (N_res = 256) the non-persistent output stage loses 1.3 % of a block, so small launches keep the gate tensor.
-    gate_in_out = (_GATE_IN_OUT_STAGE and drop is None and M >= _GATE_IN_OUT_MIN_ROWS and acc_order and ln is not None and C in (128, 256)
-                   and HC == C and c_out == C and resid is not None and o_map is None
+    # Measured at N_seq = 128, same box: on the triangle attentions at N_res = 1024 the projection and the core each get
+    # ~ 3 % faster and the output stage as much slower - 1.1 GB less memory traffic per block at the same block time; at
+    # N_res = 256 the non-persistent output stage loses 1.3 % of a block, and on the MSA attentions (256 channels) it
+    # loses slightly at both sizes.  The choice depends on the row length and the width only, never on the number of
+    # batch rows: a subset of the batch rows must give the bits of the full call.
+    gate_in_out = (_GATE_IN_OUT_STAGE and drop is None and N >= _GATE_IN_OUT_MIN_N and C in _GATE_IN_OUT_WIDTHS and acc_order
+                   and ln is not None and HC == C and c_out == C and resid is not None and o_map is None
                    and resid.data_ptr() == x.data_ptr() and a_so % 16 == 0 and a_si % 16 == 0)
     gate = None
     if not gate_in_out:
@@ -390,7 +392,8 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
 _TRIMUL_CHAN_PAD = 64
 _PAIR_BIAS_RIDES = True      # see attention(): switch for same-box comparisons
 _GATE_IN_OUT_STAGE = True    # see attention(): False keeps the gate a tensor (written by the projection, read by the core)
-_GATE_IN_OUT_MIN_ROWS = 131072
+_GATE_IN_OUT_MIN_N = 512         # shortest attended axis for which the gate moves into the output stage
+_GATE_IN_OUT_WIDTHS = (128,)     # ... and the channel widths (the kernel is built for 128 and 256)
 
 
 def triangle_multiplication(z, out, *, r, C, c, incoming, ln1, w_pk, b_pk, n_glu, ln2, wout_pk, out_bias_pk, mask,

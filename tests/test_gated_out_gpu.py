@@ -107,13 +107,14 @@ def test_attention_gate_in_output_stage_matches_gate_tensor_path(dev):
         outs = []
         for on in (True, False):
             _fused._GATE_IN_OUT_STAGE = on
-            keep, _fused._GATE_IN_OUT_MIN_ROWS = _fused._GATE_IN_OUT_MIN_ROWS, 0       # small shapes take the path too
+            keep = (_fused._GATE_IN_OUT_MIN_N, _fused._GATE_IN_OUT_WIDTHS)
+            _fused._GATE_IN_OUT_MIN_N, _fused._GATE_IN_OUT_WIDTHS = 0, (128, 256)      # small shapes and the MSA width too
             try:
                 with torch.no_grad():
                     outs.append(mod(*args).float())
             finally:
                 _fused._GATE_IN_OUT_STAGE = True
-                _fused._GATE_IN_OUT_MIN_ROWS = keep
+                _fused._GATE_IN_OUT_MIN_N, _fused._GATE_IN_OUT_WIDTHS = keep
         upd = outs[1] - args[0].float()
         assert float(upd.norm()) > 1.0
         err = float((outs[0] - outs[1]).norm() / upd.norm())
