@@ -17,7 +17,7 @@ from fastfold_amd import _lib
 from fastfold_amd.model.fastnn.kernel import LayerNorm
 from . import _fused as F_
 from . import ops as _ops
-from .ops import Linear, _PackMixin, _no_grad_guard
+from .ops import Linear, _PackMixin, _needs_grad
 
 
 def _pad_cols(x, k):
@@ -58,11 +58,25 @@ class InputEmbedder(nn.Module, _PackMixin):
                     self.linear_relpos.bias.detach().to(dt).contiguous())
         return (ktf, kmsa) + self._packed(("ie", dt, dev), ps, build)
 
+    def _train(self, tf, ri, msa):
+        """embedders.py:99-135, operator by operator; the one-hot of the clipped offset selects a row of the
+        relative-position table."""
+        dt = self.linear_relpos.weight.dtype
+        tf, msa = tf.to(dt), msa.to(dt)
+        pair_emb = self.linear_tf_z_i(tf)[..., None, :] + self.linear_tf_z_j(tf)[..., None, :, :]
+        d = ri.to(torch.float32)
+        d = (d[..., None] - d[..., None, :]).clamp(-self.relpos_k, self.relpos_k)
+        d = torch.ceil(d - 0.5).long() + self.relpos_k                      # nearest offset, the lower one on a tie
+        pair_emb = pair_emb + (self.linear_relpos.weight.t()[d] + self.linear_relpos.bias)
+        msa_emb = self.linear_msa_m(msa) + self.linear_tf_m(tf).unsqueeze(-3)
+        return msa_emb, pair_emb
+
     def forward(self, tf: torch.Tensor, ri: torch.Tensor, msa: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         """tf [N_res, tf_dim], ri [N_res], msa [N_clust, N_res, msa_dim] ->
         (msa_emb [N_clust, N_res, C_m], pair_emb [N_res, N_res, C_z])."""
         F_.check_cuda(tf, ri, msa)
-        _no_grad_guard(self, tf, msa)
+        if _needs_grad(self, tf, msa):
+            return self._train(tf, ri, msa)
         if tf.dim() != 2 or msa.dim() != 3 or ri.dim() != 1:
             raise RuntimeError("InputEmbedder: expected tf [r, tf_dim], ri [r], msa [s, r, msa_dim] without batch "
                                "dimensions, got %s / %s / %s" % (tuple(tf.shape), tuple(ri.shape), tuple(msa.shape)))
@@ -98,12 +112,23 @@ class RecyclingEmbedder(nn.Module, _PackMixin):
         self.layer_norm_m = LayerNorm(self.c_m)
         self.layer_norm_z = LayerNorm(self.c_z)
 
+    def _train(self, m, z, x):
+        """embedders.py:207-232, operator by operator (open bin intervals on the squared distances, in fp32; the
+        coordinates receive no gradient: the one-hot is piecewise constant)."""
+        x = x.detach().to(torch.float32)
+        sq = torch.linspace(self.min_bin, self.max_bin, self.no_bins, dtype=torch.float32, device=x.device) ** 2
+        upper = torch.cat([sq[1:], sq.new_tensor([self.inf])], dim=-1)
+        d = torch.sum((x[..., None, :] - x[..., None, :, :]) ** 2, dim=-1, keepdim=True)
+        d = ((d > sq) * (d < upper)).to(z.dtype)
+        return self.layer_norm_m(m), self.linear(d) + self.layer_norm_z(z)
+
     def forward(self, m: torch.Tensor, z: torch.Tensor, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         """m [N_res, C_m] (first MSA row), z [N_res, N_res, C_z], x [N_res, 3] predicted C_beta coordinates ->
         (m_update, z_update).  As in the reference, z is overwritten when a chunk size is set
         (ops.py:1137-1143) and left untouched otherwise."""
         F_.check_cuda(m, z, x)
-        _no_grad_guard(self, m, z)
+        if _needs_grad(self, m, z, x):
+            return self._train(m, z, x)
         if z.dim() != 3 or z.shape[0] != z.shape[1] or x.shape != (z.shape[0], 3):
             raise RuntimeError("RecyclingEmbedder: expected z [r, r, c_z] and x [r, 3], got %s / %s"
                                % (tuple(z.shape), tuple(x.shape)))

@@ -187,6 +187,10 @@ class ExtraMSACore(nn.Module):
         self.MSATransition = ChunkTransition(d=d_node)
 
     def forward(self, node, pair, node_mask):
+        if _needs_grad(self, node, pair):
+            node = self.MSARowAttentionWithPairBias(node, pair, node_mask)
+            node = self.MSAColumnAttention(node, node_mask)
+            return self.MSATransition(node)
         node = node.contiguous()
         out = torch.empty_like(node)
         self.MSARowAttentionWithPairBias._run(node, pair, node_mask, out)
@@ -220,6 +224,15 @@ class ExtraMSABlock(nn.Module):
     def _core(self, m, z, msa_mask, pair_mask, inplace: bool):
         """m [1, s, r, c_m], z [1, r, r, c_z] contiguous, masks [1, s, r] / [1, r, r]."""
         F_.check_nonempty("ExtraMSABlock", m, z)
+        if _needs_grad(self, m, z):
+            # the reference's operator sequence (msa.py:226-258), nothing in place
+            if self.is_multimer:
+                z = self.communication(m, msa_mask, z)
+                m = self.msa_stack(m, z, msa_mask)
+                return m, self.pair_stack(z, pair_mask)
+            m = self.msa_stack(m, z, msa_mask)
+            z = self.communication(m, msa_mask, z)
+            return m, self.pair_stack(z, pair_mask)
         if self.is_multimer:
             # msa.py:252-258, 321-332: outer product mean first, the MSA stack reads the pair tensor it leaves,
             # the pair stack runs last

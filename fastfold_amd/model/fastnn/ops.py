@@ -574,11 +574,27 @@ class GlobalAttention(nn.Module, _PackMixin):
                                    gb_pk=gb, wo_pk=wo, ob_pk=ob, c_out=self.out_dim, mask=mask, mask_ss=mask_ss,
                                    mask_sr=mask_sr, eps=self.eps, budget=_budget())
 
+    def _train(self, m, mask):
+        """ops.py:1174-1197, operator by operator (the un-chunked branch)."""
+        from .kernel import bias_sigmod_ele, fused_softmax
+        mask = mask.to(m.dtype)
+        q = torch.sum(m * mask.unsqueeze(-1), dim=-2) / (torch.sum(mask, dim=-1)[..., None] + self.eps)
+        q = self.to_q(q * self.scaling)
+        q = q.view(q.shape[:-1] + (self.n_head, -1))                        # [1, R, H, c]
+        k, v = self.to_kv(m).chunk(2, dim=-1)                               # [1, R, S, c]
+        logits = torch.matmul(q, k.transpose(-1, -2))                       # [1, R, H, S]
+        weights = fused_softmax(logits.unsqueeze(-2), mask.contiguous()).squeeze(-2)
+        weighted_avg = torch.matmul(weights, v).flatten(-2)                 # [1, R, H * c]
+        gate_values = self.gating_linear(m)
+        weighted_avg = bias_sigmod_ele(gate_values, self.gating_bias, weighted_avg.unsqueeze(-2).expand_as(gate_values))
+        return self.o_linear(weighted_avg)
+
     def forward(self, m, mask):
         """m [1, batch_size2, len, qkv_dim] (already normalised), mask [1, batch_size2, len] ->
         [1, batch_size2, len, out_dim]."""
         F_.check_cuda(m, mask)
-        _no_grad_guard(self, m)
+        if _needs_grad(self, m):
+            return self._train(m, mask)
         if m.dim() != 4 or m.shape[0] != 1 or m.shape[-1] != self.qkv_dim:
             raise RuntimeError("GlobalAttention: expected [1, B2, N, %d] input, got %s" % (self.qkv_dim, tuple(m.shape)))
         _, R, S, C = m.shape
@@ -613,7 +629,15 @@ class ChunkMSAColumnGlobalAttention(nn.Module):
                                    ln=_ln_pair(self.layernormM, M_raw.dtype), mask=mask, mask_ss=r, mask_sr=1)
         return out
 
+    def _train(self, M_raw, M_mask):
+        """ops.py:1005-1010, operator by operator."""
+        m = self.layernormM(M_raw.transpose(-2, -3))
+        m = self.global_attention._train(m, M_mask.transpose(-1, -2))
+        return M_raw + m.transpose(-2, -3)
+
     def forward(self, M_raw, M_mask):
+        if _needs_grad(self, M_raw):
+            return self._train(M_raw, M_mask)
         M_raw = M_raw.contiguous()
         return self._run(M_raw, M_mask, torch.empty_like(M_raw))
 

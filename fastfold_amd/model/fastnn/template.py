@@ -18,7 +18,7 @@ from fastfold_amd import _lib
 from . import _fused as F_
 from .ops import (AsyncChunkTriangleMultiplicationIncoming, AsyncChunkTriangleMultiplicationOutgoing,
                   ChunkTransition, ChunkTriangleAttentionEndingNode, ChunkTriangleAttentionStartingNode, Linear,
-                  _PackMixin, _no_grad_guard)
+                  _PackMixin, _needs_grad, _no_grad_guard)
 
 
 class _PointwiseProjections(nn.Module):
@@ -78,10 +78,28 @@ class TemplatePointwiseAttention(nn.Module, _PackMixin):
         out = F_.linear(o, wo, (bo * any_valid).to(dt), self.c_z, out=resid, resid=resid)   # in place with a residual
         return out.view(r, r, self.c_z)
 
+    def _train(self, t, z, template_mask):
+        """template.py:100-127 with the generic attention of nn/primitives.py:390-440 written out (gating off): the
+        softmax runs over at most 8 templates per pair position, in fp32."""
+        m, H, D = self.mha, self.no_heads, self.c_hidden
+        if template_mask is None:
+            template_mask = t.new_ones(t.shape[0])
+        tm = template_mask.to(device=z.device, dtype=torch.float32)
+        q = m.linear_q(z).unflatten(-1, (H, D)) * (float(D) ** -0.5)           # [r, r, H, D]
+        k = m.linear_k(t).unflatten(-1, (H, D))                               # [NT, r, r, H, D]
+        v = m.linear_v(t).unflatten(-1, (H, D))
+        logits = (q.unsqueeze(0).float() * k.float()).sum(-1) + (self.inf * (tm - 1.0)).view(-1, 1, 1, 1)
+        w = torch.softmax(logits, dim=0).to(v.dtype)                           # [NT, r, r, H]
+        o = (w.unsqueeze(-1) * v).sum(0).flatten(-2)                           # [r, r, H * D]
+        return m.linear_o(o) * (tm.sum() > 0).to(z.dtype)
+
     def forward(self, t: torch.Tensor, z: torch.Tensor, template_mask: Optional[torch.Tensor] = None,
                 chunk_size: Optional[int] = None) -> torch.Tensor:
         """t [N_templ, N_res, N_res, C_t], z [N_res, N_res, C_z], template_mask [N_templ]
         -> the pair update [N_res, N_res, C_z] (not yet added to z)."""
+        if _needs_grad(self, t, z):
+            F_.check_cuda(t, z, template_mask)
+            return self._train(t, z, template_mask)
         return self._run(t, z, template_mask, None)
 
     def inplace(self, t: torch.Tensor, z: torch.Tensor, template_mask: Optional[torch.Tensor] = None,
@@ -122,6 +140,12 @@ class TemplatePairBlock(nn.Module):
     def _core(self, z, mask, inplace: bool):
         """z [1, r, r, c_t] contiguous, mask [1, r, r]; order as template.py:248-256."""
         F_.check_nonempty("TemplatePairBlock", z)
+        if _needs_grad(self, z):
+            z = self.TriangleAttentionStartingNode(z, mask)
+            z = self.TriangleAttentionEndingNode(z, mask)
+            z = self.TriangleMultiplicationOutgoing(z, mask)
+            z = self.TriangleMultiplicationIncoming(z, mask)
+            return self.PairTransition(z)
         out = z if inplace else torch.empty_like(z)
         self.TriangleAttentionStartingNode._run(z, mask, out)
         self.TriangleAttentionEndingNode._run(out, mask, out)
@@ -174,6 +198,14 @@ class TemplatePairStack(nn.Module):
             raise RuntimeError("TemplatePairStack: expected [N_templ, r, r, c_t], got %s" % (tuple(t.shape),))
         if mask.shape[-3] == 1:
             mask = mask.expand(t.shape[0], *mask.shape[-2:])
+        if _needs_grad(self, t):
+            outs = []
+            for i in range(t.shape[0]):
+                z = t[i:i + 1]
+                for b in self.blocks:
+                    z = b._core(z, mask[i:i + 1], inplace=False)
+                outs.append(self.layer_norm(z[0]))
+            return torch.stack(outs, 0)
         out = t if (inplace and t.is_contiguous()) else torch.empty_like(t, memory_format=torch.contiguous_format)
         for i in range(t.shape[0]):
             with F_.mask_cache():

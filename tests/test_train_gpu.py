@@ -10,7 +10,8 @@ their gradients it yields the gradients of the re-laid-out parameters.
 Tolerances: fp32 relative L2 <= 3e-3 per gradient tensor (1e-6 is what is measured when no ReLU input changes sign
 between the float32 run and the float64 oracle; one such flip among the 2 M hidden activations of the pair
 transition moves every upstream gradient by ~ 1e-3 of its norm, and about one is expected per block at these
-sizes); bf16 relative L2 <= 5e-2 on the input gradients.
+sizes); bf16 relative L2 <= 5e-2 on the input gradients and <= 1.5e-1 on the parameter gradients (see
+test_stack_gradients_with_checkpointing).
 """
 import copy
 
@@ -122,7 +123,7 @@ def test_stack_gradients_with_checkpointing(dev, dtype):
     cot = [torch.randn(s, r, KW["c_m"], generator=g), torch.randn(r, r, KW["c_z"], generator=g),
            torch.randn(r, KW["c_s"], generator=g)]
     _mask_cotangents(cot, r, 0.1)
-    _, ref_gin, _ = _oracle_run(model, m, z, mm, pm, cot)
+    _, ref_gin, ref_gp = _oracle_run(model, m, z, mm, pm, cot)
     fast = _fast(model, dev, dtype).train()
     for mod in fast.modules():
         if hasattr(mod, "p_drop"):
@@ -134,6 +135,19 @@ def test_stack_gradients_with_checkpointing(dev, dtype):
         out = fast(mi, zi, torch.from_numpy(mm).to(dev, dtype), torch.from_numpy(pm).to(dev, dtype), chunk_size=None)
         sum((o.float() * c.to(dev)).sum() for o, c in zip(out, cot)).backward()
         grads.append((mi.grad.clone(), zi.grad.clone()))
+        # parameter gradients against the oracle, in both precisions.  bf16: forward values differ from float64 by
+        # ~ 1e-2, so about that fraction of the transitions' ReLU inputs sit on the other side of zero and every
+        # gradient upstream of one moves by the square root of that fraction (4e-2 .. 1e-1 measured, uniformly)
+        pbound = 3e-3 if dtype == torch.float32 else 1.5e-1
+        checked = 0
+        for name, p in fast.named_parameters():
+            want = ref_gp[name].detach().double()
+            assert p.grad is not None and bool(torch.isfinite(p.grad.float()).all()), name
+            if dtype == torch.float32 or float(want.norm()) > 1.0:
+                err = float((p.grad.double().cpu() - want).norm())
+                assert err <= pbound * float(want.norm()) + 1e-3, (name, err, float(want.norm()))
+                checked += 1
+        assert checked >= 70 * nb, checked
         fast.zero_grad()
     if dtype == torch.float32:
         assert _rel(grads[0][0], grads[1][0]) <= 1e-4 and _rel(grads[0][1], grads[1][1]) <= 1e-4
@@ -141,6 +155,24 @@ def test_stack_gradients_with_checkpointing(dev, dtype):
     for gm, gz in grads:
         assert _rel(gm, ref_gin[0]) <= bound, _rel(gm, ref_gin[0])
         assert _rel(gz, ref_gin[1]) <= bound, _rel(gz, ref_gin[1])
+
+
+@pytest.mark.parametrize("rows,n,k", [(9216, 128, 128), (16384, 512, 128), (40960, 32, 256)])
+def test_linear_weight_gradient_slab_branch(dev, rows, n, k):
+    """bf16 projections over 8192 rows or more reduce their weight gradient in row slabs through a batched GEMM whose
+    partial sums are added in fp32: against float64 on the bf16 operands, <= 4e-3 relative L2 (one bf16 rounding of the
+    slab partial sums and one of the result), with the cotangent and the input sliced from one tensor (the operands
+    must reach the library in two allocations)."""
+    from fastfold_amd.model.fastnn.ops import Linear
+    g = torch.Generator().manual_seed(rows)
+    lin = Linear(k, n).to(dev, torch.bfloat16)
+    both = torch.randn(rows, n + k, generator=g).to(dev, torch.bfloat16)
+    cot, x = both[:, :n], both[:, n:].detach().requires_grad_()
+    lin(x).backward(cot)
+    want_w = cot.double().t() @ x.detach().double()
+    assert _rel(lin.weight.grad, want_w) <= 4e-3, _rel(lin.weight.grad, want_w)
+    assert _rel(lin.bias.grad, cot.double().sum(0)) <= 4e-3
+    assert _rel(x.grad, cot.double() @ lin.weight.detach().double()) <= 4e-3
 
 
 def test_block_chain_the_benchmark_way(dev):
