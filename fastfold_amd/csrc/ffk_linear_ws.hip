@@ -608,6 +608,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     int s_tile[NS], s_chan[NS], s_glu[NS], s_wrow[NS];
     WsSlot sp[NS];
     bool by_rows[NS];
+    int s_wl[NS];
     bf16x8 wf[NS][WS_KS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -638,8 +639,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
             sp[s].has_bias = ts.bias != nullptr;
             by_rows[s] = ws_by_rows(ts);
         }
-#pragma unroll
-        for (int ks = 0; ks < WS_KS; ++ks) wf[s][ks] = MM::ld(W + (long)(s_wrow[s] + wl) * WS_K + ks * 16 + half * 8);
+        s_wl[s] = wl;
     }
     const int rg_first = args.plan.rg_first[wave], rg_step = args.plan.rg_step[wave];
     // launches with channel-major tiles read the rows of a group through tau (16 consecutive rows per lane)
@@ -816,13 +816,51 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     }
     const int nslabs = (M + WS_BM - 1) / WS_BM;
     int slab = blockIdx.x;                               // grid <= nslabs
-    fetch(slab, 0);
+    fetch(slab, 0);                                      // the first slab travels while the weights are fetched
+    // ---- weights: every wave reads the 32 rows of its slots as whole lines (a lane's fragments are 16-byte pieces
+    // 32 bytes apart in one row, 32 rows per request: fetched that way every request touches 32 lines and uses a
+    // quarter of each, and a workgroup's 128 .. 256 KB of weights do not stay in the first-level cache between the
+    // K steps) and re-orders them through a private piece of the slab buffer, which is idle until the first commit.
+    // A piece is 32 rows x PW channels; its 16-byte chunks are stored at chunk ^ (row % LR) so that the fragment
+    // reads (one row per lane) spread over the banks.
+    {
+        constexpr int PW = WS_K < 128 ? WS_K : 128;      // channels per piece
+        constexpr int LR = PW / 8;                       // 16-byte chunks (lanes) per row of a piece
+        constexpr int NI = 32 / (64 / LR);               // requests per piece = K steps per piece
+        constexpr int NP = WS_K / PW;                    // pieces per slot
+        static_assert(NI * NP == WS_KS, "piece geometry");
+        static_assert(WS_WAVES * 32 * PW * 2 <= 2 * WS_BM * WS_AP, "the staging area is the slab buffer");
+        unsigned char* stage = s_a + wave * (32 * PW * 2);
+        const int lrow = lane / LR, lcol = lane % LR;
+#pragma unroll
+        for (int sl = 0; sl < NS; ++sl)
+#pragma unroll
+            for (int pc = 0; pc < NP; ++pc)
+#pragma unroll
+                for (int i = 0; i < NI; ++i)
+                    wf[sl][pc * NI + i] = MM::ld(W + (long)(s_wrow[sl] + i * (64 / LR) + lrow) * WS_K + pc * PW + lcol * 8);
+#pragma unroll
+        for (int sl = 0; sl < NS; ++sl)
+#pragma unroll
+            for (int pc = 0; pc < NP; ++pc) {
+#pragma unroll
+                for (int i = 0; i < NI; ++i) {
+                    const int row = i * (64 / LR) + lrow;
+                    *reinterpret_cast<bf16x8*>(stage + row * (PW * 2) + ((lcol ^ (row & (LR - 1))) * 16)) = wf[sl][pc * NI + i];
+                }
+#pragma unroll
+                for (int k = 0; k < NI; ++k)
+                    wf[sl][pc * NI + k] = *reinterpret_cast<const bf16x8*>(
+                        stage + s_wl[sl] * (PW * 2) + (((2 * k + half) ^ (s_wl[sl] & (LR - 1))) * 16));
+            }
+    }
+    lds_barrier();                                       // every wave is done with the staging area
     commit(0);
     lds_barrier();
     int buf = 0;
     for (; slab < nslabs; slab += gridDim.x) {
-        const int nxt = slab + (int)gridDim.x < nslabs ? slab + (int)gridDim.x : slab;
-        fetch(nxt, buf ^ 1);                             // in flight during the products below
+        const bool more = slab + (int)gridDim.x < nslabs;
+        if (more) fetch(slab + (int)gridDim.x, buf ^ 1);  // in flight during the products below
         const unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
         if (PB && pb_tile >= 0) {
             // pair bias of this slab: thread -> (row tid / 4, head tid % 4); the row is the operand as the products
@@ -1051,6 +1089,7 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
                 }
             }
         }
+        if (!more) break;                                // nothing left to commit: the stores drain on their own
         commit(buf ^ 1);
         lds_barrier();
         buf ^= 1;
