@@ -157,7 +157,8 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
         } else {
             int qq = wg_q * 4 + (tile - 4);
             qq = qq < QT ? qq : QT - 1;
-            base = bias_t + ((((long)h * QT + qq) * KT) << 10);
+            // FFK_ATT_BIAS_PADDED: one unused tile after the KT tiles of each query-tile row
+            base = bias_t + ((((long)h * QT + qq) * (KT + ((flags >> 1) & 1))) << 10);
         }
         // the wave's 64 vectors of this request: vector number wv / 64 of every lane's 16 elements
         src[i] = base + (wv / 64) * VEC;
@@ -587,7 +588,8 @@ extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, co
                 "ffk_attention_fwd: head dimension %ld (32, 64 or 128; narrower heads arrive zero-padded to 32)", (long)D);
     hipStream_t st = (hipStream_t)stream;
     if (D != 32) {
-        FFK_REQUIRE(!gate, FFK_ERR_UNSUPPORTED, "ffk_attention_fwd: the gate is built for head dimension 32 only");
+        FFK_REQUIRE(!gate && !(flags & FFK_ATT_BIAS_PADDED), FFK_ERR_UNSUPPORTED,
+                    "ffk_attention_fwd: the gate and padded bias rows are built for head dimension 32 only");
         if (dtype == FFK_BF16)
             return D == 64 ? launch_attention_wide<bf16_t, 2>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st)
                            : launch_attention_wide<bf16_t, 4>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st);

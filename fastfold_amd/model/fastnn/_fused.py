@@ -247,14 +247,22 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     qscale = LOG2E / math.sqrt(float(head_dim))
     tkw = dict(inner=N, s_o=H * NT * 1024, s_h=NT * 1024)
     bias_tile = None
+    # rows of a bias buffer the caller leaves to this function (bias_in_launch with bias_t None) end in one unused tile
+    # when the projection launch writes them: with 2^n key tiles per row every query-tile row would start in the same
+    # memory channel (-2 % per triangle-attention launch at N = 1024, measured three times on one box)
+    will_ride = (bias_in_launch and acc_order and C == 128 and H <= 4 and slab >= B2 and _PAIR_BIAS_RIDES
+                 and (not gate_in_out or hasattr(w_pk, "without_gate")))
+    bias_padded = will_ride and _BIAS_ROW_PAD and bias_t is None
     if bias_in_launch:
-        bias_tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=NT * 1024, s_h=NT * NT * 1024, ncols=H,
+        ntp = NT + (1 if bias_padded else 0)
+        if bias_t is None:
+            bias_t = alloc((H, NT, ntp, 1024), dt, dev, zero=(N % 32) != 0)
+        bias_tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=ntp * 1024, s_h=NT * ntp * 1024, ncols=H,
                               scale=LOG2E)
     # With 128 input channels, at most four heads and all rows in one slab the bias rides on the projection launch:
     # the weights-stationary kernel computes its four dot products per row on the vector pipe from the rows it
     # has in LDS anyway (one read of x less than a pass of its own; -0.05 ms per triangle attention at N = 1024).
-    rides = (bias_tile is not None and acc_order and C == 128 and H <= 4 and slab >= B2 and _PAIR_BIAS_RIDES
-             and (not gate_in_out or hasattr(w_pk, "without_gate")))
+    rides = will_ride
     # Otherwise the skinny bias projection has its own pass over x.  It goes first: x was written by the launch before
     # this call and is still (partly) cache-resident, and the bias pass writes little, so the projection after
     # it finds x as warm as before - the other way round the projection's output (four times the size of x)
@@ -302,7 +310,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
             _lib.fused_linear(x, wp, tiles[t0:t0 + per], M=Ms, K=C, a_inner=inner, a_so=a_so, a_si=a_si, ln=ln,
                               w_row_off=t0 * 128, a_off=off)
         _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb[b0:b0 + nb], flags[b0:b0 + nb], gate, B2=nb, H=H, Nq=N, Nk=N,
-                           gate_tiled=acc_order)
+                           gate_tiled=acc_order, bias_padded=bias_padded)
         if gate_in_out:
             # packed rows of w_pk: q, k, v, gate blocks of HC rows each; o holds the slab's rows in logical order
             _lib.gated_out_fused(out.data_ptr() + o_off * es, x.data_ptr() + off * es, ln[0], ln[1],
@@ -391,6 +399,7 @@ def trimul_gate_in_output_stage(dtype, r, C, c):
 # (block 6.97 -> 6.885 ms in a same-box A/B at N_res = 1024; 64, 192 and 1088 elements measure the same).
 _TRIMUL_CHAN_PAD = 64
 _PAIR_BIAS_RIDES = True      # see attention(): switch for same-box comparisons
+_BIAS_ROW_PAD = True         # see attention(): switch for same-box comparisons
 _GATE_IN_OUT_STAGE = True    # see attention(): False keeps the gate a tensor (written by the projection, read by the core)
 _GATE_IN_OUT_MIN_N = 512         # shortest attended axis for which the gate moves into the output stage
 _GATE_IN_OUT_WIDTHS = (128,)     # ... and the channel widths (the kernel is built for 128 and 256)

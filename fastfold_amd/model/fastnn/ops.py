@@ -778,8 +778,6 @@ class _TriangleAttention(nn.Module, _PackMixin):
         ob = self._packed(("ob", dt, dev), [self.out_bias], lambda: F_.pack_vec([self.out_bias], dt, dev))
         pbs = self._packed(("pbs", dt, dev), [self.linear_b.weight, self.layernorm1.weight, self.layernorm1.bias],
                            lambda: F_.PairBiasScratch(C, dev))
-        NT = (r + 31) // 32
-        bias_t = F_.alloc((self.n_head, NT, NT, 1024), dt, dev, zero=(r % 32) != 0)
         mask = _mask_like(Z_mask, Z_raw)[0]
         if self._ending:    # logical row (j, i) reads z[i, j]; keys run along i
             a_map, sb, sn = (r, C, r * C), 1, r
@@ -787,7 +785,7 @@ class _TriangleAttention(nn.Module, _PackMixin):
             a_map, sb, sn = (r * r, 0, C), r, 1
         F_.attention(Z_raw, out, Z_raw, B2=r, N=r, C=C, H=self.n_head, a_map=a_map,
                      ln=_ln_pair(self.layernorm1, dt), w_pk=w_pk, gate_bias_pk=gb_pk, wo_pk=wo_pk, out_bias_pk=ob,
-                     c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=bias_t, bias_in_launch=True, pb_scratch=pbs,
+                     c_out=C, mask=mask, mask_sb=sb, mask_sn=sn, bias_t=None, bias_in_launch=True, pb_scratch=pbs,
                      head_dim=self.c, budget=_budget(), xtail=_check_tail(xtail, Z_raw),
                      drop=None if drop is None else drop.reshape(r, C).contiguous())     # logical row m: key index m % r
         return out

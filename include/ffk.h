@@ -269,7 +269,9 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  *   q_t, k_t : [B2][H][ceil(N/32)][1024]   FFK_TILE_QK or FFK_TILE_ACC order (the same for both)
  *   v_t      : [B2][H][ceil(Nk/32)][1024]  FFK_TILE_V  order
  *   bias_t   : [H][ceil(Nq/32)][ceil(Nk/32)][1024]  FFK_TILE_BIAS order (keys x queries as an
- *              MFMA operand: element (k, q) at (q%32/16)*512 + (k%32)*16 + q%16), or NULL
+ *              MFMA operand: element (k, q) at (q%32/16)*512 + (k%32)*16 + q%16), or NULL; with
+ *              FFK_ATT_BIAS_PADDED in flags [H][ceil(Nq/32)][ceil(Nk/32) + 1][1024]: one unused tile ends every
+ *              query-tile row, so that rows of 2^n key tiles do not start in the same memory channel (D = 32 only)
  *   keybias  : [B2][ceil(Nk/32)*32] fp32
  *   tileflags: [B2][ceil(Nk/32)] int32 per 32-key tile: 0 all keys valid, 1 mixed, 2 all masked
  *   gate     : multiplicative gate (already sigmoid-ed) or NULL: [B2*Nq, H*32] row-major, or with
@@ -282,7 +284,7 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  * SelfAttention.forward (fastfold/model/fastnn/ops.py:310-322) and
  * fused_attention_core (kernel/attention_core.py:17-52, kernel/triton/attention_core.py:12-190).
  */
-enum { FFK_ATT_GATE_TILED = 1 };
+enum { FFK_ATT_GATE_TILED = 1, FFK_ATT_BIAS_PADDED = 2 };
 int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t,
                       const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
                       int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int64_t D, int flags, int dtype, void* stream);
