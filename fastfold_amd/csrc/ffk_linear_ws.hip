@@ -594,16 +594,6 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     const T* A = (const T*)d.a;
     const T* W = (const T*)d.w;
 
-    // ---- bias table: no global loads in the epilogues ----
-    for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) {
-        const ffk_tile& tb = d.tiles[i >> 7];
-        const T* bp = (const T*)tb.bias;
-        // gate halves of a GLU unit ([p 32 | g 32 | p 32 | g 32]) and sigmoid tiles: pre-multiplied for ws_sigmoid_pre
-        const bool sig = tb.glu ? ((i >> 5) & 1) != 0 : tb.act == FFK_ACT_SIGMOID;
-        const float b = bp ? (float)bp[i & 127] : 0.0f;
-        s_bias[i] = sig ? -1.4426950408889634f * b : b;
-    }
-
     // ---- this wave's weight slots, resident in registers ----
     int s_tile[NS], s_chan[NS], s_glu[NS], s_wrow[NS];
     WsSlot sp[NS];
@@ -651,20 +641,6 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
     // both slabs are used as they arrive (see ws_store_rows_folded)
     const bool folded = DUAL;
     const bool ln = d.ln_gamma != nullptr && !folded;
-    {
-        if (folded) {
-            for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) s_c1[i] = ((const float*)d.ln_gamma)[i];
-        }
-        if (ln && !CM && tid < WS_K) {
-            s_ln1[tid] = ((const T*)d.ln_gamma)[tid];
-            s_ln1[WS_K + tid] = ((const T*)d.ln_beta)[tid];
-        }
-        if (ln && CM && tid < WS_K) {
-            s_cmln[tid] = (float)((const T*)d.ln_gamma)[tid];
-            s_cmln[WS_K + tid] = (float)((const T*)d.ln_beta)[tid];
-        }
-        lds_barrier();
-    }
     // row mask of the launch (all masked tiles share it): fetched with the slab, kept in LDS as fp32
     const int mt = args.plan.mask_tile;
     const T* rm = mt >= 0 ? (const T*)d.tiles[mt].rowmask : nullptr;
@@ -808,14 +784,9 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         }
     };
 
-    const int pb_tile = PB ? args.plan.bias_tile : -1;
-    if (PB && pb_tile >= 0) {
-        const int heads = d.tiles[pb_tile].ncols;
-        for (int i = tid; i < 4 * WS_K; i += WS_THREADS)
-            s_wb[i] = (i / WS_K) < heads ? W[(long)(pb_tile * 128 + i / WS_K) * WS_K + (i % WS_K)] : (T)0.0f;
-    }
     const int nslabs = (M + WS_BM - 1) / WS_BM;
     int slab = blockIdx.x;                               // grid <= nslabs
+    const int pb_tile = PB ? args.plan.bias_tile : -1;
     fetch(slab, 0);                                      // the first slab travels while the weights are fetched
     // ---- weights: every wave reads the 32 rows of its slots as whole lines (a lane's fragments are 16-byte pieces
     // 32 bytes apart in one row, 32 rows per request: fetched that way every request touches 32 lines and uses a
@@ -839,6 +810,35 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
 #pragma unroll
                 for (int i = 0; i < NI; ++i)
                     wf[sl][pc * NI + i] = MM::ld(W + (long)(s_wrow[sl] + i * (64 / LR) + lrow) * WS_K + pc * PW + lcol * 8);
+        // tables the epilogues and the commits read from LDS (no global loads there); the barrier in front of the first
+        // commit publishes them
+        for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) {
+            const ffk_tile& tb = d.tiles[i >> 7];
+            const T* bp = (const T*)tb.bias;
+            // gate halves of a GLU unit ([p 32 | g 32 | p 32 | g 32]) and sigmoid tiles: pre-multiplied for ws_sigmoid_pre
+            const bool sig = tb.glu ? ((i >> 5) & 1) != 0 : tb.act == FFK_ACT_SIGMOID;
+            const float b = bp ? (float)bp[i & 127] : 0.0f;
+            s_bias[i] = sig ? -1.4426950408889634f * b : b;
+        }
+
+        {
+            if (folded) {
+                for (int i = tid; i < d.n_tiles * 128; i += WS_THREADS) s_c1[i] = ((const float*)d.ln_gamma)[i];
+            }
+            if (ln && !CM && tid < WS_K) {
+                s_ln1[tid] = ((const T*)d.ln_gamma)[tid];
+                s_ln1[WS_K + tid] = ((const T*)d.ln_beta)[tid];
+            }
+            if (ln && CM && tid < WS_K) {
+                s_cmln[tid] = (float)((const T*)d.ln_gamma)[tid];
+                s_cmln[WS_K + tid] = (float)((const T*)d.ln_beta)[tid];
+            }
+        }
+        if (PB && pb_tile >= 0) {
+            const int heads = d.tiles[pb_tile].ncols;
+            for (int i = tid; i < 4 * WS_K; i += WS_THREADS)
+                s_wb[i] = (i / WS_K) < heads ? W[(long)(pb_tile * 128 + i / WS_K) * WS_K + (i % WS_K)] : (T)0.0f;
+        }
 #pragma unroll
         for (int sl = 0; sl < NS; ++sl)
 #pragma unroll
