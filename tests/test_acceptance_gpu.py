@@ -327,4 +327,6 @@ def test_chunked_extra_msa_block_equals_unchunked(dev, dtype, tiny_budget, monke
         col.inplace(mi, tmm[None])
         return mi[0]
     a, b = _run_both(inplace)
-    assert torch.equal(a, b) and torch.equal(a, col(tm[None], tmm[None]))
+    with torch.no_grad():                      # (with gradients enabled the module would take its differentiable path)
+        fwd = col(tm[None], tmm[None])
+    assert torch.equal(a, b) and torch.equal(a, fwd)
