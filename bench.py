@@ -246,13 +246,13 @@ def long_sequence(dev):
             "tflops": round(block_gflop(s, r) / ms, 1), "peak_device_GB": round(torch.cuda.max_memory_allocated() / 1e9, 1)}
 
 
-def forward_backward(dev, layers=4, trials=5, warm=2):
+def forward_backward(dev, layers=4, trials=5, warm=2, r=256):
     """The reference's own harness shape (benchmark/perf.py:83-183): stand-alone blocks in training mode (dropout
-    active), bf16, N_seq = 128, N_res = 256, inputs that require gradients, ``layer_inputs[1].backward(grads)``;
+    active), bf16, N_seq = 128, N_res = 256 (``r``), inputs that require gradients, ``layer_inputs[1].backward(grads)``;
     HIP-event times of the forward and of the backward pass per layer."""
     import torch
     from fastfold_amd.model.fastnn import Evoformer
-    s, r = 128, 256
+    s = 128
     torch.manual_seed(0)
     blocks = [Evoformer(c_m=256, c_z=128, first_block=(i == 0), last_block=(i == layers - 1)).to(dev, torch.bfloat16)
               for i in range(layers)]
@@ -276,7 +276,7 @@ def forward_backward(dev, layers=4, trials=5, warm=2):
         if t >= warm:
             fwd += e0.elapsed_time(e1)
             bwd += e1.elapsed_time(e2)
-    return {"workload": "benchmark/perf.py shape: %d stand-alone blocks, training mode, bf16, N_seq=128, N_res=256" % layers,
+    return {"workload": "benchmark/perf.py shape: %d stand-alone block(s), training mode, bf16, N_seq=128, N_res=%d" % (layers, r),
             "fwd_ms_per_block": round(fwd / trials / layers, 3), "bwd_ms_per_block": round(bwd / trials / layers, 3)}
 
 
@@ -469,6 +469,8 @@ def main():
         torch.cuda.empty_cache()
     if not args.no_forward_backward and not args.no_micro:
         line["forward_backward"] = forward_backward(dev)
+        if args.workload == "cfg4":         # the same at the headline size: one block, forward + backward
+            line["forward_backward_n_res_1024"] = forward_backward(dev, layers=1, trials=2, warm=1, r=1024)
         torch.cuda.empty_cache()
     if not args.no_micro:
         line["feeders"] = feeder_stacks(dev, r)
