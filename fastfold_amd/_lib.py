@@ -278,6 +278,19 @@ def attention_bwd(dq, dk, dv, dbias, lse, dsum, q_qk, q_acc, k_qk, k_acc, v_qk, 
 
 
 SIGNATURES["ffk_tile_pack"] = [_P, _P, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I, _P]
+SIGNATURES["ffk_transpose_batched"] = [_P, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]
+
+
+def transpose_batched(out, inp, *, B, X, Y, in_bs, in_xs, out_bs, out_ys, out_off=0, in_off=0):
+    """out[b][y][x] = in[b][x][y] with element strides (see include/ffk.h); ``out_off`` / ``in_off``: element offsets
+    added to the tensors' data pointers."""
+    if not (out.is_cuda and inp.is_cuda) or out.device != inp.device:
+        raise RuntimeError("fastfold_amd: tensors must be CUDA/HIP tensors on one device (got %s / %s)" % (out.device, inp.device))
+    if out.dtype != inp.dtype:
+        raise RuntimeError("transpose_batched: dtype mismatch %s / %s" % (out.dtype, inp.dtype))
+    es = inp.element_size()
+    call("ffk_transpose_batched", out.data_ptr() + out_off * es, inp.data_ptr() + in_off * es, B, X, Y, in_bs, in_xs,
+         out_bs, out_ys, dtype_tag(inp.dtype), stream_ptr())
 
 
 def tile_pack(x, kind, scale=1.0):

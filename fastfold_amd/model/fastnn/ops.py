@@ -161,6 +161,82 @@ def _chan_major(t, perm):
     return _padded_copy(permute_final_dims(t, perm)[0])
 
 
+def _cm_alloc(c, r, dtype, device):
+    """[c, r, kpad] with the last axis padded to the GEMM kernels' 16-byte K step; zeroed where padding exists."""
+    kpad = F_.round_up(r, F_.vec_of(dtype))
+    return (torch.zeros if kpad != r else torch.empty)(c, r, kpad, dtype=dtype, device=device)
+
+
+def _transpose_cm(x, r):
+    """[c, r, kpad] channel-major -> [c, r, kpad] with the two row indices exchanged: out[c, k, j] = x[c, j, k]."""
+    c, _, kpad = x.shape
+    out = _cm_alloc(c, r, x.dtype, x.device)
+    _lib.transpose_batched(out, x, B=c, X=r, Y=r, in_bs=x.stride(0), in_xs=x.stride(1), out_bs=r * kpad, out_ys=kpad)
+    return out
+
+
+class _ToChanMajorFn(torch.autograd.Function):
+    """lr [1, r, r, 2c] (channels contiguous) -> (L, R), each [c, r, kpad] channel-major in an allocation of its own:
+    L[ch, i, k] = lr[0, i, k, ch] (outgoing) or lr[0, k, i, ch] (incoming), R the same from channels c .. 2c - 1
+    (the permute_final_dims of fastnn/ops.py:400-403, 529-532).  One transposition launch per operand, forward and
+    backward; the backward pass writes both halves of the gradient of ``lr`` in place (no concatenation)."""
+
+    @staticmethod
+    def forward(ctx, lr, incoming):
+        _, r, r2, c2 = lr.shape
+        if r != r2 or lr.stride(3) != 1 or c2 % 2:
+            raise RuntimeError("_ToChanMajorFn: expected [1, r, r, 2c] with contiguous channels, got %s strides %s"
+                               % (tuple(lr.shape), lr.stride()))
+        c = c2 // 2
+        s_i, s_k = (lr.stride(2), lr.stride(1)) if incoming else (lr.stride(1), lr.stride(2))
+        outs = []
+        for side in range(2):
+            out = _cm_alloc(c, r, lr.dtype, lr.device)
+            _lib.transpose_batched(out, lr, B=r, X=r, Y=c, in_bs=s_i, in_xs=s_k, out_bs=out.stride(1),
+                                   out_ys=out.stride(0), in_off=side * c)
+            outs.append(out)
+        ctx.incoming, ctx.r, ctx.c = incoming, r, c
+        return outs[0], outs[1]
+
+    @staticmethod
+    def backward(ctx, dL, dR):
+        r, c = ctx.r, ctx.c
+        ref = dL if dL is not None else dR
+        g = torch.empty(1, r, r, 2 * c, dtype=ref.dtype, device=ref.device)
+        s_i, s_k = (g.stride(2), g.stride(1)) if ctx.incoming else (g.stride(1), g.stride(2))
+        for side, d in enumerate((dL, dR)):
+            if d is None:
+                g[..., side * c:(side + 1) * c].zero_()
+                continue
+            d = d.contiguous()
+            # g[0, i, k, side c + ch] = d[ch, i, k]: per i the [ch, k] matrix transposed
+            _lib.transpose_batched(g, d, B=r, X=c, Y=r, in_bs=d.stride(1), in_xs=d.stride(0), out_bs=s_i, out_ys=s_k,
+                                   out_off=side * c)
+        return g, None
+
+
+class _FromChanMajorFn(torch.autograd.Function):
+    """p [c, r, npad] channel-major -> [1, r, r, c] contiguous (the permute_final_dims(p, (1, 2, 0)) of
+    fastnn/ops.py:404, :533), one transposition launch each way."""
+
+    @staticmethod
+    def forward(ctx, p, r):
+        c = p.shape[0]
+        p = p.contiguous()
+        out = torch.empty(1, r, r, c, dtype=p.dtype, device=p.device)
+        _lib.transpose_batched(out, p, B=r, X=c, Y=r, in_bs=p.stride(1), in_xs=p.stride(0), out_bs=r * c, out_ys=c)
+        ctx.r, ctx.c, ctx.npad = r, c, p.shape[2]
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        r, c = ctx.r, ctx.c
+        g = g.contiguous()
+        dp = _cm_alloc(c, r, g.dtype, g.device)
+        _lib.transpose_batched(dp, g, B=r, X=r, Y=c, in_bs=r * c, in_xs=c, out_bs=dp.stride(1), out_ys=dp.stride(0))
+        return dp, None
+
+
 def _bgemm_cm(a, b, n_valid):
     """out[c, i, j] = sum_k a[c, i, k] b[c, j, k] for j < n_valid (rows of b past n_valid are padding) through
     ``ffk_bgemm_nt`` (the library's own batched NT GEMM, the kernel the fused path's contraction runs on); the
@@ -192,9 +268,9 @@ class _TriContractFn(torch.autograd.Function):
         dp = dp.contiguous()
         dL = dR = None
         if ctx.needs_input_grad[0]:      # dL[c, i, k] = sum_j dp[c, i, j] R[c, j, k]: K runs over j
-            dL = _bgemm_cm(dp, _padded_copy(R.transpose(1, 2)[:, :r]), r)
+            dL = _bgemm_cm(dp, _transpose_cm(R, r), r)
         if ctx.needs_input_grad[1]:      # dR[c, j, k] = sum_i dp[c, i, j] L[c, i, k]: K runs over i
-            dR = _bgemm_cm(_padded_copy(dp[:, :, :r].transpose(1, 2)), _padded_copy(L.transpose(1, 2)[:, :r]), r)
+            dR = _bgemm_cm(_transpose_cm(dp, r), _transpose_cm(L, r), r)
         return dL, dR, None
 
 
@@ -712,14 +788,14 @@ class _TriangleMultiplication(nn.Module, _PackMixin):
         Z = self.layernorm1(Z_raw)
         lr = Z_mask.unsqueeze(-1).to(Z.dtype) * self.left_right_projection(Z)
         lr = lr * torch.sigmoid(self.left_right_gate(Z))
-        left, right = lr.chunk(2, dim=-1)
         g = torch.sigmoid(self.output_gate(Z))
-        # channel-major operands [c, i, k] / [c, j, k] in two allocations of their own, the contraction and its two
-        # backward products on the library's own batched GEMM kernel
+        # channel-major operands [c, i, k] / [c, j, k] in two allocations of their own (incoming: L[c, i, k] =
+        # left[k, i, c]), the contraction and its two backward products on the library's own batched GEMM kernel, the
+        # re-orderings on both sides on the library's transposition kernel
         r = Z_raw.shape[1]
-        perm = (2, 1, 0) if self._incoming else (2, 0, 1)      # incoming: L[c, i, k] = left[k, i, c]
-        p = _TriContractFn.apply(_chan_major(left, perm), _chan_major(right, perm), r)[None, :, :, :r]
-        ab = self.output_projection(self.layernorm2(permute_final_dims(p, (1, 2, 0))))
+        left, right = _ToChanMajorFn.apply(lr.contiguous(), self._incoming)
+        p = _FromChanMajorFn.apply(_TriContractFn.apply(left, right, r), r)
+        ab = self.output_projection(self.layernorm2(p))
         if drop is not None:
             return bias_ele_dropout_residual(ab, self.output_bias, g, drop, Z_raw, prob=0.0, training=False)
         dropout_mask = torch.ones_like(Z[:, 0:1, :, :])

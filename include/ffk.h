@@ -325,6 +325,16 @@ int ffk_attention_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, fl
 int ffk_tile_pack(void* dst, const void* src, int64_t B2, int64_t H, int64_t N, int64_t D, int64_t s_b, int64_t s_h,
                   int64_t s_n, float scale, int kind, int dtype, void* stream);
 
+/* Batched 2-D transposition with strides (all strides in elements):
+ *     out[b][y][x] = in[b][x][y]      for b < B, x < X, y < Y,
+ * in element (b, x, y) at in + b*in_bs + x*in_xs + y (y contiguous), out element (b, y, x) at
+ * out + b*out_bs + y*out_ys + x (x contiguous); elements of 2 bytes (FFK_BF16, FFK_F16) or 4 bytes (FFK_F32).  Bytes
+ * of out that no (b, y, x) addresses (padding columns) are left as they are.  out and in must not overlap.
+ * Replaces: the permute_final_dims(...) + contiguous copies in front of the batched matmuls of the triangle
+ * multiplications and of their backward passes (fastfold/model/fastnn/ops.py:400-403, 529-532). */
+int ffk_transpose_batched(void* out, const void* in, int64_t B, int64_t X, int64_t Y, int64_t in_bs, int64_t in_xs,
+                          int64_t out_bs, int64_t out_ys, int dtype, void* stream);
+
 /* Pair bias of a biased attention, straight into the operand tiles ffk_attention_fwd reads:
  *     bias_t[h][q/32][k/32][tile(k, q)] = scale * ( LayerNorm(z[q, k, :]; gamma, beta, eps) . w[h, :] )
  * z holds N*N rows of C channels; logical row m = q*N + k lives at (m / a_inner) * a_so + (m % a_inner) * a_si

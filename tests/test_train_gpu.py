@@ -363,3 +363,60 @@ def test_block_recompute_same_dropout_in_both_passes(dev, dtype, tol):
         mo3, zo3 = blk(m.detach().requires_grad_(), z.detach().requires_grad_(), mm, pm)
     mo4, zo4 = blk._core_train(m.detach().unsqueeze(0), z.detach().unsqueeze(0), mm.unsqueeze(0), pm.unsqueeze(0), drops=zero)
     assert _rel(zo3, zo4.squeeze(0)) <= tol and _rel(mo3, mo4.squeeze(0)) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,X,Y", [(3, 64, 64), (2, 70, 33), (5, 1, 9), (1, 129, 200), (4, 40, 128), (2, 8, 8)])
+def test_transpose_batched_kernel(dev, dtype, B, X, Y):
+    """out[b][y][x] = in[b][x][y] with strides: contiguous operands, views with larger pitches (padding that must stay
+    untouched), a batch stride smaller than a row stride (the batch index is the inner one), and pointers off the
+    16-byte grid (element-wise branches)."""
+    from fastfold_amd import _lib
+    g = torch.Generator().manual_seed(B * 100 + X + Y)
+    x = torch.randn(B, X, Y, generator=g).to(dev, dtype)
+    out = torch.empty(B, Y, X, dtype=dtype, device=dev)
+    _lib.transpose_batched(out, x, B=B, X=X, Y=Y, in_bs=X * Y, in_xs=Y, out_bs=X * Y, out_ys=X)
+    assert torch.equal(out, x.transpose(1, 2))
+    # padded pitches on both sides, element offsets into the buffers
+    xp = torch.randn(B, X + 2, Y + 5, generator=g).to(dev, dtype)
+    op = torch.full((B, Y + 1, X + 3), 7.0, dtype=dtype, device=dev)
+    _lib.transpose_batched(op, xp, B=B, X=X, Y=Y, in_bs=xp.stride(0), in_xs=xp.stride(1), out_bs=op.stride(0),
+                           out_ys=op.stride(1), in_off=xp.stride(1) + 3, out_off=op.stride(1) + 2)
+    assert torch.equal(op[:, 1:, 2:2 + X], xp[:, 1:1 + X, 3:3 + Y].transpose(1, 2))
+    keep = op.clone()
+    keep[:, 1:, 2:2 + X] = 7.0
+    assert float((keep - 7.0).abs().max()) == 0.0                       # nothing outside the addressed elements
+    # the batch index as the inner one: in[x][b][y] -> out[y][b][x]
+    xi = torch.randn(X, B, Y, generator=g).to(dev, dtype)
+    oi = torch.empty(Y, B, X, dtype=dtype, device=dev)
+    _lib.transpose_batched(oi, xi, B=B, X=X, Y=Y, in_bs=Y, in_xs=B * Y, out_bs=X, out_ys=B * X)
+    assert torch.equal(oi, xi.permute(2, 1, 0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("r,c", [(40, 128), (33, 64), (64, 128)])
+@pytest.mark.parametrize("incoming", [False, True])
+def test_channel_major_functions_match_the_permutes(dev, dtype, r, c, incoming):
+    """_ToChanMajorFn / _FromChanMajorFn / _transpose_cm against the permute + copy they replace, forward and backward."""
+    from fastfold_amd.model.fastnn import ops
+    g = torch.Generator().manual_seed(r + c)
+    lr = torch.randn(1, r, r, 2 * c, generator=g).to(dev, dtype).requires_grad_()
+    L, R = ops._ToChanMajorFn.apply(lr, incoming)
+    perm = (2, 1, 0) if incoming else (2, 0, 1)
+    left, right = lr.chunk(2, dim=-1)
+    Lw, Rw = ops._chan_major(left, perm), ops._chan_major(right, perm)
+    assert torch.equal(L, Lw) and torch.equal(R, Rw)
+    assert L.untyped_storage().data_ptr() != R.untyped_storage().data_ptr()
+    cl, cr = torch.randn(L.shape, generator=g).to(dev, dtype), torch.randn(R.shape, generator=g).to(dev, dtype)
+    (gl,) = torch.autograd.grad([L, R], [lr], [cl, cr])
+    (gw,) = torch.autograd.grad([Lw, Rw], [lr], [cl, cr])
+    assert torch.equal(gl, gw)
+    assert torch.equal(ops._transpose_cm(L.detach(), r)[..., :r], L.detach()[..., :r].transpose(1, 2))
+    p = L.detach().clone().requires_grad_()
+    z = ops._FromChanMajorFn.apply(p, r)
+    zw = ops.permute_final_dims(p[None, :, :, :r], (1, 2, 0))
+    assert z.is_contiguous() and torch.equal(z, zw)
+    cz = torch.randn(z.shape, generator=g).to(dev, dtype)
+    (gp,) = torch.autograd.grad(z, p, cz)
+    (gpw,) = torch.autograd.grad(zw, p, cz)
+    assert torch.equal(gp, gpw)
