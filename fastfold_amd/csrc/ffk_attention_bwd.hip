@@ -75,6 +75,14 @@ __device__ __forceinline__ typename Mma<T>::Frag identity_frag(int i, int l32, i
     return f;
 }
 
+// Workgroup -> logical block.  The hardware hands consecutive workgroup ids to the eight XCDs in turn, each with its own
+// L2; the launches round their grids up to a multiple of eight and every XCD takes a contiguous eighth of the logical
+// order, so that the waves that walk the same k / v (or q / do) tiles run behind one L2.
+__device__ __forceinline__ long bwd_logical_block() {
+    const unsigned per_xcd = gridDim.x >> 3;
+    return (long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+}
+
 // ------------------------------------------------------------------------------ dq ----
 template <typename T, int DP, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
@@ -88,7 +96,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
-    const long item = (long)blockIdx.x * 4 + wave;
+    const long item = bwd_logical_block() * 4 + wave;
     if (item >= (long)B2 * H * QT) return;
     const int qt = (int)(item % QT);
     const long bh = item / QT;
@@ -219,7 +227,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
-    const long item = (long)blockIdx.x * 4 + wave;
+    const long item = bwd_logical_block() * 4 + wave;
     if (item >= (long)B2 * H * KT) return;
     const int kt = (int)(item % KT);
     const long bh = item / KT;
@@ -324,7 +332,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dbias_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int QT = (Nq + 31) >> 5, KT = (Nk + 31) >> 5;
-    const long item = (long)blockIdx.x * 4 + wave;             // key tile fastest: a block's waves share q and do
+    const long item = bwd_logical_block() * 4 + wave;          // key tile fastest: a block's waves share q and do
     if (item >= (long)NS * H * QT * KT) return;
     const int kt = (int)(item % KT);
     const int qt = (int)((item / KT) % QT);
@@ -393,7 +401,7 @@ int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* ds
                long Nk, float dq_scale, float dk_scale, hipStream_t st) {
     const long QT = (Nq + 31) / 32, KT = (Nk + 31) / 32;
     const long part_q = B2 * H * QT * 1024, part_k = B2 * H * KT * 1024;
-    const long g1 = (B2 * H * QT + 3) / 4, g2 = (B2 * H * KT + 3) / 4;
+    const long g1 = 8 * ((B2 * H * QT + 31) / 32), g2 = 8 * ((B2 * H * KT + 31) / 32);      // blocks of four waves, a multiple of 8
     FFK_REQUIRE(g1 < (1L << 31) && g2 < (1L << 31), FFK_ERR_SHAPE, "ffk_attention_bwd: too many tiles for one launch");
     if (bias_t) {
         attention_bwd_dq_kernel<T, DP, true><<<(unsigned)g1, 256, 0, st>>>((T*)dq, lse, dsum, (const T*)q_qk, (const T*)k_qk,
@@ -419,7 +427,7 @@ int launch_bwd(void* dq, void* dk, void* dv, float* dbias, float* lse, float* ds
     long ns = (8L * 1024 + tiles - 1) / tiles;
     if (ns > (B2 + 7) / 8) ns = (B2 + 7) / 8;
     if (ns < 1) ns = 1;
-    const long g3 = (ns * tiles + 3) / 4;
+    const long g3 = 8 * ((ns * tiles + 31) / 32);
     FFK_REQUIRE(g3 < (1L << 31), FFK_ERR_SHAPE, "ffk_attention_bwd: too many tiles for one launch");
     attention_bwd_dbias_kernel<T, DP><<<(unsigned)g3, 256, 0, st>>>(dbias, (const T*)q_qk, (const T*)k_qk, (const T*)v_qk,
                                                                   (const T*)bias_t, keybias, (const T*)do_qk, lse, dsum,
