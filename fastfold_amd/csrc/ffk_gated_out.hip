@@ -8,7 +8,8 @@
 // A workgroup (4 wavefronts) owns 128 logical rows, a wavefront 32 of them from start to end.  Set-up: the rows of x
 // are fetched once (row m at (m / inner) * s_o + (m % inner) * s_i: the transposed traversals of the column-wise
 // attentions are strides), normalised in registers and passed through LDS into the MFMA fragments of their wave.  The
-// gate channels are walked in chunks; per chunk and wave
+// gate channels are walked in chunks of 32 (the rings then take 32 KB at C = 128, the kernel 162 registers: three
+// workgroups share a CU and cover each other's set-up and epilogue, which are half of a workgroup's life); per chunk and wave
 //   first GEMM   G^T[gate channel, rows] = Wg[chunk] . x^T + bg, sigmoid, times o: lane = row, registers = gate
 //                channels, so the sixteen values of o a lane needs per 32-channel tile are two 16-byte pieces of its row;
 //   second GEMM  out^T[c, rows] += Wo[c, chunk] . (G * o)^T: the rounded products are the N operand as they stand
@@ -24,7 +25,7 @@ constexpr int GO_BM = 128;                     // rows per workgroup
 constexpr int GO_NS = 2;                       // slots of the weight rings
 template <int C> struct GoGeo {
     static constexpr int H = C;                     // gate channels (heads x 32)
-    static constexpr int HC = C == 128 ? 64 : 32;   // gate channels per chunk
+    static constexpr int HC = 32;                   // gate channels per chunk
     static constexpr int NCHUNK = H / HC;
     static constexpr int W1SLOT = HC * C * 2;       // HC rows of 2 C bytes (16 KB)
     static constexpr int W2SLOT = C * HC * 2;       // C rows of 2 HC bytes (16 KB)
@@ -35,6 +36,8 @@ template <int C> struct GoGeo {
     static constexpr int KS1 = C / 16, KS2 = HC / 16, HT = HC / 32, CT = C / 32;
     static constexpr size_t SMEM_RINGS = GO_NS * (size_t)W1SLOT + GO_NS * W2SLOT + H * sizeof(float);
     static constexpr size_t SMEM_ROWS = (size_t)GO_BM * XP;
+    static constexpr int NLD = W1SLOT / 16 / GO_THREADS;   // 16-byte requests per thread and ring slot
+    static_assert(W1SLOT == W2SLOT, "ring slots of one size");
     static constexpr size_t SMEM = SMEM_RINGS > SMEM_ROWS ? SMEM_RINGS : SMEM_ROWS;
 };
 
@@ -48,7 +51,7 @@ __device__ __forceinline__ void go_load_lds(const T* src, unsigned char* dst_wav
 }
 
 template <int GO_C>
-__global__ __launch_bounds__(GO_THREADS, 2) void gated_out_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
+__global__ __launch_bounds__(GO_THREADS, GO_C == 128 ? 3 : 2) void gated_out_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
                                                                  const T* __restrict__ gamma, const T* __restrict__ beta,
                                                                  const T* __restrict__ w1, const T* __restrict__ b1,
                                                                  const T* __restrict__ o, const T* __restrict__ w2,
@@ -57,6 +60,7 @@ __global__ __launch_bounds__(GO_THREADS, 2) void gated_out_kernel(T* __restrict_
     typedef Mma<T> MM;
     typedef GoGeo<GO_C> G;
     constexpr int NS = GO_NS;
+    constexpr int NLD = G::NLD;
     constexpr int GO_H = G::H, GO_HC = G::HC, GO_NCHUNK = G::NCHUNK, GO_W1SLOT = G::W1SLOT, GO_W2SLOT = G::W2SLOT, GO_XP = G::XP;
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* s_w1 = smem;                           // [NS][HC][2 C bytes]
@@ -129,16 +133,16 @@ __global__ __launch_bounds__(GO_THREADS, 2) void gated_out_kernel(T* __restrict_
 
     // ---- chunk loaders (direct to LDS; lane L of a wave lands at dst + 16 L) ----
     // W1 chunk: LDS row rho (0..HC-1) holds weight row 32 * (rho / 32) + sigma(rho % 32) of the chunk
-    const T* w1src[4];
+    const T* w1src[NLD];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NLD; ++i) {
         const int v = i * GO_THREADS + tid, rho = v / G::NC1, c = v % G::NC1;
         w1src[i] = w1 + (long)((rho & ~31) + go_sigma(rho & 31)) * GO_C + ((c ^ (rho & 15)) * 8);
     }
     // W2 chunk: LDS row rho (0..C-1) holds weight row 32 * (rho / 32) + tau(rho % 32)
-    const T* w2src[4];
+    const T* w2src[NLD];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NLD; ++i) {
         const int v = i * GO_THREADS + tid, rho = v / G::NC2, c = v % G::NC2;
         w2src[i] = w2 + (long)((rho & ~31) + go_tau(rho & 31)) * GO_H + ((c ^ ((rho / G::RP2) & (G::NC2 - 1))) * 8);
     }
@@ -146,10 +150,10 @@ __global__ __launch_bounds__(GO_THREADS, 2) void gated_out_kernel(T* __restrict_
         const int qc = q < GO_NCHUNK ? q : GO_NCHUNK - 1;
         unsigned char* d1 = s_w1 + (q % NS) * GO_W1SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) go_load_lds(w1src[i] + (long)qc * GO_HC * GO_C, d1 + i * (GO_THREADS * 16));
+        for (int i = 0; i < NLD; ++i) go_load_lds(w1src[i] + (long)qc * GO_HC * GO_C, d1 + i * (GO_THREADS * 16));
         unsigned char* d2 = s_w2 + (q % NS) * GO_W2SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) go_load_lds(w2src[i] + qc * GO_HC, d2 + i * (GO_THREADS * 16));
+        for (int i = 0; i < NLD; ++i) go_load_lds(w2src[i] + qc * GO_HC, d2 + i * (GO_THREADS * 16));
     };
 
     f32x16 acc2[G::CT];                                    // out^T tiles: channels 32 ct + 16 half + v, row l32

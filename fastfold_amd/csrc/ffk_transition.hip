@@ -1,14 +1,12 @@
 // Fused transition (see ffk_transition_fused in include/ffk.h):
 //     out = x + W2 . relu( W1 . LayerNorm(x) + b1 ) + b2        (C -> 4C -> C channels, C = 128 or 256, bf16)
-// with the hidden activation never leaving the registers.  The description below is for C = 128 (pair
-// transition); the MSA transition (C = 256) walks the hidden layer in 32 chunks of 32 channels, so that its
-// weight rings take the same 64 KB and two workgroups still fit a CU.
+// with the hidden activation never leaving the registers.
 //
 // A workgroup (4 wavefronts) owns 128 rows, a wavefront 32 of them from start to end.  Set-up: the rows
 // are fetched once, normalised in registers (16 lanes per row) and passed through LDS into the MFMA
-// fragments of their wave, where they stay.  The hidden layer is walked in 8 chunks of 64 channels; per
-// chunk and wave
-//   first GEMM   H^T[hidden, rows] = W1[chunk] . x^T  (+ b1, relu): 2 tiles of 32 hidden channels; lane =
+// fragments of their wave, where they stay.  The hidden layer is walked in chunks of 32 channels (16 chunks
+// at C = 128, 32 at C = 256); per chunk and wave
+//   first GEMM   H^T[hidden, rows] = W1[chunk] . x^T  (+ b1, relu): one tile of 32 hidden channels; lane =
 //                row, registers = hidden channels;
 //   second GEMM  out^T[c, rows] += W2[c, chunk] . H^T: the rounded accumulators of the first GEMM are the
 //                N operand as they stand.  A lane holds hidden channels 8a + 4h + b of a tile (h = its
@@ -16,8 +14,11 @@
 //                so the first GEMM's M-operand row i is loaded from weight row sigma(i) such that
 //                registers 8j .. 8j + 7 of half-wave h are hidden channels 16j + 8h .. 16j + 8h + 7.
 // Only the weights go through LDS: W1 / W2 chunks arrive by direct global -> LDS loads (XOR-swizzled
-// unpadded rows) one chunk ahead, shared by the four waves; one barrier per chunk.  Two workgroups fit
-// a CU, so one computes while the other waits for its rows or its barrier.
+// unpadded rows) one chunk ahead, shared by the four waves; one barrier per chunk.  A workgroup spends about
+// a third of its life fetching its rows and storing its results (measured with wall-clock stamps: 3.5 us set-up,
+// 14 us in the chunk loop, 5 us in the epilogue at C = 128 with residual tails), so as many workgroups as fit share
+// a CU and cover each other's waits: with 32-channel chunks the rings take 32 KB (C = 128; the row buffer of the
+// set-up, 34 KB, is then the larger) and the kernel 149 registers: three workgroups per CU (two at C = 256).
 #include "ffk_common.h"
 
 namespace {
@@ -27,7 +28,7 @@ constexpr int TR_THREADS = 256;
 constexpr int TR_BM = 128;                     // rows per workgroup
 template <int C, int NS> struct TrGeo {
     static constexpr int H = 4 * C;
-    static constexpr int HC = C == 128 ? 64 : 32;   // hidden channels per chunk
+    static constexpr int HC = 32;                   // hidden channels per chunk
     static constexpr int NCHUNK = H / HC;
     static constexpr int W1SLOT = HC * C * 2;       // HC rows of 2 C bytes (16 KB)
     static constexpr int W2SLOT = C * HC * 2;       // C rows of 2 HC bytes (16 KB)
@@ -38,6 +39,8 @@ template <int C, int NS> struct TrGeo {
     static constexpr int KS1 = C / 16, KS2 = HC / 16, HT = HC / 32, CT = C / 32;
     static constexpr size_t SMEM_RINGS = NS * (size_t)W1SLOT + NS * W2SLOT + H * sizeof(float);
     static constexpr size_t SMEM_ROWS = (size_t)TR_BM * XP;
+    static constexpr int NLD = W1SLOT / 16 / TR_THREADS;   // 16-byte requests per thread and ring slot
+    static_assert(W1SLOT == W2SLOT, "ring slots of one size");
     static constexpr size_t SMEM = SMEM_RINGS > SMEM_ROWS ? SMEM_RINGS : SMEM_ROWS;
 };
 
@@ -54,13 +57,14 @@ __device__ __forceinline__ void tr_load_lds(const T* src, unsigned char* dst_wav
 // other's waits; four when the launch has at most one workgroup per CU and the chunk stream has to hide the whole
 // memory latency by itself (a chunk is multiplied in less than half a microsecond).
 template <int TR_C, int NS>
-__global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
+__global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : (TR_C == 128 ? 3 : 2)) void transition_fused_kernel(T* __restrict__ out, const T* __restrict__ x, int8_t* __restrict__ xtail,
                                                                         const T* __restrict__ gamma, const T* __restrict__ beta,
                                                                         const T* __restrict__ w1, const T* __restrict__ b1,
                                                                         const T* __restrict__ w2, const T* __restrict__ b2,
                                                                         long M, float eps) {
     typedef Mma<T> MM;
     typedef TrGeo<TR_C, NS> G;
+    constexpr int NLD = G::NLD;
     constexpr int TR_H = G::H, TR_HC = G::HC, TR_NCHUNK = G::NCHUNK, TR_W1SLOT = G::W1SLOT, TR_W2SLOT = G::W2SLOT, TR_XP = G::XP;
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* s_w1 = smem;                           // [NS][HC][2 C bytes]
@@ -120,16 +124,16 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
 
     // ---- chunk loaders (direct to LDS; lane L of a wave lands at dst + 16 L) ----
     // W1 chunk: LDS row rho (0..63) holds weight row 32 * (rho / 32) + sigma(rho % 32) of the chunk; 16 columns
-    const T* w1src[4];
+    const T* w1src[NLD];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NLD; ++i) {
         const int v = i * TR_THREADS + tid, rho = v / G::NC1, c = v % G::NC1;
         w1src[i] = w1 + (long)((rho & ~31) + tr_sigma(rho & 31)) * TR_C + ((c ^ (rho & 15)) * 8);
     }
     // W2 chunk: LDS row rho (0..127) holds weight row 32 * (rho / 32) + tau(rho % 32); 8 columns
-    const T* w2src[4];
+    const T* w2src[NLD];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NLD; ++i) {
         const int v = i * TR_THREADS + tid, rho = v / G::NC2, c = v % G::NC2;
         w2src[i] = w2 + (long)((rho & ~31) + tr_tau(rho & 31)) * TR_H + ((c ^ ((rho / G::RP2) & (G::NC2 - 1))) * 8);
     }
@@ -137,10 +141,10 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
         const int qc = q < TR_NCHUNK ? q : TR_NCHUNK - 1;
         unsigned char* d1 = s_w1 + (q % NS) * TR_W1SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) tr_load_lds(w1src[i] + (long)qc * TR_HC * TR_C, d1 + i * (TR_THREADS * 16));
+        for (int i = 0; i < NLD; ++i) tr_load_lds(w1src[i] + (long)qc * TR_HC * TR_C, d1 + i * (TR_THREADS * 16));
         unsigned char* d2 = s_w2 + (q % NS) * TR_W2SLOT + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) tr_load_lds(w2src[i] + qc * TR_HC, d2 + i * (TR_THREADS * 16));
+        for (int i = 0; i < NLD; ++i) tr_load_lds(w2src[i] + qc * TR_HC, d2 + i * (TR_THREADS * 16));
     };
 
     f32x16 acc2[G::CT];                                    // out^T tiles: channels 32 ct + 16 half + v, row l32
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(TR_THREADS, NS == 4 ? 1 : 2) void transition_fused_
     for (int q = 0; q < NS - 1; ++q) fetch(q);
     for (int q = 0; q < TR_NCHUNK; ++q) {
         // chunk q has landed (this wave's part) once only the NS - 2 younger chunks (8 loads each) are outstanding
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * (NS - 2)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD * (NS - 2)) : "memory");
         __builtin_amdgcn_s_barrier();                        // ... everyone's; nobody still reads the slot of chunk q - 1
         fetch(q + NS - 1);
         const unsigned char* wa = s_w1 + (q % NS) * TR_W1SLOT;
