@@ -116,11 +116,31 @@ __global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict_
     // A2 fragment of phase B: pair row mt * 32 + l32, k2 = 16 ks + 8 half
     const int a2r = l32 * OP_PA + half * 16;
 
+    // The epilogue's operands (residual, its tail, the normaliser) are requested during the third chunk, not in the
+    // epilogue: with one workgroup per CU (154 KB of LDS) nothing else would cover their latency - four dependent round
+    // trips took 8 of a workgroup's 42 microseconds.  The wait at the top of the next chunk covers them.
+    u32x4 e_rv[2][2][2], e_tv[2][2];
+    float e_norm[2];
+    const int pf_q = 2 + (int)((blockIdx.x >> 3) % 12u);   // spread over the chunks: the workgroups of a launch run in step
     fetch(0);
     for (int q = 0; q <= OP_NCHUNK; ++q) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // chunk q has landed (this wave's part)
         __builtin_amdgcn_s_barrier();                        // ... everyone's; A2 of chunk q - 1 is complete
         if (q + 1 < OP_NCHUNK) fetch(q + 1);
+        if (q == pf_q) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                const long pr = (long)(i0 + mt0 + m) * r + j0 + l32;
+                e_norm[m] = norm[pr];
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const long o = pr * 128 + (ct0 + c) * 32 + 16 * half;
+                    e_rv[m][c][0] = *reinterpret_cast<const u32x4*>(resid + o);
+                    e_rv[m][c][1] = *reinterpret_cast<const u32x4*>(resid + o + 8);
+                    if (xtail) e_tv[m][c] = *reinterpret_cast<const u32x4*>(xtail + o);
+                }
+            }
+        }
         if (q > 0) {
             // ---- phase B of chunk q - 1 ----
             const unsigned char* a2 = s_a2 + ((q - 1) & 1) * OP_A2;
@@ -164,7 +184,7 @@ __global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict_
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
         const long pr = (long)(i0 + mt0 + m) * r + j0 + l32;
-        const float inv = 1.0f / (norm[pr] + eps);
+        const float inv = 1.0f / (e_norm[m] + eps);
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
             const int ch = (ct0 + c) * 32 + 16 * half;
@@ -172,10 +192,10 @@ __global__ __launch_bounds__(OP_THREADS, 2) void opm_fused_kernel(T* __restrict_
             u32x4 bv[2], rv[2];
             bv[0] = *reinterpret_cast<const u32x4*>(bias + ch);
             bv[1] = *reinterpret_cast<const u32x4*>(bias + ch + 8);
-            rv[0] = *reinterpret_cast<const u32x4*>(resid + o);
-            rv[1] = *reinterpret_cast<const u32x4*>(resid + o + 8);
+            rv[0] = e_rv[m][c][0];
+            rv[1] = e_rv[m][c][1];
             if (xtail) {       // extended residual stream: the update is added at 24 bits
-                const u32x4 tv = *reinterpret_cast<const u32x4*>(xtail + o);
+                const u32x4 tv = e_tv[m][c];
                 float upd[16];
 #pragma unroll
                 for (int v = 0; v < 16; ++v) upd[v] = (float)(T)((acc2[m][c][v] + (float)reinterpret_cast<const T*>(&bv[v >> 3])[v & 7]) * inv);
