@@ -257,13 +257,15 @@ def bgemm_nt(a, b, out, *, M, N, K, lda, ldb, batch=1, a_bs=0, b_bs=0, o_bs=0, i
 
 FFK_ATT_GATE_TILED = 1
 FFK_ATT_BIAS_PADDED = 2
+FFK_ATT_HALF_K = 4
 
 
 def attention_fwd(out, q_t, k_t, v_t, bias_t, keybias, tileflags, gate, *, B2, H, Nq, Nk, D=32, gate_tiled=False,
-                  bias_padded=False):
+                  bias_padded=False, half_k=False):
     call("ffk_attention_fwd", ptr(out), ptr(q_t), ptr(k_t), ptr(v_t), ptr(bias_t), ptr(keybias), ptr(tileflags),
          ptr(gate),
-         B2, H, Nq, Nk, D, (FFK_ATT_GATE_TILED if gate_tiled else 0) | (FFK_ATT_BIAS_PADDED if bias_padded else 0),
+         B2, H, Nq, Nk, D, (FFK_ATT_GATE_TILED if gate_tiled else 0) | (FFK_ATT_BIAS_PADDED if bias_padded else 0)
+         | (FFK_ATT_HALF_K if half_k else 0),
          dtype_tag(q_t.dtype), stream_ptr())
 
 

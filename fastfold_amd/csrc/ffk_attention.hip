@@ -282,8 +282,14 @@ __global__ __launch_bounds__(ATT_THREADS, sizeof(T) == 2 ? 4 : 2) void attention
             kc.load_lds(buf + bsel * 1024, lane);
             if (HAS_BIAS) bc.load_lds(buf + (4 + qsel) * 1024, lane);
             s = negm;
+            // FFK_ATT_HALF_K: elements 8 .. 15 of every lane's sixteen are zero padding in q and k (narrow heads): the
+            // second half of the score product adds nothing and is skipped
 #pragma unroll
-            for (int i = 0; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
+            for (int i = 0; i < NF / 2; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
+            if (!(flags & FFK_ATT_HALF_K)) {
+#pragma unroll
+                for (int i = NF / 2; i < NF; ++i) MM::mma(s, kc.frag(i), qf.frag(i));
+            }
             if (HAS_BIAS) {
 #pragma unroll
                 for (int i = 0; i < NF; ++i) MM::mma(s, bc.frag(i), ident[i]);
@@ -588,8 +594,8 @@ extern "C" int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, co
                 "ffk_attention_fwd: head dimension %ld (32, 64 or 128; narrower heads arrive zero-padded to 32)", (long)D);
     hipStream_t st = (hipStream_t)stream;
     if (D != 32) {
-        FFK_REQUIRE(!gate && !(flags & FFK_ATT_BIAS_PADDED), FFK_ERR_UNSUPPORTED,
-                    "ffk_attention_fwd: the gate and padded bias rows are built for head dimension 32 only");
+        FFK_REQUIRE(!gate && !(flags & (FFK_ATT_BIAS_PADDED | FFK_ATT_HALF_K)), FFK_ERR_UNSUPPORTED,
+                    "ffk_attention_fwd: the gate, padded bias rows and the narrow-head flag are built for head dimension 32 only");
         if (dtype == FFK_BF16)
             return D == 64 ? launch_attention_wide<bf16_t, 2>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st)
                            : launch_attention_wide<bf16_t, 4>(out, q_t, k_t, v_t, bias_t, keybias, tileflags, B2, H, Nq, Nk, st);

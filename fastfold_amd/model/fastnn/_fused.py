@@ -310,7 +310,8 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
             _lib.fused_linear(x, wp, tiles[t0:t0 + per], M=Ms, K=C, a_inner=inner, a_so=a_so, a_si=a_si, ln=ln,
                               w_row_off=t0 * 128, a_off=off)
         _lib.attention_fwd(o, q_t, k_t, v_t, bias_t, kb[b0:b0 + nb], flags[b0:b0 + nb], gate, B2=nb, H=H, Nq=N, Nk=N,
-                           gate_tiled=acc_order, bias_padded=bias_padded)
+                           gate_tiled=acc_order, bias_padded=bias_padded,
+                           half_k=head_dim <= (16 if acc_order else 8))
         if gate_in_out:
             # packed rows of w_pk: q, k, v, gate blocks of HC rows each; o holds the slab's rows in logical order
             _lib.gated_out_fused(out.data_ptr() + o_off * es, x.data_ptr() + off * es, ln[0], ln[1],

@@ -273,6 +273,10 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  *              FFK_ATT_BIAS_PADDED in flags [H][ceil(Nq/32)][ceil(Nk/32) + 1][1024]: one unused tile ends every
  *              query-tile row, so that rows of 2^n key tiles do not start in the same memory channel (D = 32 only)
  *   keybias  : [B2][ceil(Nk/32)*32] fp32
+ *   FFK_ATT_HALF_K in flags (D = 32 only): the caller guarantees that elements 8 .. 15 of every lane's sixteen (elements
+ *              16 l + 8 .. 16 l + 15 of each 1024-element q and k tile) are zero - zero-padded heads of at most 16 channels
+ *              in FFK_TILE_ACC order (channels 16 .. 31), of at most 8 channels in FFK_TILE_QK order (channels 8 .. 15 and
+ *              24 .. 31) -; the kernel skips that half of the score product
  *   tileflags: [B2][ceil(Nk/32)] int32 per 32-key tile: 0 all keys valid, 1 mixed, 2 all masked
  *   gate     : multiplicative gate (already sigmoid-ed) or NULL: [B2*Nq, H*32] row-major, or with
  *              FFK_ATT_GATE_TILED in flags [B2][H][ceil(Nq/32)][1024] in FFK_TILE_ACC order
@@ -284,7 +288,7 @@ int ffk_bgemm_nt(const ffk_bgemm_desc* desc, void* stream);
  * SelfAttention.forward (fastfold/model/fastnn/ops.py:310-322) and
  * fused_attention_core (kernel/attention_core.py:17-52, kernel/triton/attention_core.py:12-190).
  */
-enum { FFK_ATT_GATE_TILED = 1, FFK_ATT_BIAS_PADDED = 2 };
+enum { FFK_ATT_GATE_TILED = 1, FFK_ATT_BIAS_PADDED = 2, FFK_ATT_HALF_K = 4 };
 int ffk_attention_fwd(void* out, const void* q_t, const void* k_t, const void* v_t,
                       const void* bias_t, const float* keybias, const int32_t* tileflags, const void* gate,
                       int64_t B2, int64_t H, int64_t Nq, int64_t Nk, int64_t D, int flags, int dtype, void* stream);

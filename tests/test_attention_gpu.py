@@ -68,6 +68,31 @@ def test_attention_core(dev, dtype, tol, B2, H, N, use_bias, use_gate):
         assert torch.equal(out, out3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_attention_half_k_flag(dev, dtype, use_bias):
+    """Heads of 8 channels zero-padded to 32 (FFK_TILE_QK order: channels 8 .. 15 and 24 .. 31 are elements 8 .. 15 of a
+    lane's sixteen): with FFK_ATT_HALF_K the kernel skips the second half of the score product and gives the same bits."""
+    from fastfold_amd import _lib
+    from fastfold_amd.model.fastnn.kernel import layouts
+    B2, H, N = 3, 4, 100
+    g = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(B2, H, N, 32, generator=g).to(dev, dtype) for _ in range(3))
+    q[..., 8:] = 0
+    k[..., 8:] = 0
+    bt = layouts.tile_bias(torch.randn(H, N, N, generator=g).to(dev, dtype)) if use_bias else None
+    kb = torch.empty(B2, 128, dtype=torch.float32, device=dev)
+    fl = torch.empty(B2, 4, dtype=torch.int32, device=dev)
+    _lib.key_bias(kb, fl, None, B=B2, N=N)
+    outs = []
+    for half_k in (False, True):
+        out = torch.empty(B2 * N, H * 32, dtype=dtype, device=dev)
+        _lib.attention_fwd(out, layouts.tile_qk(q), layouts.tile_qk(k), layouts.tile_v(v), bt, kb, fl, None,
+                           B2=B2, H=H, Nq=N, Nk=N, half_k=half_k)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
 def test_attention_tiling_invariance_and_masked_keys(dev, dtype, tol):
     """Changing K/V at masked keys must not change the output; all-valid mask == no mask."""
