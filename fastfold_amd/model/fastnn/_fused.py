@@ -233,8 +233,9 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
     # (ffk_gated_out_fused).  The projection launch then writes q, k, v only and the core reads no gate.
     # Measured at N_seq = 128, same box: on the triangle attentions at N_res = 1024 the projection and the core each get
     # ~ 3 % faster and the output stage as much slower - 1.1 GB less memory traffic per block at the same block time; at
-    # N_res = 256 the non-persistent output stage loses 1.3 % of a block, and on the MSA attentions (256 channels) it
-    # loses slightly at both sizes.  The choice depends on the row length and the width only, never on the number of
+    # N_res = 256 a block gains 1.4 % (0.631 vs 0.640 ms) since the output stage runs three workgroups per CU (with two
+    # it lost 1.3 %); on the MSA attentions (256 channels, two workgroups per CU) it loses slightly at both sizes.
+    # Shorter rows were not measured and keep the gate tensor.  The choice depends on the row length and the width only, never on the number of
     # batch rows: a subset of the batch rows must give the bits of the full call.
     gate_in_out = (_GATE_IN_OUT_STAGE and drop is None and N >= _GATE_IN_OUT_MIN_N and C in _GATE_IN_OUT_WIDTHS and acc_order
                    and ln is not None and HC == C and c_out == C and resid is not None and o_map is None
@@ -402,7 +403,7 @@ _TRIMUL_CHAN_PAD = 64
 _PAIR_BIAS_RIDES = True      # see attention(): switch for same-box comparisons
 _BIAS_ROW_PAD = True         # see attention(): switch for same-box comparisons
 _GATE_IN_OUT_STAGE = True    # see attention(): False keeps the gate a tensor (written by the projection, read by the core)
-_GATE_IN_OUT_MIN_N = 512         # shortest attended axis for which the gate moves into the output stage
+_GATE_IN_OUT_MIN_N = 256         # shortest attended axis for which the gate moves into the output stage
 _GATE_IN_OUT_WIDTHS = (128,)     # ... and the channel widths (the kernel is built for 128 and 256)
 
 
