@@ -99,10 +99,11 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             }
         }
     };
-    auto fetch_next = [&]() {
-        unsigned char* slot = smem + (g_fetch & (BG_SLOTS - 1)) * SLOT + wave * 1024;
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) bg_load_lds(src[i] + f_kc * BG_BK, slot + i * 8192);
+    // A chunk's loads can be issued one by one (fetch_one), spread between the MFMAs of a step; fetch_advance moves on.
+    auto fetch_one = [&](int i) {
+        bg_load_lds(src[i] + f_kc * BG_BK, smem + (g_fetch & (BG_SLOTS - 1)) * SLOT + wave * 1024 + i * 8192);
+    };
+    auto fetch_advance = [&]() {
         ++g_fetch;
         if (++f_kc == kchunks) {                             // on to the next tile; past the last one the
             unsigned item;                                   // same chunks are re-read into free slots (harmless)
@@ -112,6 +113,11 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
                 fetch_setup(item);
             }
         }
+    };
+    auto fetch_next = [&]() {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) fetch_one(i);
+        fetch_advance();
     };
 
     // fragment addresses: A rows in natural order, B rows through tau; column (2 ks + half) un-swizzled
@@ -130,48 +136,31 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
     fetch_next();
     fetch_next();
     unsigned g_use = 0;
-    bool relaxed = false;      // previous tile was full: its stores are counted exactly
-    for (unsigned t = 0; tile_at(t, item); ++t) {
-        const long m0 = (long)(item % tiles_m) * BM, n0 = (long)((item / tiles_m) % tiles_n) * BN;
-        const int bz = (item / tiles_m) / tiles_n;
-        f32x16 acc[NI][2];   // [ni][mi]
+    f32x16 acc[NI][2];   // [ni][mi]
+    bf16x8 fa0[2], fb0[NI], fa1[2], fb1[NI];                 // fragments of K step 0 and of K step 1 of a chunk
+    auto zero_acc = [&]() {
 #pragma unroll
         for (int a = 0; a < NI; ++a)
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
-
-        for (int kc = 0; kc < kchunks; ++kc, ++g_use) {
-            // the chunk in use has landed once at most the loads of the two younger chunks are outstanding
-            // (stores of the previous tile's results are younger still)
-            // Right after a tile whose every store was issued (a full tile: no lane predicate can have
-            // skipped one), those 4 * NI stores are known to be younger than the chunks still awaited
-            // and need not be waited for.
-            if (relaxed && kc < 3) {
-                if (NLD == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
-            } else {
-                if (NLD == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-            }
-            __builtin_amdgcn_s_barrier();                    // ... for every wave; the slot used last step is free again
-            fetch_next();
-            const unsigned char* s = smem + (g_use & (BG_SLOTS - 1)) * SLOT;
+    };
+    auto read_frag = [&](const unsigned char* s, int ks, bf16x8 (&fa)[2], bf16x8 (&fb)[NI]) {
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                bf16x8 fa[2], fb[NI];
+        for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(s + fa_off[ks] + i * 32 * 64);
 #pragma unroll
-                for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(s + fa_off[ks] + i * 32 * 64);
+        for (int i = 0; i < NI; ++i) fb[i] = *reinterpret_cast<const bf16x8*>(s + fb_off[ks] + i * 32 * 64);
+    };
+    auto mma_pair = [&](const bf16x8 (&fa)[2], const bf16x8 (&fb)[NI], int ni) {
 #pragma unroll
-                for (int i = 0; i < NI; ++i) fb[i] = *reinterpret_cast<const bf16x8*>(s + fb_off[ks] + i * 32 * 64);
+        for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
+    };
+    auto mma_half = [&](const bf16x8 (&fa)[2], const bf16x8 (&fb)[NI], int h) {
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-                    for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
-            }
-        }
-
+        for (int ni = h * (NI / 2); ni < (h + 1) * (NI / 2); ++ni) mma_pair(fa, fb, ni);
+    };
+    auto epilogue = [&](long m0, long n0, int bz) {
     // ---- epilogue from registers: lane = row, registers = 16 consecutive columns ----
     T* out = (T*)d.out + (long)bz * d.o_bs;
     const T* resid = d.resid ? (const T*)d.resid + (long)bz * d.o_bs : nullptr;
@@ -254,6 +243,57 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             if (ok1) *reinterpret_cast<u32x4*>(out + o + 8) = *reinterpret_cast<const u32x4*>(&y[8]);
         }
     }
+    };
+    bool relaxed = false;      // previous tile was full: its stores are counted exactly
+    for (unsigned t = 0; tile_at(t, item); ++t) {
+        const long m0 = (long)(item % tiles_m) * BM, n0 = (long)((item / tiles_m) % tiles_n) * BN;
+        const int bz = (item / tiles_m) / tiles_n;
+        zero_acc();
+        for (int kc = 0; kc < kchunks; ++kc, ++g_use) {
+            // The chunk has landed once at most the loads of the two younger chunks are outstanding (stores of
+            // the previous tile's results are younger still).  Right after a tile whose every store was issued
+            // (a full tile: no lane predicate can have skipped one), those 4 * NI stores are known to be younger
+            // than the chunks still awaited and need not be waited for.  The fragment reads of the chunk before
+            // have returned (lgkmcnt), so behind the barrier its slot is free for every wave's next request.
+            if (relaxed && kc < 3) {
+                if (NLD == 4) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(14) lgkmcnt(0)" ::: "memory");
+            } else {
+                if (NLD == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();
+            const unsigned char* s = smem + (g_use & (BG_SLOTS - 1)) * SLOT;
+            if (kc != 0) {
+                // second K step of the chunk before; the requests for the chunk three ahead go out one by one
+                // between its MFMAs (issued in a burst they hold every wave of the CU at the same time)
+                mma_pair(fa1, fb1, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(s, 0, fa0, fb0);
+#pragma unroll
+                for (int ni = 1; ni < NI; ++ni) {
+                    fetch_one(ni - 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mma_pair(fa1, fb1, ni);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = NI - 1; i < NLD; ++i) fetch_one(i);
+                fetch_advance();
+            } else {
+                read_frag(s, 0, fa0, fb0);
+                fetch_next();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mma_half(fa0, fb0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frag(s, 1, fa1, fb1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_half(fa0, fb0, 1);
+        }
+        mma_half(fa1, fb1, 0);
+        mma_half(fa1, fb1, 1);
+        epilogue(m0, n0, bz);
         relaxed = m0 + BM <= M && n0 + BN <= N;
     }   // tiles
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // the re-reads past the end
