@@ -11,6 +11,10 @@
 // multiplied, which is what covers the memory latency with a single workgroup per CU.  Rows are
 // unpadded 64-byte lines; an XOR swizzle of their four 16-byte columns keeps the fragment reads free
 // of bank conflicts.  All addresses are set up once per tile.
+// A chunk holds two K steps of 16.  The steps are software-pipelined across the chunk barrier: the
+// fragments of a chunk's second K step are read while its first K step is multiplied, and multiplied
+// behind the next barrier while the next chunk's first fragments are on their way, so neither the
+// barrier nor the LDS read latency leaves the matrix pipe without queued work.
 // The MFMA computes C^T (rows of B are the M operand) and reads the B rows of a 32-row group through
 // the permutation tau(8a + 4h + b) = 16h + 4a + b, so that a lane ends up with 16 consecutive
 // output columns of one row: the epilogue (bias / activation / scale / row divisor / residual) works
@@ -99,11 +103,10 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             }
         }
     };
-    // A chunk's loads can be issued one by one (fetch_one), spread between the MFMAs of a step; fetch_advance moves on.
-    auto fetch_one = [&](int i) {
-        bg_load_lds(src[i] + f_kc * BG_BK, smem + (g_fetch & (BG_SLOTS - 1)) * SLOT + wave * 1024 + i * 8192);
-    };
-    auto fetch_advance = [&]() {
+    auto fetch_next = [&]() {
+        unsigned char* slot = smem + (g_fetch & (BG_SLOTS - 1)) * SLOT + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) bg_load_lds(src[i] + f_kc * BG_BK, slot + i * 8192);
         ++g_fetch;
         if (++f_kc == kchunks) {                             // on to the next tile; past the last one the
             unsigned item;                                   // same chunks are re-read into free slots (harmless)
@@ -114,12 +117,6 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
             }
         }
     };
-    auto fetch_next = [&]() {
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) fetch_one(i);
-        fetch_advance();
-    };
-
     // fragment addresses: A rows in natural order, B rows through tau; column (2 ks + half) un-swizzled
     const int ra = wm * 64 + l32, rb = BM + wn * WTN + bg_tau(l32);
     int fa_off[2], fb_off[2];
@@ -152,13 +149,11 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
 #pragma unroll
         for (int i = 0; i < NI; ++i) fb[i] = *reinterpret_cast<const bf16x8*>(s + fb_off[ks] + i * 32 * 64);
     };
-    auto mma_pair = [&](const bf16x8 (&fa)[2], const bf16x8 (&fb)[NI], int ni) {
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
-    };
     auto mma_half = [&](const bf16x8 (&fa)[2], const bf16x8 (&fb)[NI], int h) {
 #pragma unroll
-        for (int ni = h * (NI / 2); ni < (h + 1) * (NI / 2); ++ni) mma_pair(fa, fb, ni);
+        for (int ni = h * (NI / 2); ni < (h + 1) * (NI / 2); ++ni)
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi) MM::mma(acc[ni][mi], fb[ni], fa[mi]);
     };
     auto epilogue = [&](long m0, long n0, int bz) {
     // ---- epilogue from registers: lane = row, registers = 16 consecutive columns ----
@@ -249,47 +244,51 @@ __global__ __launch_bounds__(BG_THREADS, 2) void bgemm_big_kernel(const ffk_bgem
         const long m0 = (long)(item % tiles_m) * BM, n0 = (long)((item / tiles_m) % tiles_n) * BN;
         const int bz = (item / tiles_m) / tiles_n;
         zero_acc();
-        for (int kc = 0; kc < kchunks; ++kc, ++g_use) {
-            // The chunk has landed once at most the loads of the two younger chunks are outstanding (stores of
-            // the previous tile's results are younger still).  Right after a tile whose every store was issued
-            // (a full tile: no lane predicate can have skipped one), those 4 * NI stores are known to be younger
-            // than the chunks still awaited and need not be waited for.  The fragment reads of the chunk before
-            // have returned (lgkmcnt), so behind the barrier its slot is free for every wave's next request.
-            if (relaxed && kc < 3) {
+        // One step = one chunk: wait, barrier, then the second K step of the chunk before (fragments fa1 / fb1), the
+        // request for the chunk three ahead, and the first K step of this chunk.
+        // Before the barrier: this wave's loads of the chunk have landed, and its fragment reads of the chunk before
+        // have returned (lgkmcnt), so behind the barrier that slot is free for every wave's next request.
+        // Loads and stores complete in the order of issue: the chunk has landed once at most the loads of the two
+        // younger chunks are outstanding.  Right after a tile whose every store was issued (a full tile: no lane
+        // predicate can have skipped one) those 4 * NI stores are known to be younger than the chunks awaited in the
+        // first three steps and need not be waited for.
+        auto wait_chunk = [&](bool after_full_tile) {
+            if (after_full_tile) {
                 if (NLD == 4) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
                 else asm volatile("s_waitcnt vmcnt(14) lgkmcnt(0)" ::: "memory");
             } else {
                 if (NLD == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
                 else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
             }
+        };
+        auto step = [&](bool first) {                        // known at every call site
             __builtin_amdgcn_s_barrier();
             const unsigned char* s = smem + (g_use & (BG_SLOTS - 1)) * SLOT;
-            if (kc != 0) {
-                // second K step of the chunk before; the requests for the chunk three ahead go out one by one
-                // between its MFMAs (issued in a burst they hold every wave of the CU at the same time)
-                mma_pair(fa1, fb1, 0);
+            ++g_use;
+            if (!first) {
+                mma_half(fa1, fb1, 0);                       // second K step of the chunk before
                 __builtin_amdgcn_sched_barrier(0);
-                read_frag(s, 0, fa0, fb0);
-#pragma unroll
-                for (int ni = 1; ni < NI; ++ni) {
-                    fetch_one(ni - 1);
-                    __builtin_amdgcn_sched_barrier(0);
-                    mma_pair(fa1, fb1, ni);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int i = NI - 1; i < NLD; ++i) fetch_one(i);
-                fetch_advance();
-            } else {
-                read_frag(s, 0, fa0, fb0);
-                fetch_next();
             }
+            read_frag(s, 0, fa0, fb0);
+            fetch_next();
             __builtin_amdgcn_sched_barrier(0);
+            if (!first) mma_half(fa1, fb1, 1);
             mma_half(fa0, fb0, 0);
             __builtin_amdgcn_sched_barrier(0);
             read_frag(s, 1, fa1, fb1);
             __builtin_amdgcn_sched_barrier(0);
             mma_half(fa0, fb0, 1);
+            __builtin_amdgcn_sched_barrier(0);               // these MFMAs cover the reads the next wait asks for
+        };
+        wait_chunk(relaxed);
+        step(true);
+        wait_chunk(relaxed);
+        step(false);
+        wait_chunk(relaxed);
+        step(false);
+        for (int kc = 3; kc < kchunks; ++kc) {
+            wait_chunk(false);
+            step(false);
         }
         mma_half(fa1, fb1, 0);
         mma_half(fa1, fb1, 1);
