@@ -180,6 +180,29 @@ def test_bgemm_trimul_contraction(dev, dtype, tol, r):
     assert _rel(_np(out)[:, :, :r].transpose(1, 2, 0), ref) < tol
 
 
+@pytest.mark.parametrize("C,M,N,K", [
+    (3, 256, 256, 96),       # exactly the three chunks the ring is primed with
+    (2, 300, 528, 160),      # ragged tiles in both directions, an odd number of chunks
+    (9, 512, 256, 128),      # XCD-contiguous tile order (batch >= 8), 256 x 128 tiles
+    (40, 768, 768, 128),     # 360 full 256 x 256 tiles on 256 workgroups: a second tile behind a full one
+    (40, 700, 656, 96),      # ... and behind ragged ones
+])
+def test_bgemm_large_tiles(dev, C, M, N, K):
+    """The persistent large-tile kernel (M >= 256, bf16): its chunk pipeline runs on across tiles, and the wait
+    counts right after a tile depend on whether that tile stored every row."""
+    from fastfold_amd import _lib
+    g = torch.Generator().manual_seed(C * M + N + K)
+    a = torch.randn(C, M, K, generator=g).to(dev, torch.bfloat16)
+    b = torch.randn(C, N, K, generator=g).to(dev, torch.bfloat16)
+    out = torch.full((C, M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    _lib.bgemm_nt(a, b, out, M=M, N=N, K=K, lda=K, ldb=K, batch=C, a_bs=M * K, b_bs=N * K, o_bs=M * N, scale=0.125)
+    ref = 0.125 * np.einsum("cmk,cnk->cmn", _np(a).astype(np.float32), _np(b).astype(np.float32))
+    got = _np(out)
+    assert np.isfinite(got).all()
+    assert _rel(got, ref) < 4e-3
+    assert np.abs(got - ref).max() < 2e-2 * np.abs(ref).max()
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("s,r", [(24, 10), (128, 9), (50, 33)])
 def test_bgemm_outer_product_and_projection(dev, dtype, tol, s, r):
