@@ -50,7 +50,7 @@ struct WsPlan {
     int max_slots;               // largest number of slots any wave holds
     int resid_a2;                // 1: every residual is the second operand itself (same rows): taken from its LDS slab
     int bias_tile;               // index of a trailing FFK_TILE_BIAS tile (<= 4 heads, K = 128), -1 = none: it takes no
-                                 // weight slot - its few dot products per row run on the vector pipe from the slab in LDS
+                                 // weight slot - its few dot products per row are 16 x 16 x 32 MFMAs on the slab in LDS
 };
 
 struct WsArgs {
@@ -863,29 +863,33 @@ __global__ __launch_bounds__(WS_THREADS, 2) void linear_ws_kernel(const WsArgs a
         if (more) fetch(slab + (int)gridDim.x, buf ^ 1);  // in flight during the products below
         const unsigned char* sa = s_a + buf * (WS_BM * WS_AP);
         if (PB && pb_tile >= 0) {
-            // pair bias of this slab: thread -> (row tid / 4, head tid % 4); the row is the operand as the products
-            // see it (normalised, rounded to bf16), so the value equals a fifth output column group of four channels
+            // pair bias of this slab on the matrix pipe: wave w takes the rows 16 w .. 16 w + 15 as the N operand of
+            // four 16 x 16 x 32 products against the (at most four) head weight rows, zero rows up to 16 (M operand).
+            // The rows are the operand as the other products see it (normalised, rounded to bf16), so the value
+            // equals a further output column group of four channels.  Result layout: lane = row, register v = head
+            // (4 * (lane / 16) + v: only the first sixteen lanes hold real heads).
             const ffk_tile& tb = d.tiles[pb_tile];
-            const int prow = tid >> 2, hd = tid & 3;
-            const long pm = (long)slab * WS_BM + prow;
-            if (pm < M && hd < tb.ncols) {
-                typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-                const unsigned char* xr = sa + prow * WS_AP;
-                const T* wr = s_wb + hd * WS_K;
-                float acc = 0.0f;
+            const int r16 = lane & 15, kq = lane >> 4;
+            const unsigned char* xr = sa + (wave * 16 + r16) * WS_AP + kq * 16;
+            const T* wr = s_wb + (r16 & 3) * WS_K + kq * 8;
+            f32x4 pacc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int c8 = 0; c8 < WS_K / 8; ++c8) {
-                    const bf16x8 xv = *reinterpret_cast<const bf16x8*>(xr + c8 * 16);
-                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(wr + c8 * 8);
+            for (int ks = 0; ks < WS_K / 32; ++ks) {
+                const bf16x8 xv = *reinterpret_cast<const bf16x8*>(xr + ks * 64);
+                bf16x8 wv = *reinterpret_cast<const bf16x8*>(wr + ks * 32);
+                if (r16 >= 4) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const bf16x2 xp = {xv[2 * e], xv[2 * e + 1]}, wp = {wv[2 * e], wv[2 * e + 1]};
-                        acc = __builtin_amdgcn_fdot2_f32_bf16(xp, wp, acc, false);
-                    }
+                    for (int e = 0; e < 8; ++e) wv[e] = (T)0.0f;
                 }
+                pacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, xv, pacc, 0, 0, 0);
+            }
+            const long pm = (long)slab * WS_BM + wave * 16 + r16;
+            if (kq == 0 && pm < M) {
                 const unsigned hi = (unsigned)pm / (unsigned)tb.inner, lo = (unsigned)pm - hi * (unsigned)tb.inner;
-                ((T*)tb.out)[(long)hd * tb.s_h + (long)(hi >> 5) * tb.s_o + (long)(lo >> 5) * 1024 +
-                             qk_tile_off((int)(lo & 31), (int)(hi & 31))] = (T)(acc * tb.scale);
+                T* po = (T*)tb.out + (long)(hi >> 5) * tb.s_o + (long)(lo >> 5) * 1024 + qk_tile_off((int)(lo & 31), (int)(hi & 31));
+#pragma unroll
+                for (int hd = 0; hd < 4; ++hd)
+                    if (hd < tb.ncols) po[(long)hd * tb.s_h] = (T)(pacc[hd] * tb.scale);
             }
         }
         for (int rg = rg_first; rg < WS_RG; rg += rg_step) {

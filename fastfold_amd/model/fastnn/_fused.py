@@ -261,7 +261,7 @@ def attention(x, out, resid, *, B2, N, C, H, a_map, ln, w_pk, gate_bias_pk, wo_p
         bias_tile = make_tile(bias_t, kind=FFK_TILE_BIAS, inner=N, s_o=ntp * 1024, s_h=NT * ntp * 1024, ncols=H,
                               scale=LOG2E)
     # With 128 input channels, at most four heads and all rows in one slab the bias rides on the projection launch:
-    # the weights-stationary kernel computes its four dot products per row on the vector pipe from the rows it
+    # the weights-stationary kernel computes its four dot products per row (small MFMAs) from the rows it
     # has in LDS anyway (one read of x less than a pass of its own; -0.05 ms per triangle attention at N = 1024).
     rides = will_ride
     # Otherwise the skinny bias projection has its own pass over x.  It goes first: x was written by the launch before

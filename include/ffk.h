@@ -139,8 +139,8 @@ int ffk_bias_ele_dropout_res(void* out, const void* ab, const void* bias, const 
  *   FFK_TILE_QK       q / k of attention in MFMA-operand tiles: [b2][h][n/32][d/16][n%32][d%16]
  *   FFK_TILE_V        v of attention in PV-operand tiles (see ffk_attention_fwd)
  *   FFK_TILE_BIAS     pair / triangle bias in score-accumulator tiles (see ffk_attention_fwd)
- *                     (as the LAST tile of a bf16, K = 128 launch with <= 4 channels it takes no share of the matrix
- *                     work: the weights-stationary kernel computes it on the vector pipe from the rows it holds in LDS)
+ *                     (as the LAST tile of a bf16, K = 128 launch with <= 4 channels it takes no weight slot: the
+ *                     weights-stationary kernel computes it with 16 x 16 x 32 MFMAs from the rows it holds in LDS)
  *   FFK_TILE_ACC      [b2][h][n/32] tiles in MFMA accumulator order: element (n, d) of a tile at
  *                     ((d & 7) >> 2) * 512 + (n % 32) * 16 + 4 * (d >> 3) + (d & 3), i.e. the lane that
  *                     owns row n in a 32x32 accumulator holds its 16 channels contiguously.  Valid for
